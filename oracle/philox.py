@@ -1,0 +1,100 @@
+"""Philox4x32-10 and curand_uniform restated on the CPU.  TEST INFRASTRUCTURE ONLY.
+
+The reference draws its uniforms on the device from `curandStatePhilox4_32_10_t`
+(corecuda/random.spi:9,22-32) with `curand_init(seed, subsequence, offset)` and
+`curand_uniform` (corecuda/random.spi:84); seed = 12344321 (corecuda/cupy.spi:6).  cuRAND is
+a third-party dependency that is not part of the reference tree; this file restates the
+published Philox-4x32-10 algorithm (Salmon et al., "Parallel random numbers: as easy as
+1, 2, 3", SC'11) and cuRAND's documented counter layout:
+
+    key     = (seed_lo, seed_hi)
+    counter = (n_lo, n_hi, subsequence_lo, subsequence_hi)    n = index of the 4-word group
+    curand() hands out words x, y, z, w of group n in that order, then moves to group n+1
+    curand_uniform(x) = x * 2^-32 + 2^-33   (computed in f32, result in (0, 1])
+
+Pinned by the Random123 known-answer vectors and by replaying every sampled index held in
+the reference's golden outputs (tests/test_oracle_golden.py).
+"""
+import numpy as np
+
+PHILOX_M0 = np.uint64(0xD2511F53)
+PHILOX_M1 = np.uint64(0xCD9E8D57)
+PHILOX_W0 = 0x9E3779B9
+PHILOX_W1 = 0xBB67AE85
+CONSTANT_SEED = 12344321  # corecuda/cupy.spi:6
+
+_MASK32 = np.uint64(0xFFFFFFFF)
+
+
+def philox4x32_10(ctr, key):
+    """ctr: (..., 4) uint32, key: (..., 2) uint32 -> (..., 4) uint32 after 10 rounds."""
+    ctr = np.asarray(ctr, dtype=np.uint64)
+    key = np.asarray(key, dtype=np.uint64)
+    c0, c1, c2, c3 = (ctr[..., i].copy() for i in range(4))
+    k0, k1 = key[..., 0].copy(), key[..., 1].copy()
+    for r in range(10):
+        if r:
+            k0 = (k0 + np.uint64(PHILOX_W0)) & _MASK32
+            k1 = (k1 + np.uint64(PHILOX_W1)) & _MASK32
+        p0 = PHILOX_M0 * c0
+        p1 = PHILOX_M1 * c2
+        hi0, lo0 = p0 >> np.uint64(32), p0 & _MASK32
+        hi1, lo1 = p1 >> np.uint64(32), p1 & _MASK32
+        c0, c1, c2, c3 = hi1 ^ c1 ^ k0, lo1, hi0 ^ c3 ^ k1, lo0
+    return np.stack([c0, c1, c2, c3], axis=-1).astype(np.uint32)
+
+
+def curand_words(seed, subsequence, draw_index):
+    """The `draw_index`-th (0-based) 32-bit output of curand() for a Philox state initialised
+    with curand_init(seed, subsequence, offset=0).  `subsequence` and `draw_index` broadcast."""
+    subsequence = np.asarray(subsequence, dtype=np.uint64)
+    draw_index = np.asarray(draw_index, dtype=np.uint64)
+    subsequence, draw_index = np.broadcast_arrays(subsequence, draw_index)
+    group = draw_index >> np.uint64(2)
+    ctr = np.stack([group & _MASK32, group >> np.uint64(32),
+                    subsequence & _MASK32, subsequence >> np.uint64(32)], axis=-1)
+    key = np.empty(ctr.shape[:-1] + (2,), dtype=np.uint64)
+    key[..., 0] = np.uint64(seed & 0xFFFFFFFF)
+    key[..., 1] = np.uint64((seed >> 32) & 0xFFFFFFFF)
+    out = philox4x32_10(ctr, key)
+    word = (draw_index & np.uint64(3)).astype(np.int64)
+    return np.take_along_axis(out, word[..., None], axis=-1)[..., 0]
+
+
+def curand_uniform(words):
+    """uint32 -> f32 in (0, 1], cuRAND's mapping, evaluated in f32 like the device does."""
+    w = np.asarray(words, dtype=np.uint32).astype(np.float32)  # RNE u32 -> f32, as the device cvt
+    return w * np.float32(2.3283064e-10) + np.float32(1.1641532e-10)
+
+
+def row_uniforms_block(rows, cols, seed=CONSTANT_SEED, threads_per_block=256):
+    """Uniform used by each row of a block-level `row_map_reduce` sampling op
+    (ml/primitives.spi:786-791 with rng subsequence = thread-in-block, :927).  Every thread
+    draws one uniform per element it holds (4 for f32) and the reduction keeps the draw that is
+    attached to column 0, i.e. the first draw of the row's lane 0 in that row-iteration."""
+    t = cols // 4
+    r_per_iter = threads_per_block // t
+    r = np.arange(rows)
+    return curand_uniform(curand_words(seed, (r % r_per_iter) * t, 4 * (r // r_per_iter)))
+
+
+def row_uniforms_grid(rows, cols, seed=CONSTANT_SEED, threads_per_block=256, blocks=24):
+    """Same for `grid_row_map_reduce` (subsequence = thread-in-grid, ml/primitives.spi:1014;
+    row-iterations are block-strided, :493)."""
+    t = cols // 4
+    r_per_iter = threads_per_block // t
+    r = np.arange(rows)
+    it = r // r_per_iter
+    sub = (it % blocks) * threads_per_block + (r % r_per_iter) * t
+    return curand_uniform(curand_words(seed, sub, 4 * (it // blocks)))
+
+
+def row_uniforms_gather(n_threads, cols, seed=CONSTANT_SEED, threads_per_block=256):
+    """Same for `row_gather_reduce`, where every *thread* owns one short row and the block
+    transposes them through shared memory (corecuda/transposing_loop.spi:80-91)."""
+    t_per_row = cols // 4
+    d = threads_per_block // t_per_row
+    t = np.arange(n_threads)
+    lt = t % threads_per_block
+    sub = (t // threads_per_block) * threads_per_block + (lt % d) * t_per_row
+    return curand_uniform(curand_words(seed, sub, 4 * (lt // d)))

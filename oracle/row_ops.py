@@ -1,0 +1,241 @@
+"""Row primitives restated in NumPy (f32 / i32 arithmetic).  TEST INFRASTRUCTURE ONLY.
+
+Follows ml/primitives.spi: every function below acts on the innermost dimension of a
+row-major (rows, cols) tensor, exactly like the user lambdas that `row_map`, `row_reduce`
+and `row_map_reduce` (ml/primitives.spi:423-590) run on one row at a time.
+
+Float summation order.  The reference sums a row as: sequentially over the 4 elements a
+thread holds, then a butterfly / scan across the threads of the row
+(ml/primitives.spi:295-348, corecuda/cooperative_groups.spi:58-80); the order inside the
+cooperative-groups collectives is not specified by CUDA.  Two orders are offered here:
+
+  order="sequential"  left-to-right f32 accumulation (np.cumsum), the textbook reading
+  order="wave"        the association the HIP kernels use, restated exactly so that the
+                      cumulative distribution (and therefore the sampled index) can be
+                      compared bit for bit:
+                        lane t owns columns 4t..4t+3 of each 4*T-column chunk (T lanes per row)
+                        s_t   = ((x0 + x1) + x2) + x3
+                        incl  = Hillis-Steele inclusive scan of s over the T lanes
+                                (for d = 1, 2, 4, ...: v_t += v_{t-d} for t >= d)
+                        start = carry + (incl_{t-1} or 0);  out_k = (...(start + x0) + ...) + x_k
+                        carry = carry + incl_{T-1}                      (next chunk)
+"""
+import numpy as np
+
+INT_MAX = np.int32(2147483647)  # corebase/limit.spi, neutral element of `min` on i32
+F32 = np.float32
+
+
+def _f32(x):
+    return np.ascontiguousarray(x, dtype=np.float32)
+
+
+def lanes_per_row(cols):
+    """Lanes that share one row: one lane per 4 columns, rounded up to a power of two, at most 64."""
+    t = 1
+    while t * 4 < cols and t < 64:
+        t *= 2
+    return t
+
+
+# ----------------------------------------------------------------------------------------------
+# reductions
+# ----------------------------------------------------------------------------------------------
+
+def reduce_sum(x):
+    """`reduce 0 (+)` over a whole tensor (ml/primitives.spi:136-197).  Exact for integers."""
+    x = np.asarray(x)
+    if x.dtype.kind in "iu":
+        return x.sum(dtype=x.dtype)
+    return np.float32(x.astype(np.float64).sum())
+
+
+def row_max(x):
+    """`local_max` (ml/primitives.spi:346)."""
+    return _f32(x).max(axis=-1)
+
+
+def row_sum(x):
+    """`local_sum` (ml/primitives.spi:338); f64 accumulation rounded once, compare to tolerance."""
+    return _f32(x).sum(axis=-1, dtype=np.float64).astype(np.float32)
+
+
+def argmax(x):
+    """`local_argmax` (ml/primitives.spi:705-708).  The reference keeps `a` when `a.v > b.v` in a
+    butterfly whose operand order is unspecified, so ties are arbitrary there; this build fixes
+    the lowest index, which is np.argmax."""
+    return np.argmax(_f32(x), axis=-1).astype(np.int32)
+
+
+# ----------------------------------------------------------------------------------------------
+# row maps
+# ----------------------------------------------------------------------------------------------
+
+def softmax(x, shift="max"):
+    """`local_softmax` (ml/primitives.spi:711-716).  The reference shifts by the row *mean*
+    (author's TODO at :712); shifting by the max is the same function of x and is what the HIP
+    kernels do.  Both are offered so the golden files can be checked against either."""
+    x = _f32(x)
+    s = x.max(axis=-1, keepdims=True) if shift == "max" else \
+        (x.sum(axis=-1, keepdims=True, dtype=np.float32) / F32(x.shape[-1]))
+    e = np.exp(x - s)
+    return e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+
+
+def softmax_stats(x):
+    """(row max, sum of exp(x - max)) as emitted by the fused row kernel."""
+    x = _f32(x)
+    m = x.max(axis=-1)
+    return m, np.exp(x - m[..., None]).sum(axis=-1, dtype=np.float32)
+
+
+def masked_softmax(x, size, shift="max"):
+    """`local_masked_softmax` with mask `j < size` (ml/primitives.spi:748-759, ml/layers.spi:409)."""
+    x = _f32(x)
+    mask = np.arange(x.shape[-1]) < size
+    xm = np.where(mask, x, -np.inf).astype(np.float32)
+    if shift == "max":
+        s = xm.max(axis=-1, keepdims=True)
+    else:
+        s = np.where(mask, x, 0).sum(axis=-1, keepdims=True, dtype=np.float32) / F32(mask.sum())
+    e = np.exp(xm - s)
+    return e / e.sum(axis=-1, keepdims=True, dtype=np.float32)
+
+
+def ln_l2(x):
+    """`local_ln_l2` (ml/primitives.spi:701-703): x / sum(x^2), or 0 when the sum is 0."""
+    x = _f32(x)
+    s = (x * x).sum(axis=-1, keepdims=True, dtype=np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return np.where(s != 0, x / s, F32(0)).astype(np.float32)
+
+
+def regret_matching(x):
+    """`local_regret_matching` (ml/primitives.spi:718-722)."""
+    x = _f32(x)
+    r = np.maximum(x, F32(0))
+    s = r.sum(axis=-1, keepdims=True, dtype=np.float32)
+    inv_len = F32(1) / F32(x.shape[-1])
+    with np.errstate(divide="ignore", invalid="ignore"):
+        return np.where(s != 0, r / s, inv_len).astype(np.float32)
+
+
+def masked_regret_matching(x, size):
+    """`local_masked_regret_matching` with mask `j < size` (ml/primitives.spi:761-780)."""
+    x = _f32(x)
+    mask = np.arange(x.shape[-1]) < size
+    r = np.where(mask, np.maximum(x, F32(0)), F32(0)).astype(np.float32)
+    s = r.sum(axis=-1, keepdims=True, dtype=np.float32)
+    inv_len = F32(1) / F32(mask.sum())
+    with np.errstate(divide="ignore", invalid="ignore"):
+        out = np.where(s != 0, r / s, inv_len)
+    return np.where(mask, out, F32(0)).astype(np.float32)
+
+
+def relu(x):
+    """`relu = max 0` (ml/layers.spi:355)."""
+    return np.maximum(_f32(x), F32(0))
+
+
+# ----------------------------------------------------------------------------------------------
+# scans
+# ----------------------------------------------------------------------------------------------
+
+def _wave_scan(x, inclusive=True):
+    x = np.asarray(x)
+    rows, cols = x.shape
+    t = lanes_per_row(cols)
+    chunk = 4 * t
+    n_chunks = -(-cols // chunk)
+    pad = n_chunks * chunk - cols
+    xp = np.concatenate([x, np.zeros((rows, pad), dtype=x.dtype)], axis=1) if pad else x
+    xp = xp.reshape(rows, n_chunks, t, 4)
+    out = np.empty_like(xp)
+    carry = np.zeros(rows, dtype=x.dtype)
+    for c in range(n_chunks):
+        v = xp[:, c]                                  # (rows, T, 4)
+        s = ((v[..., 0] + v[..., 1]) + v[..., 2]) + v[..., 3]
+        incl = s.copy()
+        d = 1
+        while d < t:
+            nxt = incl.copy()
+            nxt[:, d:] = incl[:, d:] + incl[:, :-d]
+            incl = nxt
+            d *= 2
+        excl = np.concatenate([np.zeros((rows, 1), dtype=x.dtype), incl[:, :-1]], axis=1)
+        run = carry[:, None] + excl
+        for k in range(4):
+            if inclusive:
+                run = run + v[..., k]
+                out[:, c, :, k] = run
+            else:
+                out[:, c, :, k] = run
+                run = run + v[..., k]
+        carry = carry + incl[:, -1]
+    return out.reshape(rows, n_chunks * chunk)[:, :cols]
+
+
+def inclusive_scan_sum(x, order="sequential"):
+    """`local_inclusive_scan_sum` (ml/primitives.spi:323-325)."""
+    x = np.asarray(x)
+    if x.dtype.kind in "iu":
+        return np.cumsum(x, axis=-1, dtype=x.dtype)
+    x = _f32(x)
+    if order == "sequential":
+        return np.cumsum(x, axis=-1, dtype=np.float32)
+    return _wave_scan(x.reshape(-1, x.shape[-1]), True).reshape(x.shape)
+
+
+def exclusive_scan(x, order="sequential"):
+    """`local_exclusive_scan config 0 (+)` (ml/primitives.spi:327, used on i32 in test2 :948-950)."""
+    x = np.asarray(x)
+    if x.dtype.kind in "iu" or order == "sequential":
+        c = np.cumsum(x, axis=-1, dtype=x.dtype)
+        return np.concatenate([np.zeros_like(c[..., :1]), c[..., :-1]], axis=-1)
+    return _wave_scan(_f32(x).reshape(-1, x.shape[-1]), False).reshape(x.shape)
+
+
+# ----------------------------------------------------------------------------------------------
+# sampling
+# ----------------------------------------------------------------------------------------------
+
+def discrete_sampling(p, u, cdf=None, order="sequential"):
+    """`local_discrete_sampling` (ml/primitives.spi:782-798).
+
+    cdf = inclusive scan of p; m = max cdf over the entries with p > 0; thr = u * m (f32);
+    result = the smallest j with p_j > 0 and cdf_j - thr >= 0.  `u` is one uniform in (0, 1]
+    per row.  A row without any p > 0 yields INT_MAX (the reference asserts in debug builds and
+    returns the reduction's neutral element otherwise).  Pass `cdf` to sample from a given
+    cumulative distribution instead of recomputing it."""
+    p = _f32(p)
+    u = _f32(u)
+    if cdf is None:
+        cdf = inclusive_scan_sum(p, order)
+    cdf = _f32(cdf)
+    valid = p > 0
+    m = np.where(valid, cdf, -np.inf).max(axis=-1)
+    thr = (u * m).astype(np.float32)
+    hit = valid & ((cdf - thr[..., None]).astype(np.float32) >= 0)
+    j = np.arange(p.shape[-1], dtype=np.int64)
+    idx = np.where(hit, j, np.int64(INT_MAX)).min(axis=-1)
+    return idx.astype(np.int32)
+
+
+def get_prob(p, action):
+    """`local_get_prob` (ml/primitives.spi:824-830): probability of the selected action."""
+    p = _f32(p)
+    return np.take_along_axis(p, np.asarray(action, dtype=np.int64)[..., None], axis=-1)[..., 0]
+
+
+def binarize(x, modulo):
+    """`local_binarize` (ml/primitives.spi:817-821): bit j set iff x_j > 0, OR-ed, mod `modulo`.
+    Device shifts wrap at 32 bits: `1 << j` uses j mod 32 on the reference's hardware."""
+    x = _f32(x)
+    j = np.arange(x.shape[-1], dtype=np.uint64) % np.uint64(32)
+    bits = np.where(x > 0, np.uint64(1) << j, np.uint64(0))
+    return (np.bitwise_or.reduce(bits, axis=-1) & np.uint64(0xFFFFFFFF)) % np.uint64(modulo)
+
+
+def transpose_inner(x):
+    """`grid_transpose_snd` (ml/primitives.spi:36-112): swap the two innermost dimensions."""
+    return np.ascontiguousarray(np.swapaxes(np.asarray(x), -1, -2))

@@ -1,0 +1,161 @@
+"""Checks that pin the oracle where the reference holds no vectors: known-answer vectors of the
+published algorithm, closed forms, brute force on tiny inputs and invariants."""
+import numpy as np
+import pytest
+
+from oracle import gemm, layers, philox, row_ops
+
+
+def test_philox_known_answers():
+    # Random123 kat_vectors, philox4x32 with 10 rounds
+    kat = [
+        ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+        ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+        ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+         (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
+    ]
+    for ctr, key, want in kat:
+        got = philox.philox4x32_10(np.array(ctr, dtype=np.uint32), np.array(key, dtype=np.uint32))
+        assert tuple(int(v) for v in got) == want
+
+
+def test_curand_uniform_range():
+    u = philox.curand_uniform(np.array([0, 1, 0x7fffffff, 0xffffffff], dtype=np.uint32))
+    assert u[0] > 0 and u[-1] == 1.0 and (np.diff(u) >= 0).all()
+
+
+def test_gemm_bruteforce_and_algebra():
+    rng = np.random.default_rng(0)
+    a = rng.standard_normal((16, 8), dtype=np.float32)
+    b = rng.standard_normal((16, 8), dtype=np.float32)
+    c = rng.standard_normal((16, 16), dtype=np.float32)
+    for alpha, beta in ((1.0, 0.0), (1.0, 1.0), (0.5, -2.0)):
+        want = gemm.gemm_abt_bruteforce(a, b, c, alpha, beta)
+        got = gemm.gemm_abt(a, b, c, alpha, beta)
+        assert gemm.rel_frobenius(got, want) < 1e-6
+    # a transposed operand or a swapped A/B must fail: B = identity gives C = A, not A^T
+    a2 = rng.standard_normal((8, 8), dtype=np.float32)
+    assert (gemm.gemm_abt(a2, np.eye(8, dtype=np.float32)) == a2).all()
+    # non-square: C[i, j] = <A_i, B_j>
+    a3 = np.arange(6, dtype=np.float32).reshape(2, 3)
+    b3 = np.arange(12, dtype=np.float32).reshape(4, 3)
+    assert (gemm.gemm_abt(a3, b3) == np.array([[5, 14, 23, 32], [14, 50, 86, 122]], dtype=np.float32)).all()
+    # NaNs in C do not propagate when beta == 0 (ml/matmul/kernel.spi:152-154)
+    assert np.isfinite(gemm.gemm_abt(a, b, np.full((16, 16), np.nan, dtype=np.float32), 1.0, 0.0)).all()
+    with pytest.raises(AssertionError):
+        gemm.gemm_abt(a, b, alpha=0.0)
+
+
+def test_gemm_integer_inputs_exact():
+    # the reference's commented `arange` alternative (ml/matmul/run.spi:52): integer results are exact
+    a = (np.arange(32 * 16) % 7).astype(np.float32).reshape(32, 16)
+    b = (np.arange(24 * 16) % 5).astype(np.float32).reshape(24, 16)
+    want = (a.astype(np.int64) @ b.astype(np.int64).T)
+    assert (gemm.gemm_abt(a, b).astype(np.int64) == want).all()
+
+
+def test_bf16_rounding():
+    x = np.array([1.0, 1.00390625, 1.01171875, -2.5, 3.0e38, 1e-40, np.inf], dtype=np.float32)
+    bits = gemm.f32_to_bf16_bits(x)
+    back = gemm.bf16_bits_to_f32(bits)
+    assert back[0] == 1.0 and back[3] == -2.5 and np.isinf(back[-1])
+    # 1 + 2^-8 is a tie between 1.0 and 1 + 2^-7: RNE picks the even mantissa (1.0)
+    assert back[1] == 1.0
+    # 1 + 3*2^-8 is a tie between 1+2^-7 (odd) and 1+2^-6 (even)
+    assert back[2] == np.float32(1.015625)
+    import torch
+    t = torch.from_numpy(np.random.default_rng(1).standard_normal(4096).astype(np.float32))
+    want = t.to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (gemm.f32_to_bf16_bits(t.numpy()) == want).all()
+    assert np.isnan(gemm.bf16_bits_to_f32(gemm.f32_to_bf16_bits(np.array([np.nan], dtype=np.float32)))).all()
+
+
+def test_tile_heuristic_matches_generated_code():
+    # ml/matmul/run.py (96 KB build): 128x128x64 tiles (ldm 136 = 128 + 8); 224 KB: 128x256x64
+    assert gemm.matmul_tile_config(8192, 8192, 4096, 96 * 1024) == (128, 128, 64)
+    assert gemm.matmul_tile_config(8192, 8192, 4096, 224 * 1024) == (128, 256, 64)
+    assert gemm.matmul_tile_config(16, 16, 8) == (16, 16, 8)
+    with pytest.raises(AssertionError):
+        gemm.matmul_tile_config(16384, 3, 256)
+
+
+def test_softmax_invariants():
+    rng = np.random.default_rng(2)
+    x = (rng.standard_normal((64, 256)) * 2).astype(np.float32)
+    p = row_ops.softmax(x)
+    assert np.abs(p.sum(axis=1) - 1).max() < 1e-5
+    assert np.abs(row_ops.softmax(x + 3.0) - p).max() < 1e-6
+    assert np.abs(row_ops.softmax(x, "mean") - p).max() < 1e-6
+    assert (row_ops.masked_softmax(x, 256) == p).all()
+    m, s = row_ops.softmax_stats(x)
+    assert (m == x.max(axis=1)).all() and np.allclose(np.exp(x - m[:, None]) / s[:, None], p, rtol=1e-6)
+
+
+def test_regret_matching_closed_forms():
+    x = np.array([[1, -1, 3, 0], [-1, -2, -3, -4], [0, 0, 0, 0], [2, 2, 0, -5]], dtype=np.float32)
+    want = np.array([[.25, 0, .75, 0], [.25] * 4, [.25] * 4, [.5, .5, 0, 0]], dtype=np.float32)
+    assert (row_ops.regret_matching(x) == want).all()
+    assert (row_ops.masked_regret_matching(x, 4) == want).all()
+    m = row_ops.masked_regret_matching(x, 2)
+    assert (m == np.array([[1, 0, 0, 0], [.5, .5, 0, 0], [.5, .5, 0, 0], [.5, .5, 0, 0]], dtype=np.float32)).all()
+
+
+def test_scan_orders():
+    rng = np.random.default_rng(3)
+    for cols in (4, 12, 16, 64, 128, 256, 260, 512, 1024):
+        xi = rng.integers(-1000, 1000, size=(7, cols)).astype(np.int32)
+        assert (row_ops._wave_scan(xi, True) == np.cumsum(xi, axis=1)).all()
+        assert (row_ops._wave_scan(xi, False) == np.cumsum(xi, axis=1) - xi).all()
+        xf = rng.random((7, cols), dtype=np.float32)
+        seq = row_ops.inclusive_scan_sum(xf, "sequential")
+        wav = row_ops.inclusive_scan_sum(xf, "wave")
+        assert np.abs(seq - wav).max() <= 1e-6 * cols
+        # brute-force sequential reading
+        acc = np.float32(0)
+        for j in range(cols):
+            acc = np.float32(acc + xf[0, j])
+            assert acc == seq[0, j]
+
+
+def test_discrete_sampling_invariants():
+    rng = np.random.default_rng(4)
+    p = row_ops.softmax((rng.standard_normal((200, 64)) * 2).astype(np.float32))
+    p[:, ::3] = 0  # zero-probability entries must never be selected
+    u = (1 - rng.random(200, dtype=np.float32)).astype(np.float32)
+    idx = row_ops.discrete_sampling(p, u)
+    assert (np.take_along_axis(p, idx[:, None].astype(np.int64), 1) > 0).all()
+    tiny = np.full(200, np.float32(1e-30))
+    first = np.argmax(p > 0, axis=1)
+    last = p.shape[1] - 1 - np.argmax(p[:, ::-1] > 0, axis=1)
+    assert (row_ops.discrete_sampling(p, tiny) == first).all()
+    assert (row_ops.discrete_sampling(p, np.ones(200, dtype=np.float32)) == last).all()
+    # monotone in u
+    us = np.sort(rng.random(50, dtype=np.float32))[::-1].copy()
+    one = np.repeat(p[:1], 50, axis=0)
+    assert (np.diff(row_ops.discrete_sampling(one, 1 - us)) >= 0).all()
+    # brute force
+    for r in range(20):
+        cdf = np.cumsum(p[r], dtype=np.float32)
+        m = max(cdf[j] for j in range(64) if p[r, j] > 0)
+        thr = np.float32(u[r] * m)
+        want = min(j for j in range(64) if p[r, j] > 0 and np.float32(cdf[j] - thr) >= 0)
+        assert idx[r] == want
+    assert row_ops.discrete_sampling(np.zeros((1, 8), np.float32), np.ones(1, np.float32))[0] == row_ops.INT_MAX
+
+
+def test_mlp_forward_composition():
+    rng = np.random.default_rng(5)
+    x = (rng.random((32, 32)) < 0.2).astype(np.float32)
+    ws = [gemm.round_to(layers.weight_init(rng, o, i), "f16") for o, i in ((256, 32), (256, 256), (256, 256), (3, 256))]
+    u = (1 - rng.random(32, dtype=np.float32)).astype(np.float32)
+    policy, action, logits = layers.mlp_forward(x, ws, u=u)
+    h = x
+    for w in ws[:-1]:
+        h = np.maximum(h.astype(np.float64) @ w.astype(np.float64).T, 0)
+    want_logits = h @ ws[-1].astype(np.float64).T
+    assert gemm.rel_frobenius(logits, want_logits) < 1e-5
+    e = np.exp(want_logits - want_logits.max(axis=1, keepdims=True))
+    assert np.abs(policy - e / e.sum(axis=1, keepdims=True)).max() < 1e-5
+    assert ((action >= 0) & (action < 3)).all()
+    pol16, _, _ = layers.mlp_forward(x, ws, u=u, act_dtype="f16")
+    assert gemm.rel_frobenius(pol16, policy) < 3e-3
