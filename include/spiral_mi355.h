@@ -1,0 +1,230 @@
+/*
+ * spiral_mi355.h - C ABI of libspiral_mi355.so, the MI355X (gfx950) implementation of the
+ * data-parallel hot path of mrakgr/Spiral-s-ML-Library: tiled GEMM C = A.B^T, dense-layer
+ * forward, and the row primitives (reductions, scans, softmax, argmax, categorical sampling).
+ *
+ * The reference has no C ABI: its device entry points are `extern "C" __global__ entry{N}`
+ * kernels compiled at import time by CuPy's RawModule and launched with
+ * `fn((blocks,),(threads,),(arrays...),shared_mem=S)` (corecuda/base.spi:52-111), with all
+ * shapes baked in as compile-time literals.  Each function below names the reference
+ * interface it stands in for.
+ *
+ * Conventions (all functions):
+ *   - every tensor is row-major, contiguous, innermost stride 1 (corebase/tensorm/utils.spir:27);
+ *   - device pointers must be 16-byte aligned (corecuda/base.spi:158 asserts the same);
+ *   - the library borrows the buffers, writes results in place, never allocates device memory
+ *     and never synchronises: work is enqueued on `stream` (a hipStream_t, NULL = default stream);
+ *   - return value: SP_OK (0) or a negative sp_status; sp_last_error_string() describes the
+ *     last failure on the calling thread.  Nothing throws.
+ */
+#ifndef SPIRAL_MI355_H
+#define SPIRAL_MI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    SP_OK = 0,
+    SP_ERR_NULL = -1,        /* a required pointer is NULL */
+    SP_ERR_SHAPE = -2,       /* a dimension is non-positive, too large, or violates a divisibility rule */
+    SP_ERR_ALIGN = -3,       /* a pointer is not 16-byte aligned */
+    SP_ERR_DTYPE = -4,       /* unsupported dtype combination */
+    SP_ERR_ARG = -5,         /* any other invalid argument (alpha == 0, unknown op, bad mask size ...) */
+    SP_ERR_UNSUPPORTED = -6, /* valid request this build has no kernel for */
+    SP_ERR_DEVICE = -7       /* HIP reported an error at launch; see sp_last_error_string() */
+} sp_status;
+
+typedef enum { SP_F32 = 0, SP_F16 = 1, SP_BF16 = 2 } sp_dtype;
+
+/* ------------------------------------------------------------------------------------------ */
+/* library                                                                                     */
+/* ------------------------------------------------------------------------------------------ */
+
+/* Human-readable description of the last error on this thread ("" if none). */
+const char* sp_last_error_string(void);
+
+typedef struct {
+    char name[128];
+    char arch[64];              /* gcnArchName, must start with "gfx950" for the kernels to run */
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t lds_bytes_per_cu;   /* shared memory per workgroup limit */
+    int32_t max_clock_khz;
+    int64_t hbm_bytes;
+    int32_t l2_bytes;
+} sp_device_info_t;
+
+/* Replaces the host-side device probing of corecuda/base.spi:73 (SM-count assert) and
+ * ml/max_blocks_per_sm.py:2-31 (device attribute queries). */
+int sp_device_info(sp_device_info_t* out);
+
+/* Occupancy report for a named kernel family of this library ("gemm_bf16_256x256", "row_ops",
+ * "mlp_forward", ...): registers, LDS bytes and resident workgroups per CU.  Stands in for
+ * ml/max_blocks_per_sm.py:2-31.  Returns SP_ERR_ARG for an unknown name. */
+typedef struct {
+    int32_t vgprs;              /* architected + accumulation VGPRs per lane (from the code object) */
+    int32_t sgprs;
+    int32_t static_lds_bytes;
+    int32_t threads_per_block;
+    int32_t max_blocks_per_cu;
+} sp_kernel_info_t;
+int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
+
+/* ------------------------------------------------------------------------------------------ */
+/* GEMM                                                                                        */
+/* ------------------------------------------------------------------------------------------ */
+
+#define SP_GEMM_RELU 0x1u       /* apply max(0, .) after bias (build extension; the reference
+                                   fuses nothing: game/leduc/model_cem.spi:59 "TODO: Fuse this relu") */
+#define SP_GEMM_FORCE_GENERIC 0x100u /* testing aid: use the shape-agnostic kernel even for tileable shapes */
+
+/*
+ * C = alpha * A . B^T + beta * C  [+ bias[n]] [ReLU]
+ *
+ * Replaces `matmul_tf32 false true alpha a b beta c` (ml/matmul/run.spi:21-26 ->
+ * matmul_tf32_template, ml/matmul/kernel.spi:25-240; generated entry point
+ * `entry0(float* A, float* B, float* C)`, ml/matmul/run.py:300,1232) and the grid-strided
+ * variant tests/matmul/test3_kernel.spi:148.
+ *
+ *   A (M,K), B (N,K), C (M,N) row-major.  dtype_in in {SP_F32, SP_F16, SP_BF16} is the storage
+ *   type of A and B; products are exact and accumulation is f32 (MFMA).  dtype_out is the storage
+ *   type of C (SP_F32, or the same 16-bit type as the input).  bias (N,) f32 may be NULL.
+ *   alpha must be non-zero (kernel.spi:49).  beta == 0 means C is never read, so NaNs in the
+ *   old C do not propagate (kernel.spi:152-154).
+ *   Fast MFMA path: M, N multiples of 64 and K a multiple of 64 (16-bit) / 32 (f32); any other
+ *   positive shape with K a multiple of 8 (16-bit) / 4 (f32) runs on a slower general kernel.
+ */
+int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
+                int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream);
+
+/* Which tile configuration sp_gemm_abt picks for a shape (the counterpart of
+ * `matmul_config_tf32`, ml/matmul/run.spi:8-19).  Writes block tile sizes and the workgroup size;
+ * tile_m == 0 means the general kernel. */
+int sp_gemm_config(int dtype_in, int64_t M, int64_t N, int64_t K,
+                   int32_t* tile_m, int32_t* tile_n, int32_t* tile_k, int32_t* threads);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Row primitives                                                                              */
+/* ------------------------------------------------------------------------------------------ */
+
+/*
+ * Fused row pipeline over logits (rows, cols) f32: row max, sum of exp(x - max), softmax,
+ * inclusive prefix sum of the probabilities, argmax, and inverse-CDF sampling with one uniform
+ * u[row] in (0, 1] per row.  One pass over HBM; any output pointer may be NULL to skip it.
+ *
+ * Replaces the chain row_reduce(local_argmax) / row_map(local_softmax + local_inclusive_scan_sum) /
+ * row_map_reduce(local_softmax_and_discrete_sampling) of ml/primitives.spi:514-536,705-716,782-802
+ * (test2, :925-955).  Sampling rule (:782-798): m = max cdf over p > 0; result = smallest j with
+ * p_j > 0 and cdf_j >= u * m.  argmax ties resolve to the lowest index.
+ * cols: multiple of 4, 4 <= cols <= 1024.
+ */
+int sp_row_ops(const float* logits, const float* u, float* rowmax, float* rowsum, float* probs, float* cdf,
+               int32_t* argmax, int32_t* sample, int64_t rows, int64_t cols, uint32_t flags, void* stream);
+
+typedef enum {
+    SP_ROW_IDENTITY = 0,                /* row_map (fun config x i j_tns => x)          primitives.spi:929 */
+    SP_ROW_SOFTMAX = 1,                 /* local_softmax                                primitives.spi:711-716 */
+    SP_ROW_MASKED_SOFTMAX = 2,          /* local_masked_softmax, mask j < mask_size     primitives.spi:748-759 */
+    SP_ROW_LN_L2 = 3,                   /* local_ln_l2                                  primitives.spi:701-703 */
+    SP_ROW_REGRET_MATCHING = 4,         /* local_regret_matching                        primitives.spi:718-722 */
+    SP_ROW_MASKED_REGRET_MATCHING = 5,  /* local_masked_regret_matching                 primitives.spi:761-780 */
+    SP_ROW_INCLUSIVE_SCAN = 6,          /* local_inclusive_scan_sum                     primitives.spi:323-325 */
+    SP_ROW_EXCLUSIVE_SCAN = 7           /* local_exclusive_scan config 0 (+)            primitives.spi:327 */
+} sp_row_op;
+
+/* out = op(x) row by row, x and out (rows, cols) f32.  Replaces `row_map f x out`
+ * (ml/primitives.spi:514-520) for the lambdas listed in sp_row_op.  mask_size is used by the
+ * masked ops only (1 <= mask_size <= cols). */
+int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, int64_t cols, int32_t mask_size, void* stream);
+
+/* Integer scans (SP_ROW_INCLUSIVE_SCAN / SP_ROW_EXCLUSIVE_SCAN / SP_ROW_IDENTITY) on i32 rows; exact
+ * (wrap-around two's complement like the device adds of the reference, test2 :948-950). */
+int sp_row_map_i32(int op, const int32_t* x, int32_t* out, int64_t rows, int64_t cols, void* stream);
+
+/* How a sampling op obtains its uniforms when no `u` tensor is given: the reference's device-side
+ * Philox4_32_10 stream (corecuda/random.spi:22-32,84) with curand_init(seed, subsequence, 0). */
+typedef enum {
+    SP_PHILOX_BLOCK = 0,   /* row_map_reduce: subsequence = thread-in-block        primitives.spi:927 */
+    SP_PHILOX_GRID = 1,    /* grid_row_map_reduce: subsequence = thread-in-grid    primitives.spi:1014,493 */
+    SP_PHILOX_GATHER = 2   /* row_gather_reduce: one row per thread                primitives.spi:409-413 */
+} sp_philox_mode;
+
+typedef struct {
+    uint64_t seed;               /* reference: 12344321 (corecuda/cupy.spi:6) */
+    int32_t mode;                /* sp_philox_mode */
+    int32_t threads_per_block;   /* reference: 256 */
+    int32_t blocks_per_grid;     /* reference: 24 (RTX 4060) or 112 (H100), corecuda/base.spi:14-42 */
+    int32_t reserved;
+} sp_philox_t;
+
+/*
+ * probs = op(x) (op in IDENTITY, SOFTMAX, MASKED_SOFTMAX, REGRET_MATCHING, MASKED_REGRET_MATCHING),
+ * then sample = local_discrete_sampling(probs).  Replaces `row_map_reduce
+ * (local_softmax_and_discrete_sampling rng) x probs sample` and its masked / regret-matching
+ * siblings (ml/primitives.spi:528-536,800-814).  Exactly one of `u` (rows,) f32 in (0,1] and
+ * `philox` must be given.  probs_out, cdf_out and u_out (the uniform each row used) may be NULL.
+ */
+int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* philox, float* probs_out, float* cdf_out,
+                  float* u_out, int32_t* sample_out, int64_t rows, int64_t cols, int32_t mask_size, void* stream);
+
+typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID = 3 } sp_map_op;
+
+/* out[i] = f(x[i]) over n f32 elements (n multiple of 4).  Replaces `primitives.map f from to`
+ * (ml/primitives.spi:115-133) for the activation lambdas of ml/layers.spi:353-355. */
+int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream);
+
+/* Sum of all n elements into out[0].  dtype: 0 = f32, 1 = i32, 2 = u64.  `workspace` must hold
+ * at least sp_reduce_workspace_bytes() bytes of device memory (partials; no allocation here).
+ * Replaces `reduce 0 (+)` / `grid_reduce grid 0 (+)` (ml/primitives.spi:136-197, test6 :1102-1105). */
+int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes, void* stream);
+int64_t sp_reduce_workspace_bytes(void);
+
+/* to[a][c][b] = from[a][b][c] for 4-byte elements.  Replaces `grid_transpose_snd`
+ * (ml/primitives.spi:36-112, test5 :1078-1088). */
+int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int64_t c, void* stream);
+
+/* ------------------------------------------------------------------------------------------ */
+/* Dense layers                                                                                */
+/* ------------------------------------------------------------------------------------------ */
+
+typedef enum {
+    SP_HEAD_NONE = 0,            /* policy_out receives the last layer's outputs */
+    SP_HEAD_SOFTMAX = 1,         /* softmax                          ml/layers.spi:374-380 */
+    SP_HEAD_REGRET_MATCHING = 2, /* regret_matching                  ml/layers.spi:382-388 */
+    SP_HEAD_SOFTMAX_RM = 3       /* softmax, then regret matching of the probabilities */
+} sp_head;
+
+/*
+ * Fused forward pass of a dense stack: h_0 = x; h_{i+1} = relu(h_i . W_i^T [+ b_i]) for all but the
+ * last layer; policy = head(h_{n-1} . W_{n-1}^T [+ b_{n-1}]); action = discrete sample of policy
+ * with u[row].  One kernel; activations never leave the CU.
+ *
+ * Replaces the interpreter chain block_matmul -> block_map(relu) -> ... -> block_row_map_reduce
+ * (ml/layers.spi:194-240; generated ml/layers.py:4531-4546, launched through
+ * `entry0(weights, workspace, adjoint)`, ml/layers.py:4500,5894), where every arrow is a round
+ * trip through the global-memory workspace.
+ *
+ *   dtype        SP_F16 or SP_BF16: storage type of x and of every weight matrix
+ *   x            (batch, dims[0])
+ *   weights[i]   (dims[i+1], dims[i]) row-major = the B operand of A.B^T (ml/layers.spi:467);
+ *                `weights` is a HOST array of n_layers device pointers
+ *   biases       NULL, or a host array of n_layers device pointers to f32 (dims[i+1],) (entries may be NULL)
+ *   dims         host array of n_layers + 1 layer widths; dims[0..n_layers-1] multiples of 16 and <= 512,
+ *                hidden widths multiples of 32 and <= 512, dims[n_layers] <= 64
+ *   u            (batch,) f32 in (0, 1], or NULL when action_out is NULL
+ *   policy_out   (batch, dims[n_layers]) f32
+ *   action_out   (batch,) i32 or NULL
+ *   logits_out   (batch, dims[n_layers]) f32 or NULL
+ *   mask_size    0 = no mask, else the head only considers columns j < mask_size (ml/layers.spi:409-424)
+ */
+int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights, const float* const* biases,
+                   const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,
+                   int64_t batch, int32_t head, int32_t mask_size, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SPIRAL_MI355_H */

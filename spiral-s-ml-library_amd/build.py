@@ -1,0 +1,64 @@
+#!/usr/bin/env python3
+"""Build libspiral_mi355.so (HIP, gfx950) in-tree.
+
+    python spiral-s-ml-library_amd/build.py [--force]
+
+hipcc cross-compiles for gfx950 without a GPU.  The shared library is written next to this file;
+the Python host modules under ml/ load it with ctypes and fail loudly when it is missing.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
+LIB = os.path.join(HERE, "libspiral_mi355.so")
+SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip"]
+FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"),
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
+         "-Wno-unknown-warning-option"]
+
+
+def hipcc():
+    for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
+        if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
+            return cand
+    raise RuntimeError("hipcc not found")
+
+
+def _run(cmd):
+    p = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(ln for ln in p.stdout.splitlines() if "packed-fp32-ops" not in ln)
+    if p.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build(force=True, verbose=False):
+    """Compile every HIP source and link the shared library.  Returns the library path."""
+    os.makedirs(OBJ, exist_ok=True)
+    cc = hipcc()
+    headers = [os.path.join(CSRC, "common.h"), os.path.join(ROOT, "include", "spiral_mi355.h")]
+    newest_header = max(os.path.getmtime(h) for h in headers)
+
+    def compile_one(src):
+        s = os.path.join(CSRC, src)
+        o = os.path.join(OBJ, src.replace(".hip", ".o"))
+        if not force and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_header):
+            return o
+        out = _run([cc] + FLAGS + ["-c", s, "-o", o])
+        if verbose and out.strip():
+            print(out)
+        return o
+
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
+        objs = list(ex.map(compile_one, SOURCES))
+    _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(force="--force" in sys.argv, verbose=True))

@@ -1,0 +1,123 @@
+// Library-level entry points: error slot, device probing, kernel occupancy report.
+#include "common.h"
+
+#include <string.h>
+
+#include <mutex>
+#include <string>
+#include <vector>
+
+namespace sp {
+
+char* error_buffer() {
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+
+struct DeviceCache {
+    bool probed = false;
+    bool ok = false;
+    int cus = 0;
+    char arch[64] = {0};
+};
+
+static DeviceCache& device_cache(int dev) {
+    static DeviceCache cache[64];
+    return cache[dev < 0 || dev >= 64 ? 0 : dev];
+}
+
+static std::mutex g_mutex;
+
+static int probe(DeviceCache** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipGetDevice failed: %s", hipGetErrorString(e));
+    DeviceCache& c = device_cache(dev);
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!c.probed) {
+        hipDeviceProp_t prop;
+        e = hipGetDeviceProperties(&prop, dev);
+        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+        strncpy(c.arch, prop.gcnArchName, sizeof(c.arch) - 1);
+        c.cus = prop.multiProcessorCount;
+        c.ok = strncmp(c.arch, "gfx950", 6) == 0;
+        c.probed = true;
+    }
+    *out = &c;
+    return SP_OK;
+}
+
+int require_gfx950(const char* what) {
+    DeviceCache* c = nullptr;
+    int rc = probe(&c);
+    if (rc != SP_OK) return rc;
+    if (!c->ok)
+        return fail(SP_ERR_DEVICE, "%s: this library is built for gfx950 (MI355X) only; current device is %s", what,
+                    c->arch);
+    return SP_OK;
+}
+
+int device_cu_count() {
+    DeviceCache* c = nullptr;
+    if (probe(&c) != SP_OK || c->cus <= 0) return 256;
+    return c->cus;
+}
+
+struct KernelEntry {
+    std::string name;
+    const void* fn;
+    int threads;
+};
+
+static std::vector<KernelEntry>& registry() {
+    static std::vector<KernelEntry> r;
+    return r;
+}
+
+void register_kernel(const char* name, const void* fn, int threads) { registry().push_back({name, fn, threads}); }
+
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" const char* sp_last_error_string(void) { return error_buffer(); }
+
+extern "C" int sp_device_info(sp_device_info_t* out) {
+    if (out == nullptr) return fail(SP_ERR_NULL, "sp_device_info: out is NULL");
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipGetDevice failed: %s", hipGetErrorString(e));
+    hipDeviceProp_t prop;
+    e = hipGetDeviceProperties(&prop, dev);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    memset(out, 0, sizeof(*out));
+    strncpy(out->name, prop.name, sizeof(out->name) - 1);
+    strncpy(out->arch, prop.gcnArchName, sizeof(out->arch) - 1);
+    out->compute_units = prop.multiProcessorCount;
+    out->wavefront_size = prop.warpSize;
+    out->lds_bytes_per_cu = (int32_t)prop.sharedMemPerBlock;
+    out->max_clock_khz = prop.clockRate;
+    out->hbm_bytes = (int64_t)prop.totalGlobalMem;
+    out->l2_bytes = prop.l2CacheSize;
+    return SP_OK;
+}
+
+extern "C" int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out) {
+    if (kernel_family == nullptr || out == nullptr) return fail(SP_ERR_NULL, "sp_kernel_info: NULL argument");
+    for (const KernelEntry& k : registry()) {
+        if (k.name != kernel_family) continue;
+        hipFuncAttributes attr;
+        hipError_t e = hipFuncGetAttributes(&attr, k.fn);
+        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncGetAttributes failed: %s", hipGetErrorString(e));
+        out->vgprs = attr.numRegs;
+        out->sgprs = 0;
+        out->static_lds_bytes = (int32_t)attr.sharedSizeBytes;
+        out->threads_per_block = k.threads;
+        int blocks = 0;
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, k.fn, k.threads, 0);
+        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "occupancy query failed: %s", hipGetErrorString(e));
+        out->max_blocks_per_cu = blocks;
+        return SP_OK;
+    }
+    return fail(SP_ERR_ARG, "sp_kernel_info: unknown kernel family '%s'", kernel_family);
+}

@@ -1,0 +1,165 @@
+// Elementwise map, full-tensor sum and inner-dimension transpose for gfx950.  All three are
+// HBM-bound: 16-byte accesses, grid-stride loops, no MFMA.
+//
+// Semantics: primitives.map (ml/primitives.spi:115-133), reduce / grid_reduce (:136-197),
+// grid_transpose_snd (:36-112).
+#include "common.h"
+
+namespace sp {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+constexpr int EW_THREADS = 256;
+constexpr int REDUCE_MAX_BLOCKS = 1024;
+
+template <int OP>
+__device__ __forceinline__ float map_op(float x) {
+    if constexpr (OP == SP_MAP_RELU) return fmaxf(x, 0.f);
+    else if constexpr (OP == SP_MAP_TANH) return tanhf(x);
+    else if constexpr (OP == SP_MAP_SIGMOID) return 1.f / (1.f + expf(-x));
+    else return x;
+}
+
+template <int OP>
+__global__ __launch_bounds__(EW_THREADS) void map_kernel(const f32x4* __restrict__ x, f32x4* __restrict__ out, long n4) {
+    const long stride = (long)gridDim.x * EW_THREADS;
+    for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < n4; i += stride) {
+        f32x4 v = x[i];
+        v.x = map_op<OP>(v.x); v.y = map_op<OP>(v.y); v.z = map_op<OP>(v.z); v.w = map_op<OP>(v.w);
+        out[i] = v;
+    }
+}
+
+// Block-wide sum: lanes -> wave (shuffles) -> LDS (one slot per wave) -> first wave.
+template <typename T>
+__device__ __forceinline__ T block_sum(T v, T* slots) {
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) v += __shfl_xor(v, d, WAVE);
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+    if (lane == 0) slots[wave] = v;
+    __syncthreads();
+    T r = (threadIdx.x < EW_THREADS / WAVE) ? slots[threadIdx.x] : T(0);
+    if (wave == 0) {
+#pragma unroll
+        for (int d = 1; d < EW_THREADS / WAVE; d <<= 1) r += __shfl_xor(r, d, WAVE);
+    }
+    __syncthreads();
+    return r;  // valid in wave 0
+}
+
+template <typename T>
+__global__ __launch_bounds__(EW_THREADS) void reduce_partial_kernel(const T* __restrict__ x, T* __restrict__ partial, long n) {
+    __shared__ T slots[EW_THREADS / WAVE];
+    T acc = T(0);
+    const long stride = (long)gridDim.x * EW_THREADS;
+    for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) acc += x[i];
+    acc = block_sum(acc, slots);
+    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(EW_THREADS) void reduce_final_kernel(const T* __restrict__ partial, T* __restrict__ out, int count) {
+    __shared__ T slots[EW_THREADS / WAVE];
+    T acc = T(0);
+    for (int i = threadIdx.x; i < count; i += EW_THREADS) acc += partial[i];
+    acc = block_sum(acc, slots);
+    if (threadIdx.x == 0) out[0] = acc;
+}
+
+// to[a][c][b] = from[a][b][c]; 64x64 tiles through LDS, padded by one word per row so that the
+// transposed (column) reads hit 64 different banks.
+__global__ __launch_bounds__(EW_THREADS) void transpose_kernel(const unsigned* __restrict__ from, unsigned* __restrict__ to,
+                                                               long B, long C, long tiles_b, long tiles_c) {
+    __shared__ unsigned tile[64][65];
+    const long t = blockIdx.x;
+    const long a = t / (tiles_b * tiles_c);
+    const long tb = (t / tiles_c) % tiles_b, tc = t % tiles_c;
+    const unsigned* src = from + a * B * C;
+    unsigned* dst = to + a * B * C;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        const long b = tb * 64 + r, c = tc * 64 + tx;
+        if (b < B && c < C) tile[r][tx] = src[b * C + c];
+    }
+    __syncthreads();
+    for (int r = ty; r < 64; r += 4) {
+        const long c = tc * 64 + r, b = tb * 64 + tx;
+        if (b < B && c < C) dst[c * B + b] = tile[tx][r];
+    }
+}
+
+template <typename T>
+static int run_reduce(const void* x, void* out, int64_t n, void* workspace, hipStream_t stream) {
+    long blocks = (n + EW_THREADS * 8 - 1) / (EW_THREADS * 8);
+    if (blocks > REDUCE_MAX_BLOCKS) blocks = REDUCE_MAX_BLOCKS;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(reduce_partial_kernel<T>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x,
+                       (T*)workspace, (long)n);
+    hipLaunchKernelGGL(reduce_final_kernel<T>, dim3(1), dim3(EW_THREADS), 0, stream, (const T*)workspace, (T*)out,
+                       (int)blocks);
+    return check_launch("sp_reduce_sum");
+}
+
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    if (n <= 0 || n % 4 != 0) return fail(SP_ERR_SHAPE, "sp_map_f32: n must be a positive multiple of 4, got %lld", (long long)n);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    const long n4 = n / 4;
+    long blocks = (n4 + EW_THREADS - 1) / EW_THREADS;
+    const long cap = (long)device_cu_count() * 8;
+    if (blocks > cap) blocks = cap;
+    hipStream_t s = (hipStream_t)stream;
+    const f32x4* xi = (const f32x4*)x;
+    f32x4* xo = (f32x4*)out;
+    switch (op) {
+        case SP_MAP_COPY: hipLaunchKernelGGL(map_kernel<SP_MAP_COPY>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, s, xi, xo, n4); break;
+        case SP_MAP_RELU: hipLaunchKernelGGL(map_kernel<SP_MAP_RELU>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, s, xi, xo, n4); break;
+        case SP_MAP_TANH: hipLaunchKernelGGL(map_kernel<SP_MAP_TANH>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, s, xi, xo, n4); break;
+        case SP_MAP_SIGMOID: hipLaunchKernelGGL(map_kernel<SP_MAP_SIGMOID>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, s, xi, xo, n4); break;
+        default: return fail(SP_ERR_ARG, "sp_map_f32: unknown op %d", op);
+    }
+    return check_launch(__func__);
+}
+
+extern "C" int64_t sp_reduce_workspace_bytes(void) { return (int64_t)REDUCE_MAX_BLOCKS * 8; }
+
+extern "C" int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes,
+                             void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    SP_REQUIRE_PTR(workspace);
+    if (n <= 0) return fail(SP_ERR_SHAPE, "sp_reduce_sum: n must be positive");
+    if (workspace_bytes < sp_reduce_workspace_bytes())
+        return fail(SP_ERR_ARG, "sp_reduce_sum: workspace must hold %lld bytes, got %lld",
+                    (long long)sp_reduce_workspace_bytes(), (long long)workspace_bytes);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype) {
+        case 0: return run_reduce<float>(x, out, n, workspace, s);
+        case 1: return run_reduce<int>(x, out, n, workspace, s);
+        case 2: return run_reduce<unsigned long long>(x, out, n, workspace, s);
+    }
+    return fail(SP_ERR_DTYPE, "sp_reduce_sum: dtype must be 0 (f32), 1 (i32) or 2 (u64), got %d", dtype);
+}
+
+extern "C" int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int64_t c, void* stream) {
+    SP_REQUIRE_PTR(from);
+    SP_REQUIRE_PTR(to);
+    if (a <= 0 || b <= 0 || c <= 0) return fail(SP_ERR_SHAPE, "sp_transpose_inner_b32: dimensions must be positive");
+    if (from == to) return fail(SP_ERR_ARG, "sp_transpose_inner_b32: in-place transpose is not supported");
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    const long tiles_b = (b + 63) / 64, tiles_c = (c + 63) / 64;
+    const long blocks = a * tiles_b * tiles_c;
+    if (blocks > 0x7fffffffL) return fail(SP_ERR_SHAPE, "sp_transpose_inner_b32: too many tiles");
+    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, (hipStream_t)stream,
+                       (const unsigned*)from, (unsigned*)to, (long)b, (long)c, tiles_b, tiles_c);
+    return check_launch(__func__);
+}

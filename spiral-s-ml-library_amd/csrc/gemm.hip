@@ -1,0 +1,396 @@
+// C = alpha * A . B^T + beta * C [+ bias] [ReLU] for gfx950 (CDNA4) with MFMA.
+//
+// A (M,K) and B (N,K) are both K-contiguous, so neither operand needs a transposing read: a
+// 32x32 MFMA fragment of either one is "32 rows x one 16-byte K-chunk per lane".
+//
+// Data movement per workgroup and K-tile (128 bytes of K per row: 64 bf16/f16 or 32 f32):
+//   global --16-byte loads--> registers --ds_write_b128--> LDS (double buffered, XOR-swizzled
+//   16-byte chunks) --ds_read_b128--> MFMA operands.  One barrier per K-tile; the global loads
+//   of tile k+1 are in flight while tile k is multiplied.
+//
+// Semantics follow matmul_tf32_template (ml/matmul/kernel.spi:25-240) with a_trans=false,
+// b_trans=true; the f32 path multiplies in full f32 (v_mfma_f32_32x32x2_f32), not TF32.
+#include "common.h"
+
+namespace sp {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
+struct GemmArgs {
+    const void* A;
+    const void* B;
+    void* C;
+    const float* bias;
+    long M, N, K;
+    float alpha, beta;
+    int relu;
+    int out_dtype;
+    int tiles_m, tiles_n;
+};
+
+constexpr int ROW_BYTES = 128;  // bytes of K per LDS row and K-tile
+constexpr int CHUNKS = 8;       // 16-byte chunks per LDS row
+
+// 16-byte chunk `kc` of LDS row `row` lives at chunk slot kc ^ swz(row): any 8 consecutive rows
+// read at the same kc touch 8 different slots, and rows r, r+8 land in different 128-byte halves.
+__device__ __forceinline__ int lds_offset(int row, int kc) {
+    return row * ROW_BYTES + (((kc ^ row ^ (row >> 3)) & 7) << 4);
+}
+
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float x) {
+    unsigned u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return (unsigned short)(u >> 16);
+}
+
+// Map the linear workgroup id to an output tile.  Workgroups are dealt round-robin to the 8 XCDs
+// (each with a private L2), so id % 8 selects the XCD; each XCD gets a contiguous range of the
+// tile sequence, and the sequence walks the tile grid in column-major groups of GROUP_M tile rows
+// so that an XCD's concurrent tiles share A and B panels.
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int XCDS = 8;
+    constexpr int GROUP_M = 4;
+    const int n = tiles_m * tiles_n;
+    const int xcd = pid % XCDS;
+    const int idx = pid / XCDS;
+    const int base = n / XCDS, rem = n % XCDS;
+    const int t = xcd * base + (xcd < rem ? xcd : rem) + idx;
+    const int group_size = GROUP_M * tiles_n;
+    const int g = t / group_size;
+    const int first_m = g * GROUP_M;
+    const int gsz = (tiles_m - first_m) < GROUP_M ? (tiles_m - first_m) : GROUP_M;
+    const int in_group = t % group_size;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <int I>
+__device__ __forceinline__ void load_rows(u32x4 (&r)[I], const unsigned char* src, long row_step) {
+#pragma unroll
+    for (int i = 0; i < I; ++i) r[i] = *reinterpret_cast<const u32x4*>(src + i * row_step);
+}
+
+template <int I, int ROW_STRIDE>
+__device__ __forceinline__ void store_rows(const u32x4 (&r)[I], unsigned char* tile, int row, int kc) {
+#pragma unroll
+    for (int i = 0; i < I; ++i) *reinterpret_cast<u32x4*>(tile + lds_offset(row + i * ROW_STRIDE, kc)) = r[i];
+}
+
+template <int DT, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int ES = (DT == SP_F32) ? 4 : 2;          // element size
+    constexpr int BK = ROW_BYTES / ES;                   // elements of K per tile
+    constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile
+    constexpr int TM = WTM / 32, TN = WTN / 32;          // 32x32 fragments per wave
+    constexpr int IA = BM * CHUNKS / NT, IB = BN * CHUNKS / NT;
+    static_assert(BM * CHUNKS % NT == 0 && BN * CHUNKS % NT == 0, "tile must be a multiple of the loader footprint");
+    static_assert(TM >= 1 && TN >= 1, "wave tile too small");
+    constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    int tm, tn;
+    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+    const long m0 = (long)tm * BM, n0 = (long)tn * BN;
+    const long K = g.K;
+
+    // ---- loader: thread -> (row, chunk) of the A and B tiles ----
+    const int ld_row = tid >> 3, ld_kc = tid & 7;
+    const unsigned char* a_src = (const unsigned char*)g.A + ((m0 + ld_row) * K) * ES + ld_kc * 16;
+    const unsigned char* b_src = (const unsigned char*)g.B + ((n0 + ld_row) * K) * ES + ld_kc * 16;
+    const long row_step = (long)(NT / 8) * K * ES;  // bytes between a thread's consecutive rows
+    u32x4 ra[IA], rb[IB];
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int frag_row = lane & 31, frag_half = lane >> 5;
+
+    auto compute = [&](int stage) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const int kc = 2 * ks + frag_half;
+            u32x4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int row = wm * WTM + i * 32 + frag_row;  // swizzle uses the tile-relative row
+                fa[i] = *reinterpret_cast<const u32x4*>(lds + stage * STAGE_BYTES + lds_offset(row, kc));
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int row = wn * WTN + j * 32 + frag_row;
+                fb[j] = *reinterpret_cast<const u32x4*>(lds + stage * STAGE_BYTES + BM * ROW_BYTES +
+                                                        lds_offset(row, kc));
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j) {
+                    if constexpr (DT == SP_BF16) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(bf16x8, fa[i]), __builtin_bit_cast(bf16x8, fb[j]), acc[i][j], 0, 0, 0);
+                    } else if constexpr (DT == SP_F16) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                            __builtin_bit_cast(f16x8, fa[i]), __builtin_bit_cast(f16x8, fb[j]), acc[i][j], 0, 0, 0);
+                    } else {
+                        // the chunk holds 4 consecutive k for this half-wave; A and B use the same
+                        // k for the same (half, step), which is all the MFMA needs
+                        const f32x4 pa = __builtin_bit_cast(f32x4, fa[i]);
+                        const f32x4 pb = __builtin_bit_cast(f32x4, fb[j]);
+#pragma unroll
+                        for (int s = 0; s < 4; ++s)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[s], pb[s], acc[i][j], 0, 0, 0);
+                    }
+                }
+        }
+    };
+
+    const int nk = (int)(K / BK);
+    load_rows<IA>(ra, a_src, row_step);
+    load_rows<IB>(rb, b_src, row_step);
+    store_rows<IA, NT / 8>(ra, lds, ld_row, ld_kc);
+    store_rows<IB, NT / 8>(rb, lds + BM * ROW_BYTES, ld_row, ld_kc);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const bool more = kt + 1 < nk;
+        if (more) {
+            a_src += ROW_BYTES;
+            b_src += ROW_BYTES;
+            load_rows<IA>(ra, a_src, row_step);
+            load_rows<IB>(rb, b_src, row_step);
+        }
+        compute(kt & 1);
+        if (more) {
+            unsigned char* st = lds + ((kt + 1) & 1) * STAGE_BYTES;
+            store_rows<IA, NT / 8>(ra, st, ld_row, ld_kc);
+            store_rows<IB, NT / 8>(rb, st + BM * ROW_BYTES, ld_row, ld_kc);
+        }
+        __syncthreads();
+    }
+
+    // ---- epilogue: D fragment layout of the 32x32 MFMA: register r of lane l holds
+    //      row 8*(r/4) + 4*(l/32) + r%4, column l%32 ----
+    const float alpha = g.alpha, beta = g.beta;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const long col = n0 + wn * WTN + j * 32 + frag_row;
+            const float bias = g.bias ? g.bias[col] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const long row = m0 + wm * WTM + i * 32 + (r >> 2) * 8 + frag_half * 4 + (r & 3);
+                const long idx = row * g.N + col;
+                float v = alpha * acc[i][j][r];
+                if (g.out_dtype == SP_F32) {
+                    float* c = (float*)g.C;
+                    if (beta != 0.f) v += beta * c[idx];
+                    v += bias;
+                    if (g.relu) v = fmaxf(v, 0.f);
+                    c[idx] = v;
+                } else if (g.out_dtype == SP_BF16) {
+                    unsigned short* c = (unsigned short*)g.C;
+                    if (beta != 0.f) v += beta * __uint_as_float((unsigned)c[idx] << 16);
+                    v += bias;
+                    if (g.relu) v = fmaxf(v, 0.f);
+                    c[idx] = f32_to_bf16_rne(v);
+                } else {
+                    _Float16* c = (_Float16*)g.C;
+                    if (beta != 0.f) v += beta * (float)c[idx];
+                    v += bias;
+                    if (g.relu) v = fmaxf(v, 0.f);
+                    c[idx] = (_Float16)v;
+                }
+            }
+        }
+}
+
+// Shape-agnostic kernel: one thread per output element, 16-byte loads along K.  Used for shapes
+// the tiled kernels do not divide (the MLP's K = 32 or N = 3 for instance).
+template <int DT>
+__global__ __launch_bounds__(256) void gemm_abt_generic_kernel(const GemmArgs g) {
+    constexpr int ES = (DT == SP_F32) ? 4 : 2;
+    constexpr int PER = 16 / ES;
+    const long n = (long)blockIdx.x * 16 + (threadIdx.x & 15);
+    const long m = (long)blockIdx.y * 16 + (threadIdx.x >> 4);
+    if (m >= g.M || n >= g.N) return;
+    const unsigned char* a = (const unsigned char*)g.A + m * g.K * ES;
+    const unsigned char* b = (const unsigned char*)g.B + n * g.K * ES;
+    float s = 0.f;
+    for (long k = 0; k < g.K; k += PER) {
+        const u32x4 va = *reinterpret_cast<const u32x4*>(a + k * ES);
+        const u32x4 vb = *reinterpret_cast<const u32x4*>(b + k * ES);
+        if constexpr (DT == SP_F32) {
+            const float* fa = reinterpret_cast<const float*>(&va);
+            const float* fb = reinterpret_cast<const float*>(&vb);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s += fa[i] * fb[i];
+        } else if constexpr (DT == SP_F16) {
+            const _Float16* fa = reinterpret_cast<const _Float16*>(&va);
+            const _Float16* fb = reinterpret_cast<const _Float16*>(&vb);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += (float)fa[i] * (float)fb[i];
+        } else {
+            const unsigned short* fa = reinterpret_cast<const unsigned short*>(&va);
+            const unsigned short* fb = reinterpret_cast<const unsigned short*>(&vb);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                s += __uint_as_float((unsigned)fa[i] << 16) * __uint_as_float((unsigned)fb[i] << 16);
+        }
+    }
+    const long idx = m * g.N + n;
+    float v = g.alpha * s;
+    const float bias = g.bias ? g.bias[n] : 0.f;
+    if (g.out_dtype == SP_F32) {
+        float* c = (float*)g.C;
+        if (g.beta != 0.f) v += g.beta * c[idx];
+        v += bias;
+        if (g.relu) v = fmaxf(v, 0.f);
+        c[idx] = v;
+    } else if (g.out_dtype == SP_BF16) {
+        unsigned short* c = (unsigned short*)g.C;
+        if (g.beta != 0.f) v += g.beta * __uint_as_float((unsigned)c[idx] << 16);
+        v += bias;
+        if (g.relu) v = fmaxf(v, 0.f);
+        c[idx] = f32_to_bf16_rne(v);
+    } else {
+        _Float16* c = (_Float16*)g.C;
+        if (g.beta != 0.f) v += g.beta * (float)c[idx];
+        v += bias;
+        if (g.relu) v = fmaxf(v, 0.f);
+        c[idx] = (_Float16)v;
+    }
+}
+
+// ---- host side: tile choice and launch -------------------------------------------------------
+
+struct TileCfg {
+    int bm, bn, wm, wn;
+};
+static const TileCfg kTileCfgs[] = {{256, 256, 2, 4}, {128, 128, 2, 2}, {64, 64, 2, 2}};
+constexpr int kNumCfgs = 3;
+
+// Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.
+static int choose_cfg(int dtype_in, long M, long N, long K) {
+    const int bk = dtype_in == SP_F32 ? 32 : 64;
+    if (K % bk != 0) return -1;
+    const int cus = device_cu_count();
+    int smallest = -1;
+    for (int i = 0; i < kNumCfgs; ++i) {
+        const TileCfg& c = kTileCfgs[i];
+        if (M % c.bm != 0 || N % c.bn != 0) continue;
+        smallest = i;
+        const long tiles = (M / c.bm) * (N / c.bn);
+        if (tiles * 5 >= (long)cus * 4) return i;
+    }
+    return smallest;
+}
+
+template <int DT, int BM, int BN, int WM, int WN>
+static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
+    auto kernel = gemm_abt_kernel<DT, BM, BN, WM, WN>;
+    const int lds_bytes = 2 * (BM + BN) * ROW_BYTES;
+    static bool attr_set[64] = {false};
+    int dev = 0;
+    hipGetDevice(&dev);
+    if (!attr_set[dev & 63]) {
+        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes,
+                                         hipGetErrorString(e));
+        attr_set[dev & 63] = true;
+    }
+    const long tiles = (long)g.tiles_m * g.tiles_n;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(WM * WN * 64), lds_bytes, stream, g);
+    return check_launch("sp_gemm_abt");
+}
+
+template <int DT>
+static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
+    switch (cfg) {
+        case 0: return launch_tiled<DT, 256, 256, 2, 4>(g, stream);
+        case 1: return launch_tiled<DT, 128, 128, 2, 2>(g, stream);
+        case 2: return launch_tiled<DT, 64, 64, 2, 2>(g, stream);
+    }
+    dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16));
+    hipLaunchKernelGGL(gemm_abt_generic_kernel<DT>, grid, dim3(256), 0, stream, g);
+    return check_launch("sp_gemm_abt(generic)");
+}
+
+static int validate_gemm(int dtype_in, int dtype_out, int64_t M, int64_t N, int64_t K) {
+    if (dtype_in != SP_F32 && dtype_in != SP_F16 && dtype_in != SP_BF16)
+        return fail(SP_ERR_DTYPE, "sp_gemm_abt: unknown input dtype %d", dtype_in);
+    if (dtype_out != SP_F32 && dtype_out != dtype_in)
+        return fail(SP_ERR_DTYPE, "sp_gemm_abt: output dtype must be f32 or the input dtype (in %d, out %d)", dtype_in,
+                    dtype_out);
+    if (M <= 0 || N <= 0 || K <= 0)
+        return fail(SP_ERR_SHAPE, "sp_gemm_abt: M, N, K must be positive (got %lld, %lld, %lld)", (long long)M,
+                    (long long)N, (long long)K);
+    const int per = dtype_in == SP_F32 ? 4 : 8;
+    if (K % per != 0)
+        return fail(SP_ERR_SHAPE, "sp_gemm_abt: K must be a multiple of %d (16-byte rows), got %lld", per, (long long)K);
+    if (M > (1ll << 31) || N > (1ll << 31) || K > (1ll << 31)) return fail(SP_ERR_SHAPE, "sp_gemm_abt: dimension too large");
+    return SP_OK;
+}
+
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_gemm_config(int dtype_in, int64_t M, int64_t N, int64_t K, int32_t* tile_m, int32_t* tile_n,
+                              int32_t* tile_k, int32_t* threads) {
+    if (!tile_m || !tile_n || !tile_k || !threads) return fail(SP_ERR_NULL, "sp_gemm_config: NULL output");
+    int rc = validate_gemm(dtype_in, SP_F32, M, N, K);
+    if (rc != SP_OK) return rc;
+    const int cfg = choose_cfg(dtype_in, M, N, K);
+    if (cfg < 0) {
+        *tile_m = 0; *tile_n = 0; *tile_k = 0; *threads = 256;
+    } else {
+        *tile_m = kTileCfgs[cfg].bm; *tile_n = kTileCfgs[cfg].bn; *tile_k = dtype_in == SP_F32 ? 32 : 64;
+        *threads = kTileCfgs[cfg].wm * kTileCfgs[cfg].wn * 64;
+    }
+    return SP_OK;
+}
+
+extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
+                           int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream) {
+    SP_REQUIRE_PTR(A);
+    SP_REQUIRE_PTR(B);
+    SP_REQUIRE_PTR(C);
+    SP_OPTIONAL_PTR(bias);
+    int rc = validate_gemm(dtype_in, dtype_out, M, N, K);
+    if (rc != SP_OK) return rc;
+    if (alpha == 0.f) return fail(SP_ERR_ARG, "sp_gemm_abt: The alpha must not be zero.");
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    int cfg = (flags & SP_GEMM_FORCE_GENERIC) ? -1 : choose_cfg(dtype_in, M, N, K);
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
+    g.relu = (flags & SP_GEMM_RELU) ? 1 : 0;
+    g.out_dtype = dtype_out;
+    if (cfg >= 0) {
+        g.tiles_m = (int)(M / kTileCfgs[cfg].bm);
+        g.tiles_n = (int)(N / kTileCfgs[cfg].bn);
+    }
+    hipStream_t s = (hipStream_t)stream;
+    switch (dtype_in) {
+        case SP_F32: return launch_dtype<SP_F32>(cfg, g, s);
+        case SP_F16: return launch_dtype<SP_F16>(cfg, g, s);
+        default: return launch_dtype<SP_BF16>(cfg, g, s);
+    }
+}

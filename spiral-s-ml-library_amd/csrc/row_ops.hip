@@ -1,0 +1,465 @@
+// Row primitives for gfx950: one group of T lanes (T = cols/4 rounded up to a power of two, at
+// most one wave64) owns a row and keeps it in registers, 4 contiguous columns per lane and chunk,
+// so every fused pipeline is a single pass over HBM: one 16-byte load per lane and chunk, shuffles
+// for the cross-lane reductions/scans, 16-byte stores.  Bandwidth-bound; no LDS, no MFMA.
+//
+// Semantics follow ml/primitives.spi (row_ :423-512, local_* :295-348 and :701-814).
+#include "common.h"
+
+// The scan/sampling results are compared bit for bit with a CPU restatement, so no operation in
+// this file may be fused or re-associated.
+#pragma clang fp contract(off)
+
+namespace sp {
+
+constexpr int ROW_THREADS = 256;
+constexpr int INT_MAX_ = 2147483647;
+
+struct RowArgs {
+    const float* x;
+    const float* u;        // per-row uniforms, or nullptr -> philox (if sample requested)
+    float* rowmax;
+    float* rowsum;
+    float* out;            // mapped output (probabilities / op result)
+    float* cdf;
+    float* u_out;
+    int* argmax;
+    int* sample;
+    long rows;
+    int cols;
+    int op;                // sp_row_op
+    int mask_size;         // columns j < mask_size are valid for the masked ops
+    int want_stats;        // rowmax/rowsum are of softmax(x) regardless of op (fused pipeline)
+    // philox
+    unsigned long long seed;
+    int philox_mode;       // -1: none
+    int tpb;
+    int blocks;
+};
+
+// Philox4x32-10 (Salmon et al., SC'11) with cuRAND's counter layout: key = seed, counter =
+// (group, 0, subsequence_lo, subsequence_hi); returns the first word of the group, mapped to (0, 1]
+// like curand_uniform (corecuda/random.spi:22-32,84).
+__device__ __forceinline__ float philox_uniform_x(unsigned long long seed, unsigned long long subsequence,
+                                                  unsigned long long group) {
+    unsigned c0 = (unsigned)group, c1 = (unsigned)(group >> 32), c2 = (unsigned)subsequence,
+             c3 = (unsigned)(subsequence >> 32);
+    unsigned k0 = (unsigned)seed, k1 = (unsigned)(seed >> 32);
+#pragma unroll
+    for (int r = 0; r < 10; ++r) {
+        if (r) {
+            k0 += 0x9E3779B9u;
+            k1 += 0xBB67AE85u;
+        }
+        unsigned hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+        unsigned hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+        unsigned n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
+        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    }
+    return (float)c0 * 2.3283064e-10f + 1.1641532e-10f;
+}
+
+// Which (subsequence, 4-word group) the reference's sampling op uses for row r: every thread of
+// the row draws once per element it holds and the draw attached to column 0 wins
+// (ml/primitives.spi:786-791), i.e. the first draw of the row's lane 0 in that row-iteration.
+__device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r) {
+    const long t = a.cols / 4;            // threads per row in the reference
+    const long per_iter = a.tpb / t;      // rows per block-iteration
+    unsigned long long sub, group;
+    if (a.philox_mode == SP_PHILOX_BLOCK) {
+        sub = (r % per_iter) * t;
+        group = r / per_iter;
+    } else if (a.philox_mode == SP_PHILOX_GRID) {
+        const long it = r / per_iter;
+        sub = (it % a.blocks) * a.tpb + (r % per_iter) * t;
+        group = it / a.blocks;
+    } else {  // SP_PHILOX_GATHER: row r belongs to thread r
+        const long lt = r % a.tpb;
+        sub = (r / a.tpb) * a.tpb + (lt % per_iter) * t;
+        group = lt / per_iter;
+    }
+    return philox_uniform_x(a.seed, sub, group);
+}
+
+__device__ __forceinline__ float sum4(const float (&v)[4]) { return ((v[0] + v[1]) + v[2]) + v[3]; }
+
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
+    constexpr int ROWS_PER_WAVE = WAVE / T;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int l = lane % T;          // lane inside the row group
+    const int sub = lane / T;        // which of the wave's rows
+    const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
+    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    const float NEG_INF = -__builtin_inff();
+    const int cols = a.cols;
+    const bool masked = (a.op == SP_ROW_MASKED_SOFTMAX || a.op == SP_ROW_MASKED_REGRET_MATCHING);
+    const int limit = masked ? a.mask_size : cols;
+
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += n_waves * ROWS_PER_WAVE) {
+        const long row = row0 + sub;
+        const bool row_ok = row < a.rows;
+        const float* xr = a.x + row * (long)cols;
+
+        float v[C][4];
+        bool ok[C];
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int col = c * 4 * T + 4 * l;
+            ok[c] = row_ok && col < cols;
+            if (ok[c]) {
+                const float4 t4 = *reinterpret_cast<const float4*>(xr + col);
+                v[c][0] = t4.x; v[c][1] = t4.y; v[c][2] = t4.z; v[c][3] = t4.w;
+            } else {
+                v[c][0] = v[c][1] = v[c][2] = v[c][3] = 0.f;
+            }
+        }
+
+        // ---- argmax (and the row max of the raw input): lowest index among equal maxima ----
+        float bv = NEG_INF;
+        int bi = INT_MAX_;
+        if (a.argmax != nullptr || a.rowmax != nullptr || a.want_stats) {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int j = c * 4 * T + 4 * l + k;
+                    if (ok[c] && (bi == INT_MAX_ || v[c][k] > bv)) { bv = v[c][k]; bi = j; }
+                }
+#pragma unroll
+            for (int d = 1; d < T; d <<= 1) {
+                const float ov = __shfl_xor(bv, d, WAVE);
+                const int oi = __shfl_xor(bi, d, WAVE);
+                if (oi != INT_MAX_ && (bi == INT_MAX_ || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
+            }
+        }
+
+        // ---- the row map ----
+        float p[C][4];
+        float stat_sum = 0.f;
+        const int op = a.op;
+        if (op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX) {
+            float m = NEG_INF;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int j = c * 4 * T + 4 * l + k;
+                    const float xv = (ok[c] && j < limit) ? v[c][k] : NEG_INF;
+                    p[c][k] = xv;
+                    m = fmaxf(m, xv);
+                }
+            m = group_allreduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = (p[c][k] == NEG_INF) ? 0.f : expf(p[c][k] - m);
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
+            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+            stat_sum = s;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] / s;
+        } else if (op == SP_ROW_REGRET_MATCHING || op == SP_ROW_MASKED_REGRET_MATCHING) {
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int j = c * 4 * T + 4 * l + k;
+                    p[c][k] = (ok[c] && j < limit) ? fmaxf(v[c][k], 0.f) : 0.f;
+                }
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
+            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+            const float inv_len = 1.f / (float)limit;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int j = c * 4 * T + 4 * l + k;
+                    p[c][k] = (j < limit) ? (s != 0.f ? p[c][k] / s : inv_len) : 0.f;
+                }
+        } else if (op == SP_ROW_LN_L2) {
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                float q[4];
+#pragma unroll
+                for (int k = 0; k < 4; ++k) q[k] = v[c][k] * v[c][k];
+                s = (c == 0) ? sum4(q) : s + sum4(q);
+            }
+            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = (s != 0.f) ? v[c][k] / s : 0.f;
+        } else {  // identity and the scans act on the raw input
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = v[c][k];
+        }
+
+        // ---- prefix sums of p (needed by the scans and by sampling) ----
+        const bool want_sample = a.sample != nullptr;
+        const bool is_scan = (op == SP_ROW_INCLUSIVE_SCAN || op == SP_ROW_EXCLUSIVE_SCAN);
+        float cdf[C][4];
+        if (want_sample || a.cdf != nullptr || is_scan) {
+            float carry = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float s = sum4(p[c]);
+                const float incl = group_inclusive_scan<T>(s, l);
+                float prev = __shfl_up(incl, 1, T);
+                if (l == 0) prev = 0.f;
+                float run = carry + prev;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    if (op == SP_ROW_EXCLUSIVE_SCAN) {
+                        cdf[c][k] = run;
+                        run = run + p[c][k];
+                    } else {
+                        run = run + p[c][k];
+                        cdf[c][k] = run;
+                    }
+                }
+                if (C > 1) carry = carry + __shfl(incl, T - 1, T);
+            }
+        }
+
+        // ---- inverse-CDF sampling (local_discrete_sampling, ml/primitives.spi:782-798) ----
+        int pick = INT_MAX_;
+        float uu = 0.f;
+        if (want_sample) {
+            float m = NEG_INF;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (p[c][k] > 0.f) m = fmaxf(m, cdf[c][k]);
+            m = group_allreduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
+            if (row_ok) uu = (a.u != nullptr) ? a.u[row] : reference_row_uniform(a, row);
+            const float thr = uu * m;
+#pragma unroll
+            for (int c = C - 1; c >= 0; --c)
+#pragma unroll
+                for (int k = 3; k >= 0; --k)
+                    if (p[c][k] > 0.f && cdf[c][k] >= thr) pick = c * 4 * T + 4 * l + k;
+            pick = group_allreduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
+        }
+
+        // ---- stores ----
+        float* out_ptr = is_scan ? nullptr : a.out;
+        float* cdf_ptr = is_scan ? a.out : a.cdf;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int col = c * 4 * T + 4 * l;
+            if (ok[c]) {
+                if (out_ptr != nullptr)
+                    *reinterpret_cast<float4*>(out_ptr + row * (long)cols + col) =
+                        make_float4(p[c][0], p[c][1], p[c][2], p[c][3]);
+                if (cdf_ptr != nullptr)
+                    *reinterpret_cast<float4*>(cdf_ptr + row * (long)cols + col) =
+                        make_float4(cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]);
+            }
+        }
+        if (row_ok && l == 0) {
+            if (a.rowmax != nullptr) a.rowmax[row] = bv;
+            if (a.rowsum != nullptr) a.rowsum[row] = stat_sum;
+            if (a.argmax != nullptr) a.argmax[row] = bi;
+            if (a.sample != nullptr) a.sample[row] = pick;
+            if (a.u_out != nullptr) a.u_out[row] = uu;
+        }
+    }
+}
+
+// Integer rows: identity and exact scans (two's complement wrap-around).
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) void row_kernel_i32(const int* __restrict__ x, int* __restrict__ out,
+                                                              long rows, int cols, int op) {
+    constexpr int ROWS_PER_WAVE = WAVE / T;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int l = lane % T;
+    const int sub = lane / T;
+    const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
+    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < rows; row0 += n_waves * ROWS_PER_WAVE) {
+        const long row = row0 + sub;
+        const bool row_ok = row < rows;
+        int carry = 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int col = c * 4 * T + 4 * l;
+            const bool ok = row_ok && col < cols;
+            int4 v = make_int4(0, 0, 0, 0);
+            if (ok) v = *reinterpret_cast<const int4*>(x + row * (long)cols + col);
+            const int s = ((v.x + v.y) + v.z) + v.w;
+            const int incl = group_inclusive_scan<T>(s, l);
+            int prev = __shfl_up(incl, 1, T);
+            if (l == 0) prev = 0;
+            const int start = carry + prev;
+            int4 r;
+            if (op == SP_ROW_EXCLUSIVE_SCAN) {
+                r.x = start; r.y = r.x + v.x; r.z = r.y + v.y; r.w = r.z + v.z;
+            } else if (op == SP_ROW_INCLUSIVE_SCAN) {
+                r.x = start + v.x; r.y = r.x + v.y; r.z = r.y + v.z; r.w = r.z + v.w;
+            } else {
+                r = v;
+            }
+            if (ok) *reinterpret_cast<int4*>(out + row * (long)cols + col) = r;
+            if (C > 1) carry = carry + __shfl(incl, T - 1, T);
+        }
+    }
+}
+
+static int lanes_per_row(long cols) {
+    int t = 1;
+    while (t * 4 < cols && t < 64) t *= 2;
+    return t;
+}
+
+static int row_grid(long rows, int t) {
+    const long rows_per_block = (long)(WAVE / t) * (ROW_THREADS / WAVE);
+    long blocks = (rows + rows_per_block - 1) / rows_per_block;
+    const long cap = (long)device_cu_count() * 8;  // 8 workgroups of 4 waves = 8 waves per SIMD
+    if (blocks > cap) blocks = cap;
+    return (int)(blocks < 1 ? 1 : blocks);
+}
+
+template <typename F>
+static int dispatch_tc(int t, int c, F&& f) {
+    switch (t) {
+        case 1: f(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 2: f(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 4: f(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 8: f(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 16: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 32: f(std::integral_constant<int, 32>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 64:
+            switch (c) {
+                case 1: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 1>{}); return SP_OK;
+                case 2: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 2>{}); return SP_OK;
+                case 3: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 3>{}); return SP_OK;
+                case 4: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 4>{}); return SP_OK;
+            }
+    }
+    return fail(SP_ERR_SHAPE, "row kernels: unsupported lanes/chunks %d/%d", t, c);
+}
+
+static int check_rows_cols(const char* fn, int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return fail(SP_ERR_SHAPE, "%s: rows and cols must be positive (got %lld, %lld)", fn,
+                                            (long long)rows, (long long)cols);
+    if (cols % 4 != 0) return fail(SP_ERR_SHAPE, "%s: cols must be a multiple of 4 (16-byte rows), got %lld", fn,
+                                   (long long)cols);
+    if (cols > 1024) return fail(SP_ERR_SHAPE, "%s: cols must be <= 1024, got %lld", fn, (long long)cols);
+    if (rows > (int64_t)1 << 40) return fail(SP_ERR_SHAPE, "%s: rows too large", fn);
+    return SP_OK;
+}
+
+static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
+    int rc = require_gfx950(fn);
+    if (rc != SP_OK) return rc;
+    const int t = lanes_per_row(a.cols);
+    const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
+    const int grid = row_grid(a.rows, t);
+    rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
+        hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
+                           stream, a);
+    });
+    if (rc != SP_OK) return rc;
+    return check_launch(fn);
+}
+
+}  // namespace sp
+
+using namespace sp;
+
+extern "C" int sp_row_ops(const float* logits, const float* u, float* rowmax, float* rowsum, float* probs, float* cdf,
+                          int32_t* argmax, int32_t* sample, int64_t rows, int64_t cols, uint32_t flags, void* stream) {
+    (void)flags;
+    SP_REQUIRE_PTR(logits);
+    SP_OPTIONAL_PTR(rowmax); SP_OPTIONAL_PTR(rowsum); SP_OPTIONAL_PTR(probs); SP_OPTIONAL_PTR(cdf);
+    SP_OPTIONAL_PTR(argmax); SP_OPTIONAL_PTR(sample); SP_OPTIONAL_PTR(u);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (sample != nullptr && u == nullptr) return fail(SP_ERR_NULL, "sp_row_ops: sample requested but u is NULL");
+    RowArgs a{};
+    a.x = logits; a.u = u; a.rowmax = rowmax; a.rowsum = rowsum; a.out = probs; a.cdf = cdf; a.argmax = argmax;
+    a.sample = sample; a.rows = rows; a.cols = (int)cols; a.op = SP_ROW_SOFTMAX; a.mask_size = (int)cols;
+    a.want_stats = 1; a.philox_mode = -1;
+    return launch_row(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, int64_t cols, int32_t mask_size,
+                              void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (op < SP_ROW_IDENTITY || op > SP_ROW_EXCLUSIVE_SCAN) return fail(SP_ERR_ARG, "sp_row_map_f32: unknown op %d", op);
+    const bool masked = (op == SP_ROW_MASKED_SOFTMAX || op == SP_ROW_MASKED_REGRET_MATCHING);
+    if (masked && (mask_size < 1 || mask_size > cols))
+        return fail(SP_ERR_ARG, "sp_row_map_f32: mask_size must be in [1, cols], got %d", mask_size);
+    RowArgs a{};
+    a.x = x; a.out = out; a.rows = rows; a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols;
+    a.philox_mode = -1;
+    return launch_row(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* philox, float* probs_out,
+                             float* cdf_out, float* u_out, int32_t* sample_out, int64_t rows, int64_t cols,
+                             int32_t mask_size, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(sample_out);
+    SP_OPTIONAL_PTR(u); SP_OPTIONAL_PTR(probs_out); SP_OPTIONAL_PTR(cdf_out); SP_OPTIONAL_PTR(u_out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (!(op == SP_ROW_IDENTITY || op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX ||
+          op == SP_ROW_REGRET_MATCHING || op == SP_ROW_MASKED_REGRET_MATCHING))
+        return fail(SP_ERR_ARG, "sp_row_sample: op %d cannot feed a sampler", op);
+    const bool masked = (op == SP_ROW_MASKED_SOFTMAX || op == SP_ROW_MASKED_REGRET_MATCHING);
+    if (masked && (mask_size < 1 || mask_size > cols))
+        return fail(SP_ERR_ARG, "sp_row_sample: mask_size must be in [1, cols], got %d", mask_size);
+    if ((u == nullptr) == (philox == nullptr))
+        return fail(SP_ERR_ARG, "sp_row_sample: exactly one of u and philox must be given");
+    RowArgs a{};
+    a.x = x; a.u = u; a.out = probs_out; a.cdf = cdf_out; a.u_out = u_out; a.sample = sample_out; a.rows = rows;
+    a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols; a.philox_mode = -1;
+    if (philox != nullptr) {
+        if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_GATHER)
+            return fail(SP_ERR_ARG, "sp_row_sample: unknown philox mode %d", philox->mode);
+        const int64_t t = cols / 4;
+        if (philox->threads_per_block <= 0 || philox->threads_per_block % t != 0)
+            return fail(SP_ERR_ARG, "sp_row_sample: threads_per_block (%d) must be a positive multiple of cols/4 (%lld)",
+                        philox->threads_per_block, (long long)t);
+        if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
+            return fail(SP_ERR_ARG, "sp_row_sample: blocks_per_grid must be positive");
+        a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
+        a.blocks = philox->blocks_per_grid;
+    }
+    return launch_row(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_row_map_i32(int op, const int32_t* x, int32_t* out, int64_t rows, int64_t cols, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (!(op == SP_ROW_IDENTITY || op == SP_ROW_INCLUSIVE_SCAN || op == SP_ROW_EXCLUSIVE_SCAN))
+        return fail(SP_ERR_ARG, "sp_row_map_i32: op %d is not an integer op", op);
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    const int t = lanes_per_row(cols);
+    const int c = (int)((cols + 4 * t - 1) / (4 * t));
+    const int grid = row_grid(rows, t);
+    rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
+        hipLaunchKernelGGL((row_kernel_i32<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
+                           (hipStream_t)stream, x, out, (long)rows, (int)cols, op);
+    });
+    if (rc != SP_OK) return rc;
+    return check_launch(__func__);
+}

@@ -1,0 +1,114 @@
+"""ctypes binding of libspiral_mi355.so (declared in include/spiral_mi355.h)."""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(_HERE), "libspiral_mi355.so")
+
+SP_F32, SP_F16, SP_BF16 = 0, 1, 2
+GEMM_RELU, GEMM_FORCE_GENERIC = 0x1, 0x100
+(ROW_IDENTITY, ROW_SOFTMAX, ROW_MASKED_SOFTMAX, ROW_LN_L2, ROW_REGRET_MATCHING, ROW_MASKED_REGRET_MATCHING,
+ ROW_INCLUSIVE_SCAN, ROW_EXCLUSIVE_SCAN) = range(8)
+PHILOX_BLOCK, PHILOX_GRID, PHILOX_GATHER = 0, 1, 2
+MAP_COPY, MAP_RELU, MAP_TANH, MAP_SIGMOID = 0, 1, 2, 3
+HEAD_NONE, HEAD_SOFTMAX, HEAD_REGRET_MATCHING, HEAD_SOFTMAX_RM = 0, 1, 2, 3
+
+ERROR_NAMES = {0: "SP_OK", -1: "SP_ERR_NULL", -2: "SP_ERR_SHAPE", -3: "SP_ERR_ALIGN", -4: "SP_ERR_DTYPE",
+               -5: "SP_ERR_ARG", -6: "SP_ERR_UNSUPPORTED", -7: "SP_ERR_DEVICE"}
+
+
+class SpiralError(RuntimeError):
+    """A C-ABI call returned a negative sp_status."""
+
+    def __init__(self, code, message):
+        super().__init__("%s (%d): %s" % (ERROR_NAMES.get(code, "?"), code, message))
+        self.code = code
+
+
+class PhiloxConfig(C.Structure):
+    _fields_ = [("seed", C.c_uint64), ("mode", C.c_int32), ("threads_per_block", C.c_int32),
+                ("blocks_per_grid", C.c_int32), ("reserved", C.c_int32)]
+
+
+class DeviceInfo(C.Structure):
+    _fields_ = [("name", C.c_char * 128), ("arch", C.c_char * 64), ("compute_units", C.c_int32),
+                ("wavefront_size", C.c_int32), ("lds_bytes_per_cu", C.c_int32), ("max_clock_khz", C.c_int32),
+                ("hbm_bytes", C.c_int64), ("l2_bytes", C.c_int32)]
+
+
+class KernelInfo(C.Structure):
+    _fields_ = [("vgprs", C.c_int32), ("sgprs", C.c_int32), ("static_lds_bytes", C.c_int32),
+                ("threads_per_block", C.c_int32), ("max_blocks_per_cu", C.c_int32)]
+
+
+_P, _I64, _I32, _U32, _F = C.c_void_p, C.c_int64, C.c_int32, C.c_uint32, C.c_float
+
+SIGNATURES = {
+    "sp_last_error_string": (C.c_char_p, []),
+    "sp_device_info": (C.c_int, [C.POINTER(DeviceInfo)]),
+    "sp_kernel_info": (C.c_int, [C.c_char_p, C.POINTER(KernelInfo)]),
+    "sp_gemm_abt": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, _P, _I64, _I64, _I64, _F, _F, _U32, _P]),
+    "sp_gemm_config": (C.c_int, [C.c_int, _I64, _I64, _I64] + [C.POINTER(C.c_int32)] * 4),
+    "sp_row_ops": (C.c_int, [_P] * 8 + [_I64, _I64, _U32, _P]),
+    "sp_row_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_row_map_i32": (C.c_int, [C.c_int, _P, _P, _I64, _I64, _P]),
+    "sp_row_sample": (C.c_int, [C.c_int, _P, _P, C.POINTER(PhiloxConfig), _P, _P, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
+    "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),
+    "sp_reduce_workspace_bytes": (C.c_int64, []),
+    "sp_transpose_inner_b32": (C.c_int, [_P, _P, _I64, _I64, _I64, _P]),
+    "sp_mlp_forward": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
+                                 _I64, _I32, _I32, _P]),
+}
+
+
+def load(path=LIB_PATH):
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: build it with `python spiral-s-ml-library_amd/build.py` "
+                           "(there is no CPU fallback)" % path)
+    lib = C.CDLL(path)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+lib = load()
+
+
+def check(rc):
+    if rc != 0:
+        raise SpiralError(rc, lib.sp_last_error_string().decode())
+
+
+def stream_ptr():
+    """torch's current HIP stream as a hipStream_t."""
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+DTYPES = {torch.float32: SP_F32, torch.float16: SP_F16, torch.bfloat16: SP_BF16}
+
+
+def ptr(t, dtype=None, name="tensor"):
+    """Device pointer of a contiguous ROCm tensor (None passes through as NULL)."""
+    if t is None:
+        return None
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor" % name)
+    if not t.is_cuda:
+        raise ValueError("%s must live on the GPU (got %s)" % (name, t.device))
+    if not t.is_contiguous():
+        raise ValueError("%s must be contiguous (row-major, innermost stride 1)" % name)
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError("%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    return C.c_void_p(t.data_ptr())
+
+
+def device_info():
+    info = DeviceInfo()
+    check(lib.sp_device_info(C.byref(info)))
+    return {f: (getattr(info, f).decode() if isinstance(getattr(info, f), bytes) else getattr(info, f))
+            for f, _ in DeviceInfo._fields_}

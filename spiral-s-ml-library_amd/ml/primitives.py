@@ -1,0 +1,288 @@
+"""Host surface of the row primitives (reference: ml/primitives.spi, generated ml/primitives.py).
+
+The reference exposes `row_map`, `row_reduce` and `row_map_reduce` that run a user lambda built
+from `local_*` pieces on each row (ml/primitives.spi:514-536).  A HIP library cannot take a
+lambda, so every lambda the reference's tests and layers use is a named function here with the
+same meaning; each one is a single fused kernel launch (libspiral_mi355.so, sp_row_*).
+`main()` / `main_body()` keep the meaning of the generated module: run tests 2-6 and write the
+tensors in the golden text format under test_text_outputs/primitives/.
+"""
+import ctypes as C
+import os
+
+import torch
+
+from . import _console, _lib
+from ._lib import PhiloxConfig, check, lib, ptr, stream_ptr
+
+CONSTANT_SEED = 12344321            # corecuda/cupy.spi:6
+THREADS_PER_BLOCK = 256             # corecuda/base.spi:14-42
+BLOCKS_PER_GRID = 24
+
+
+def _rows_cols(x):
+    if x.dim() < 2:
+        raise ValueError("expected a tensor with at least 2 dimensions")
+    cols = x.shape[-1]
+    return x.numel() // cols, cols
+
+
+def _row_map(op, x, out=None, mask_size=0):
+    rows, cols = _rows_cols(x)
+    if out is None:
+        out = torch.empty_like(x)
+    if x.dtype == torch.float32:
+        check(lib.sp_row_map_f32(op, ptr(x, name="x"), ptr(out, torch.float32, "out"), rows, cols, mask_size,
+                                 stream_ptr()))
+    elif x.dtype == torch.int32:
+        check(lib.sp_row_map_i32(op, ptr(x, name="x"), ptr(out, torch.int32, "out"), rows, cols, stream_ptr()))
+    else:
+        raise TypeError("row primitives take f32 or i32 tensors, got %s" % x.dtype)
+    return out
+
+
+def identity(x, out=None):
+    """row_map (fun config x i j_tns => x) (ml/primitives.spi:929)."""
+    return _row_map(_lib.ROW_IDENTITY, x, out)
+
+
+def softmax(x, out=None):
+    """row_map local_softmax (ml/primitives.spi:711-716, test2 :934)."""
+    return _row_map(_lib.ROW_SOFTMAX, x, out)
+
+
+def masked_softmax(x, size, out=None):
+    """row_map (local_masked_softmax (j < size)) (ml/primitives.spi:748-759)."""
+    return _row_map(_lib.ROW_MASKED_SOFTMAX, x, out, size)
+
+
+def ln_l2(x, out=None):
+    """row_map local_ln_l2 (ml/primitives.spi:701-703)."""
+    return _row_map(_lib.ROW_LN_L2, x, out)
+
+
+def regret_matching(x, out=None):
+    """row_map local_regret_matching (ml/primitives.spi:718-722)."""
+    return _row_map(_lib.ROW_REGRET_MATCHING, x, out)
+
+
+def masked_regret_matching(x, size, out=None):
+    """row_map (local_masked_regret_matching (j < size)) (ml/primitives.spi:761-780)."""
+    return _row_map(_lib.ROW_MASKED_REGRET_MATCHING, x, out, size)
+
+
+def inclusive_scan_sum(x, out=None):
+    """row_map local_inclusive_scan_sum (ml/primitives.spi:323-325); f32 or i32."""
+    return _row_map(_lib.ROW_INCLUSIVE_SCAN, x, out)
+
+
+def exclusive_scan_sum(x, out=None):
+    """row_map (local_exclusive_scan config 0 (+)) (ml/primitives.spi:327, test2 :948-950)."""
+    return _row_map(_lib.ROW_EXCLUSIVE_SCAN, x, out)
+
+
+def row_ops(logits, u=None, want=("rowmax", "rowsum", "probs", "cdf", "argmax", "sample")):
+    """The fused pipeline of one pass over the logits: row max, sum of exp(x - max), softmax,
+    inclusive prefix sum, argmax and inverse-CDF sampling (sp_row_ops).  Returns a dict with the
+    requested outputs."""
+    rows, cols = _rows_cols(logits)
+    lead = logits.shape[:-1]
+    dev = logits.device
+    out = {}
+    for name in want:
+        if name in ("probs", "cdf"):
+            out[name] = torch.empty_like(logits)
+        elif name in ("rowmax", "rowsum"):
+            out[name] = torch.empty(lead, dtype=torch.float32, device=dev)
+        elif name in ("argmax", "sample"):
+            out[name] = torch.empty(lead, dtype=torch.int32, device=dev)
+        else:
+            raise ValueError("unknown output %r" % name)
+    check(lib.sp_row_ops(ptr(logits, torch.float32, "logits"), ptr(u, torch.float32, "u"), ptr(out.get("rowmax")),
+                         ptr(out.get("rowsum")), ptr(out.get("probs")), ptr(out.get("cdf")), ptr(out.get("argmax")),
+                         ptr(out.get("sample")), rows, cols, 0, stream_ptr()))
+    return out
+
+
+def argmax(x):
+    """row_reduce local_argmax (ml/primitives.spi:705-708, test2 :940); ties -> lowest index."""
+    return row_ops(x, want=("argmax",))["argmax"]
+
+
+def philox(mode=_lib.PHILOX_BLOCK, seed=CONSTANT_SEED, threads_per_block=THREADS_PER_BLOCK,
+           blocks_per_grid=BLOCKS_PER_GRID):
+    """The reference's device RNG: Philox4_32_10 seeded like `random.init {seed subsequence offset=0}`
+    (ml/primitives.spi:927,1014; corecuda/random.spi:22-32)."""
+    return PhiloxConfig(seed, mode, threads_per_block, blocks_per_grid, 0)
+
+
+def _sample(op, x, u=None, rng=None, mask_size=0, want_cdf=False, want_u=False):
+    rows, cols = _rows_cols(x)
+    probs = torch.empty_like(x)
+    sample = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device)
+    cdf = torch.empty_like(x) if want_cdf else None
+    u_out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if want_u else None
+    if (u is None) == (rng is None):
+        raise ValueError("give exactly one of u (a tensor of uniforms in (0, 1]) and rng (a PhiloxConfig)")
+    check(lib.sp_row_sample(op, ptr(x, torch.float32, "x"), ptr(u, torch.float32, "u"),
+                            C.byref(rng) if rng is not None else None, ptr(probs), ptr(cdf), ptr(u_out), ptr(sample),
+                            rows, cols, mask_size, stream_ptr()))
+    res = (probs, sample)
+    if want_cdf:
+        res += (cdf,)
+    if want_u:
+        res += (u_out,)
+    return res
+
+
+def discrete_sampling(p, u=None, rng=None, **kw):
+    """row_reduce local_discrete_sampling (ml/primitives.spi:782-798)."""
+    return _sample(_lib.ROW_IDENTITY, p, u, rng, **kw)
+
+
+def softmax_and_discrete_sampling(x, u=None, rng=None, **kw):
+    """row_map_reduce local_softmax_and_discrete_sampling (ml/primitives.spi:800-802)."""
+    return _sample(_lib.ROW_SOFTMAX, x, u, rng, **kw)
+
+
+def masked_softmax_and_discrete_sampling(x, size, u=None, rng=None, **kw):
+    """row_map_reduce local_masked_softmax_and_discrete_sampling (ml/primitives.spi:804-806)."""
+    return _sample(_lib.ROW_MASKED_SOFTMAX, x, u, rng, mask_size=size, **kw)
+
+
+def regret_matching_and_discrete_sampling(x, u=None, rng=None, **kw):
+    """row_map_reduce local_regret_matching_and_discrete_sampling (ml/primitives.spi:808-810)."""
+    return _sample(_lib.ROW_REGRET_MATCHING, x, u, rng, **kw)
+
+
+def masked_regret_matching_and_discrete_sampling(x, size, u=None, rng=None, **kw):
+    """row_map_reduce local_masked_regret_matching_and_discrete_sampling (ml/primitives.spi:812-814)."""
+    return _sample(_lib.ROW_MASKED_REGRET_MATCHING, x, u, rng, mask_size=size, **kw)
+
+
+def map(op, x, out=None):  # noqa: A001  (the reference's name, ml/primitives.spi:128)
+    """primitives.map f from to for f in {"copy", "relu", "tanh", "sigmoid"} (ml/layers.spi:353-355)."""
+    code = {"copy": _lib.MAP_COPY, "relu": _lib.MAP_RELU, "tanh": _lib.MAP_TANH, "sigmoid": _lib.MAP_SIGMOID}[op]
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib.sp_map_f32(code, ptr(x, torch.float32, "x"), ptr(out, torch.float32, "out"), x.numel(), stream_ptr()))
+    return out
+
+
+_workspace = {}
+
+
+def reduce_sum(x):
+    """reduce 0 (+) / grid_reduce grid 0 (+) over a whole tensor (ml/primitives.spi:176-197).
+    f32, i32 or u64 (carried as int64 by torch).  Returns a 0-d tensor on the device."""
+    code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
+    key = x.device.index
+    if key not in _workspace:
+        _workspace[key] = torch.empty(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=x.device)
+    ws = _workspace[key]
+    out = torch.empty(4, dtype=x.dtype, device=x.device)  # 16-byte aligned scalar slot
+    check(lib.sp_reduce_sum(code, ptr(x, name="x"), ptr(out), x.numel(), ptr(ws), ws.numel(), stream_ptr()))
+    return out[0]
+
+
+def transpose_snd(x, out=None):
+    """grid_transpose_snd from to: swap the two innermost dimensions (ml/primitives.spi:107-109)."""
+    if x.element_size() != 4 or x.dim() < 2:
+        raise TypeError("transpose_snd takes tensors of 4-byte elements with >= 2 dimensions")
+    b, c = x.shape[-2], x.shape[-1]
+    a = x.numel() // (b * c)
+    if out is None:
+        out = torch.empty(x.shape[:-2] + (c, b), dtype=x.dtype, device=x.device)
+    check(lib.sp_transpose_inner_b32(ptr(x, name="x"), ptr(out, name="out"), a, b, c, stream_ptr()))
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# self-tests in the reference's format
+# ----------------------------------------------------------------------------------------------
+
+def _dump(root, head_dir, name, limit, *tensors):
+    d = os.path.join(root, head_dir)
+    os.makedirs(d, exist_ok=True)
+    _console.write_ln(os.path.join(d, name), limit, *[t.cpu().numpy() for t in tensors])
+
+
+def _row_test(root, m, n, head_dir, grid, seed=CONSTANT_SEED):
+    """ml/primitives.spi test2 (:904-988, block level) and test4 (:992-1076, grid level).  They differ
+    in which Philox subsequence a row uses and in test2 overwriting output_softmax'.txt."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    ident = torch.arange(m * n, dtype=torch.int32, device="cuda").reshape(m, n)
+    x = torch.randn((m, n), generator=gen, device="cuda", dtype=torch.float32)
+    rng = philox(_lib.PHILOX_GRID if grid else _lib.PHILOX_BLOCK)
+    ii = torch.arange(m, dtype=torch.int32, device="cuda")[:, None].expand(m, n)
+    jj = torch.arange(n, dtype=torch.int32, device="cuda")[None, :].expand(m, n)
+    sm = softmax(x)
+    probs1, sample1 = softmax_and_discrete_sampling(x, rng=rng)
+    probs2, sample2 = masked_softmax_and_discrete_sampling(x, 11, rng=rng)
+    if not grid:
+        _dump(root, head_dir, "output_reduce.txt", 1024, reduce_sum(x))
+    _dump(root, head_dir, "input.txt", 1024, x)
+    _dump(root, head_dir, "input_identity.txt", 1024, ident)
+    _dump(root, head_dir, "output_softmax.txt", 1024, sm)
+    _dump(root, head_dir, "output_masked_softmax.txt", 1024, masked_softmax(x, 4))
+    _dump(root, head_dir, "output_ln.txt", 1024, ln_l2(x))
+    _dump(root, head_dir, "output_argmax.txt", 1024, argmax(x))
+    _dump(root, head_dir, "output_softmax_scan.txt", m * n, sm, inclusive_scan_sum(sm))
+    _dump(root, head_dir, "output_identity.txt", m * n, identity(ident))
+    _dump(root, head_dir, "output_indices_map.txt", m * n, ii, jj)
+    _dump(root, head_dir, "output_indices_reduction.txt", m * n, ii[:, 0])
+    _dump(root, head_dir, "output_sum_exclusive.txt", m * n, exclusive_scan_sum(ident))
+    _dump(root, head_dir, "output_softmax'.txt", 1024, probs1)
+    _dump(root, head_dir, "output_sampling.txt", 1024, sample1)
+    _dump(root, head_dir, "output_softmax'.txt" if not grid else "output_softmax''.txt", 1024, probs2)
+    _dump(root, head_dir, "output_sampling'.txt", 1024, sample2)
+
+
+def test2(m, n, head_dir, root="test_text_outputs/primitives/"):
+    _row_test(root, m, n, head_dir, grid=False)
+
+
+def test4(m, n, head_dir, root="test_text_outputs/primitives/"):
+    _row_test(root, m, n, head_dir, grid=True)
+
+
+def test5(l, m, n, head_dir, root="test_text_outputs/primitives/"):
+    """ml/primitives.spi test5 (:1078-1088): transpose of arange(l, m, n)."""
+    x = torch.arange(l * m * n, dtype=torch.int32, device="cuda").reshape(l, m, n)
+    y = transpose_snd(x)
+    d = os.path.join(root, head_dir)
+    os.makedirs(d, exist_ok=True)
+    with open(os.path.join(d, "transpose.txt"), "w") as f:
+        f.write(_console.format_tensor(2 ** 31 - 1, x.cpu().numpy()) + "\n")
+        f.write(_console.format_tensor(2 ** 31 - 1, y.cpu().numpy()) + "\n")
+
+
+def test6(m, n, head_dir, root="test_text_outputs/primitives/"):
+    """ml/primitives.spi test6 (:1090-1110): u64 sum of arange(m * n), block and grid variants."""
+    x = torch.arange(m * n, dtype=torch.int64, device="cuda").reshape(m, n)
+    r = reduce_sum(x)
+    _dump(root, head_dir, "input_identity.txt", 1024, x)
+    _dump(root, head_dir, "output_reduce_block.txt", 1024, r)
+    _dump(root, head_dir, "output_reduce_grid.txt", 1024, r)
+
+
+def main_body(root="test_text_outputs/primitives/"):
+    """ml/primitives.spi main (:1112-1137).  test3 (row_gather_*) is not part of this build."""
+    test2(1 << 6, 1 << 7, "test2/a/", root)
+    test2(1 << 7, 1 << 6, "test2/b/", root)
+    test4(1 << 7, 1 << 6, "test4/b/", root)
+    test4(1 << 6, 1 << 7, "test4/a/", root)
+    test5(2, 4, 8, "test5/a", root)
+    test5(2, 128, 256, "test5/b", root)
+    test6(128, 128, "test6/a", root)
+
+
+def main():
+    main_body()
+    torch.cuda.current_stream().synchronize()
+    print("Done.")
+
+
+if __name__ == "__main__":
+    main()

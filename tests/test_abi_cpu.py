@@ -1,0 +1,110 @@
+"""CPU-side checks of the C-ABI boundary: the shared library loads, exports every symbol the
+header declares, and rejects every host-checkable bad argument with an error code before any
+device work (so these run without a GPU)."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "spiral_mi355.h")
+
+
+@pytest.fixture(scope="module")
+def L():
+    from ml import _lib
+    return _lib
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sp_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_exported(L):
+    names = declared_functions()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(L.lib, n), "libspiral_mi355.so does not export %s" % n
+        assert n in L.SIGNATURES, "ml/_lib.py has no ctypes signature for %s" % n
+
+
+def test_missing_library_fails_loudly(L, tmp_path):
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        L.load(str(tmp_path / "libspiral_mi355.so"))
+
+
+def _err(L):
+    return L.lib.sp_last_error_string().decode()
+
+
+def test_gemm_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x1000)
+    args = lambda **kw: [kw.get("din", 2), kw.get("dout", 0), kw.get("A", p), kw.get("B", p), kw.get("C", p),
+                         kw.get("bias", None), kw.get("M", 64), kw.get("N", 64), kw.get("K", 64),
+                         kw.get("alpha", 1.0), 0.0, 0, None]
+    assert lib.sp_gemm_abt(*args(A=None)) == -1 and "A is NULL" in _err(L)
+    assert lib.sp_gemm_abt(*args(B=C.c_void_p(0x1004))) == -3 and "16-byte" in _err(L)
+    assert lib.sp_gemm_abt(*args(M=0)) == -2
+    assert lib.sp_gemm_abt(*args(K=60)) == -2 and "multiple of 8" in _err(L)
+    assert lib.sp_gemm_abt(*args(din=0, K=6)) == -2 and "multiple of 4" in _err(L)
+    assert lib.sp_gemm_abt(*args(din=7)) == -4
+    assert lib.sp_gemm_abt(*args(din=1, dout=2)) == -4
+    assert lib.sp_gemm_abt(*args(alpha=0.0)) == -5 and "alpha must not be zero" in _err(L)
+
+
+def test_row_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x2000)
+    assert lib.sp_row_ops(None, None, None, None, None, None, None, None, 8, 8, 0, None) == -1
+    assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 8, 6, 0, None) == -2
+    assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 8, 2048, 0, None) == -2
+    assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 0, 8, 0, None) == -2
+    assert lib.sp_row_ops(p, None, None, None, None, None, None, p, 8, 8, 0, None) == -1  # sample without u
+    assert lib.sp_row_ops(p, None, None, None, C.c_void_p(0x2008), None, None, None, 8, 8, 0, None) == -3
+    assert lib.sp_row_map_f32(99, p, p, 8, 8, 0, None) == -5
+    assert lib.sp_row_map_f32(L.ROW_MASKED_SOFTMAX, p, p, 8, 8, 0, None) == -5
+    assert lib.sp_row_map_f32(L.ROW_MASKED_SOFTMAX, p, p, 8, 8, 9, None) == -5
+    assert lib.sp_row_map_i32(L.ROW_SOFTMAX, p, p, 8, 8, None) == -5
+    ph = L.PhiloxConfig(1, 0, 256, 24, 0)
+    assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, None, None, None, None, p, 8, 8, 0, None) == -5
+    assert lib.sp_row_sample(L.ROW_SOFTMAX, p, p, C.byref(ph), None, None, None, p, 8, 8, 0, None) == -5
+    assert lib.sp_row_sample(L.ROW_LN_L2, p, p, None, None, None, None, p, 8, 8, 0, None) == -5
+    bad = L.PhiloxConfig(1, 0, 100, 24, 0)  # 100 threads is not a multiple of cols/4 = 16
+    assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, C.byref(bad), None, None, None, p, 8, 64, 0, None) == -5
+
+
+def test_misc_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x3000)
+    assert lib.sp_map_f32(0, p, p, 6, None) == -2
+    assert lib.sp_map_f32(0, None, p, 8, None) == -1
+    assert lib.sp_reduce_sum(0, p, p, 8, p, 16, None) == -5
+    assert lib.sp_reduce_workspace_bytes() >= 1024
+    assert lib.sp_transpose_inner_b32(p, p, 1, 8, 8, None) == -5
+    assert lib.sp_transpose_inner_b32(p, C.c_void_p(0x4000), 0, 8, 8, None) == -2
+    assert lib.sp_device_info(None) == -1
+
+
+def test_mlp_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x5000)
+    w = (C.c_void_p * 2)(p, p)
+    dims = lambda *d: (C.c_int32 * len(d))(*d)
+    call = lambda dtype=1, x=p, n=2, ws=w, d=dims(32, 64, 3), u=None, pol=p, act=None, batch=8, head=3, mask=0: \
+        lib.sp_mlp_forward(dtype, x, n, ws, None, d, u, pol, act, None, batch, head, mask, None)
+    assert call(dtype=0) == -4
+    assert call(x=None) == -1
+    assert call(n=0) == -5 and call(n=9) == -5
+    assert call(d=dims(30, 64, 3)) == -2
+    assert call(d=dims(32, 48, 3)) == -2
+    assert call(d=dims(32, 512, 3)) == -2
+    assert call(d=dims(32, 64, 128)) == -2
+    assert call(batch=0) == -2
+    assert call(head=7) == -5
+    assert call(mask=4) == -5
+    assert call(act=p) == -1  # action without u
+    assert call(ws=(C.c_void_p * 2)(p, None)) == -1

@@ -1,0 +1,185 @@
+"""GEMM C = alpha A.B^T + beta C on the GPU (through the C ABI) against the NumPy oracle.
+Bar (relative Frobenius error): <= 1e-5 for f32, <= 3e-3 for f16/bf16 inputs evaluated on the
+rounded inputs; exactly representable integer problems are bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f32": 1e-5, "f16": 3e-3, "bf16": 3e-3}
+TORCH = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+@pytest.fixture(scope="module")
+def MM():
+    from ml import matmul
+    return matmul
+
+
+def make(rng, m, n, k, dtype, scale=None):
+    scale = (1.0 / np.sqrt(k)) if scale is None else scale
+    a = ogemm.round_to(rng.standard_normal((m, k), dtype=np.float32) * np.float32(scale), dtype)
+    b = ogemm.round_to(rng.standard_normal((n, k), dtype=np.float32) * np.float32(scale), dtype)
+    return a, b
+
+
+def run(MM, a, b, dtype, **kw):
+    return host(MM.matmul_abt(dev(a, TORCH[dtype]), dev(b, TORCH[dtype]), **kw))
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 128, 128), (256, 256, 192), (512, 256, 64), (192, 320, 128),
+                                   (1024, 1024, 256)])
+def test_tiled_shapes(MM, dtype, m, n, k):
+    announce("gemm tiled %s %dx%dx%d" % (dtype, m, n, k))
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a, b = make(rng, m, n, k, dtype)
+    got = run(MM, a, b, dtype)
+    assert ogemm.rel_frobenius(got, ogemm.gemm_abt(a, b)) < TOL[dtype]
+    generic = run(MM, a, b, dtype, force_generic=True)
+    assert ogemm.rel_frobenius(generic, ogemm.gemm_abt(a, b)) < TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+def test_integer_inputs_are_exact(MM, dtype):
+    """Small integers are exact in every dtype and every partial sum fits f32: any indexing slip
+    (transposed operand, wrong fragment row, dropped K-chunk) changes the integer result."""
+    announce("gemm integer exact " + dtype)
+    m, n, k = 256, 512, 320
+    a = ((np.arange(m * k).reshape(m, k) * 7 + 3) % 11 - 5).astype(np.float32)
+    b = ((np.arange(n * k).reshape(n, k) * 5 + 1) % 13 - 6).astype(np.float32)
+    want = a.astype(np.int64) @ b.astype(np.int64).T
+    assert (run(MM, a, b, dtype).astype(np.int64) == want).all()
+    assert (run(MM, a, b, dtype, force_generic=True).astype(np.int64) == want).all()
+    ident = np.eye(256, dtype=np.float32)
+    a2 = ogemm.round_to(np.random.default_rng(1).standard_normal((256, 256), dtype=np.float32), dtype)
+    assert (run(MM, a2, ident, dtype) == a2).all()       # B = I  ->  C = A (not A^T)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_alpha_beta_bias_relu(MM, dtype):
+    announce("gemm alpha/beta/bias/relu " + dtype)
+    rng = np.random.default_rng(11)
+    m, n, k = 256, 256, 128
+    a, b = make(rng, m, n, k, dtype)
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    bias = rng.standard_normal(n, dtype=np.float32)
+    for alpha, beta in ((1.0, 1.0), (0.5, -2.0), (2.0, 0.0)):
+        c = dev(c0.copy())
+        MM.matmul_abt(dev(a, TORCH[dtype]), dev(b, TORCH[dtype]), c, alpha, beta)
+        assert ogemm.rel_frobenius(host(c), ogemm.gemm_abt(a, b, c0, alpha, beta)) < TOL[dtype]
+    # beta == 0 never reads C: NaNs must not propagate (ml/matmul/kernel.spi:152-154)
+    c = torch.full((m, n), float("nan"), device="cuda")
+    MM.matmul_abt(dev(a, TORCH[dtype]), dev(b, TORCH[dtype]), c, 1.0, 0.0)
+    assert np.isfinite(host(c)).all()
+    got = run(MM, a, b, dtype, bias=dev(bias), relu=True)
+    want = ogemm.gemm_abt(a, b, bias=bias, relu=True)
+    assert ogemm.rel_frobenius(got, want) < TOL[dtype]
+    assert (got >= 0).all() and ((got == 0) == (want == 0)).mean() > 0.999
+    with pytest.raises(AssertionError, match="alpha must not be zero"):
+        MM.matmul_abt(dev(a, TORCH[dtype]), dev(b, TORCH[dtype]), alpha=0.0)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_sixteen_bit_output(MM, dtype):
+    announce("gemm 16-bit output " + dtype)
+    rng = np.random.default_rng(12)
+    a, b = make(rng, 512, 512, 256, dtype)
+    got = run(MM, a, b, dtype, out_dtype=TORCH[dtype])
+    want = ogemm.gemm_abt(a, b, out_dtype=dtype)
+    assert ogemm.rel_frobenius(got, want) < TOL[dtype]
+    # rounding of the f32 accumulator is RNE: at most one ulp away from the rounded oracle,
+    # and equal nearly everywhere
+    assert (got == want).mean() > 0.98
+
+
+def test_generic_shapes(MM):
+    announce("gemm generic shapes")
+    rng = np.random.default_rng(13)
+    for dtype, (m, n, k) in (("f32", (16, 16, 8)), ("f32", (33, 7, 12)), ("f16", (100, 3, 256)), ("bf16", (5, 65, 40))):
+        a, b = make(rng, m, n, k, dtype)
+        assert ogemm.rel_frobenius(run(MM, a, b, dtype), ogemm.gemm_abt(a, b)) < TOL[dtype]
+    a, b = make(rng, 16, 16, 8, "f32")
+    assert ogemm.rel_frobenius(run(MM, a, b, "f32"), ogemm.gemm_abt_bruteforce(a, b)) < 1e-6
+
+
+def test_reference_call_signature(MM):
+    """matmul_tf32 a_trans b_trans alpha a b beta c with all four layouts (ml/matmul/run.spi:25)."""
+    announce("gemm matmul_tf32 layouts")
+    rng = np.random.default_rng(14)
+    m, n, k = 128, 192, 64
+    a = rng.standard_normal((m, k), dtype=np.float32)
+    b = rng.standard_normal((n, k), dtype=np.float32)
+    c0 = rng.standard_normal((m, n), dtype=np.float32)
+    want = ogemm.gemm_abt(a, b, c0, 1.0, 1.0)
+    for a_trans in (False, True):
+        for b_trans in (False, True):
+            am = dev(a.T.copy() if a_trans else a)
+            bm = dev(b if b_trans else b.T.copy())
+            c = dev(c0.copy())
+            MM.matmul_tf32(a_trans, b_trans, 1.0, am, bm, 1.0, c)
+            assert ogemm.rel_frobenius(host(c), want) < TOL["f32"]
+    cfg = MM.matmul_config_tf32(False, True, 8192, 8192, 4096)
+    assert cfg["m_tile"] > 0 and 8192 % cfg["m_tile"] == 0 and 4096 % cfg["k_tile"] == 0
+
+
+def test_config1_fp32_1024(MM):
+    announce("gemm config 1: f32 1024^3")
+    rng = np.random.default_rng(1)
+    a = rng.standard_normal((1024, 1024), dtype=np.float32)
+    b = rng.standard_normal((1024, 1024), dtype=np.float32)
+    got = run(MM, a, b, "f32")
+    assert ogemm.rel_frobenius(got, ogemm.gemm_abt(a, b)) < TOL["f32"]
+    want64 = ogemm.gemm_abt(a, b, acc=np.float64)
+    assert ogemm.rel_frobenius(got, want64) < TOL["f32"]
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_config2_4096(MM, dtype):
+    announce("gemm config 2: 4096^3 " + dtype)
+    rng = np.random.default_rng(2)
+    a, b = make(rng, 4096, 4096, 4096, dtype)
+    want = ogemm.gemm_abt(a, b)
+    assert ogemm.rel_frobenius(run(MM, a, b, dtype), want) < TOL[dtype]
+    got16 = run(MM, a, b, dtype, out_dtype=TORCH[dtype])
+    assert ogemm.rel_frobenius(got16, ogemm.round_to(want, dtype)) < TOL[dtype]
+
+
+def test_config2_8192_sampled_rows(MM):
+    """8192^3 in bf16: the oracle is evaluated on 192 sampled rows of C (a full CPU product is
+    ~1.1 TFLOP); linearity is checked on the whole output: (2A).B^T == 2 (A.B^T) exactly."""
+    announce("gemm config 2: 8192^3 bf16 (sampled rows)")
+    rng = np.random.default_rng(3)
+    n = 8192
+    a, b = make(rng, n, n, n, "bf16")
+    ad, bd = dev(a, torch.bfloat16), dev(b, torch.bfloat16)
+    c = MM.matmul_abt(ad, bd)
+    rows = rng.choice(n, 192, replace=False)
+    assert ogemm.rel_frobenius(host(c[torch.from_numpy(rows).cuda()]), ogemm.gemm_abt(a[rows], b)) < TOL["bf16"]
+    c2 = MM.matmul_abt(ad * 2, bd)
+    assert torch.equal(c2, c * 2)
+
+
+@pytest.mark.parametrize("k,n", [(256, 256), (512, 1024), (2048, 256)])
+def test_config4_tall_skinny(MM, k, n):
+    announce("gemm config 4: 65536 x %d x %d bf16" % (n, k))
+    rng = np.random.default_rng(4 + k)
+    m = 65536
+    a, b = make(rng, m, n, k, "bf16")
+    bias = rng.standard_normal(n, dtype=np.float32)
+    got = run(MM, a, b, "bf16")
+    assert ogemm.rel_frobenius(got, ogemm.gemm_abt(a, b)) < TOL["bf16"]
+    got = run(MM, a, b, "bf16", bias=dev(bias), relu=True)
+    assert ogemm.rel_frobenius(got, ogemm.gemm_abt(a, b, bias=bias, relu=True)) < TOL["bf16"]
+
+
+def test_reference_self_test(MM):
+    """ml/matmul/run.spi main: max |C - (A.B^T + C0)| on a smaller instance of the same recipe."""
+    announce("gemm reference self-test 1024x1024x512")
+    diff = float(MM.main_body(1024, 1024, 512))
+    torch.cuda.synchronize()
+    assert diff < 1e-3

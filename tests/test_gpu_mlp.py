@@ -1,0 +1,98 @@
+"""Fused dense-stack forward on the GPU (through the C ABI) against the NumPy oracle.
+Bar: policy within a relative Frobenius error of 3e-3 of the f32 oracle evaluated on the rounded
+inputs; sampled actions bit-exact given the kernel's own policy and the same uniforms."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm, layers as olayers, row_ops as orow
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+
+TORCH = {"f16": torch.float16, "bf16": torch.bfloat16}
+HEAD_CODE = {"softmax": olayers.HEAD_SOFTMAX, "regret_matching": olayers.HEAD_REGRET_MATCHING,
+             "softmax_regret_matching": olayers.HEAD_SOFTMAX_RM, None: olayers.HEAD_NONE}
+
+
+@pytest.fixture(scope="module")
+def LY():
+    from ml import layers
+    return layers
+
+
+def make_problem(rng, batch, dims, dtype):
+    x = (rng.random((batch, dims[0])) < 0.2).astype(np.float32)
+    ws = [ogemm.round_to(olayers.weight_init(rng, o, i), dtype) for i, o in zip(dims[:-1], dims[1:])]
+    u = (1 - rng.random(batch, dtype=np.float32)).astype(np.float32)
+    return x, ws, u
+
+
+def check(LY, x, ws, u, dtype, head="softmax_regret_matching", mask=0, biases=None):
+    t = TORCH[dtype]
+    bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
+    policy, action, logits = LY.mlp_forward(dev(x, t), [dev(w, t) for w in ws], bd, head, dev(u), mask, True)
+    policy, action, logits = host(policy), host(action), host(logits)
+    want_p, _, want_l = olayers.mlp_forward(x, ws, biases, HEAD_CODE[head], u, None, mask or None)
+    assert ogemm.rel_frobenius(logits, want_l) < 3e-3
+    assert ogemm.rel_frobenius(policy, want_p) < 3e-3
+    # against the oracle that rounds hidden activations to the storage dtype like the kernel does:
+    # only summation order differs, which now and then flips a rounded activation by one ulp
+    tight_p, _, tight_l = olayers.mlp_forward(x, ws, biases, HEAD_CODE[head], u, dtype, mask or None)
+    assert ogemm.rel_frobenius(logits, tight_l) < 2e-4
+    assert ogemm.rel_frobenius(policy, tight_p) < 2e-4
+    # bit-exact action given the kernel's policy and the same uniforms
+    if head is not None:
+        assert (action == orow.discrete_sampling(policy, u)).all()
+        assert (np.take_along_axis(policy, action[:, None].astype(np.int64), 1) > 0).all()
+        if mask:
+            assert (action < mask).all() and (policy[:, mask:] == 0).all()
+        assert np.abs(policy.sum(axis=1) - 1).max() < 1e-5
+    return policy, action
+
+
+def test_config3_leduc_policy(LY):
+    """BASELINE config 3: batch 16384, 32 -> 256 -> 256 -> 256 -> 3, f16, softmax head, regret-matching sampling."""
+    announce("mlp config 3")
+    rng = np.random.default_rng(3)
+    x, ws, u = make_problem(rng, 16384, [32, 256, 256, 256, 3], "f16")
+    policy, action = check(LY, x, ws, u, "f16")
+    counts = np.bincount(action, minlength=3) / len(action)
+    assert np.abs(counts - policy.mean(axis=0)).max() < 0.02   # sampled frequencies follow the policy
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("batch", [1, 100, 640])
+def test_ragged_batches_and_dtypes(LY, dtype, batch):
+    announce("mlp ragged batch=%d %s" % (batch, dtype))
+    rng = np.random.default_rng(batch)
+    x, ws, u = make_problem(rng, batch, [32, 256, 256, 256, 3], dtype)
+    check(LY, x, ws, u, dtype)
+
+
+@pytest.mark.parametrize("dims,head,mask", [([128, 64, 64], "regret_matching", 3), ([64, 64, 64], "softmax", 3),
+                                            ([16, 32, 8], "softmax", 0), ([256, 256, 64], None, 0),
+                                            ([32, 96, 160, 5], "softmax_regret_matching", 0), ([48, 3], "softmax", 0)])
+def test_other_stacks(LY, dims, head, mask):
+    """Shapes of the reference's real models: Leduc input(128) -> 64 -> 64 (3 valid) with a masked
+    regret-matching head (game/leduc/model_cem.spi:47-63)."""
+    announce("mlp stack %s head=%s mask=%d" % (dims, head, mask))
+    rng = np.random.default_rng(len(dims) * 100 + dims[0])
+    x, ws, u = make_problem(rng, 300, dims, "f16")
+    if head is None:
+        t = TORCH["f16"]
+        policy, _, logits = LY.mlp_forward(dev(x, t), [dev(w, t) for w in ws], None, None, None, 0, True)
+        want = olayers.mlp_forward(x, ws, head=olayers.HEAD_NONE, act_dtype="f16")[2]
+        assert ogemm.rel_frobenius(host(policy), want) < 2e-4 and (host(policy) == host(logits)).all()
+    else:
+        check(LY, x, ws, u, "f16", head, mask)
+
+
+def test_bias_extension(LY):
+    announce("mlp biases")
+    rng = np.random.default_rng(9)
+    dims = [32, 64, 64, 3]
+    x, ws, u = make_problem(rng, 200, dims, "bf16")
+    biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
+    biases[1] = None
+    check(LY, x, ws, u, "bf16", biases=biases)

@@ -1,0 +1,184 @@
+"""Row primitives on the GPU (through the C ABI) against the reference's golden vectors and the
+NumPy oracle.  Bar: indices, integer scans and the f32 prefix sums bit-exact; other floats within
+a relative Frobenius error of 1e-5."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm, philox as ophilox, row_ops as orow
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+
+FLOAT_TOL = 1e-5          # relative Frobenius, f32 outputs
+PRINT_TOL = 1.5e-6        # golden files carry 6 decimals
+ROW_CASES = ["primitives_test2_a", "primitives_test2_b", "primitives_test4_a", "primitives_test4_b"]
+
+
+@pytest.fixture(scope="module")
+def P():
+    from ml import primitives
+    return primitives
+
+
+@pytest.mark.parametrize("case", ROW_CASES)
+def test_golden_row_maps(P, golden, case):
+    announce("golden row maps " + case)
+    g = golden(case)
+    x = dev(g["input"])
+    assert np.abs(host(P.softmax(x)) - g["output_softmax"]).max() < PRINT_TOL
+    assert np.abs(host(P.masked_softmax(x, 4)) - g["output_masked_softmax"]).max() < PRINT_TOL
+    assert np.abs(host(P.ln_l2(x)) - g["output_ln"]).max() < PRINT_TOL
+    assert (host(P.argmax(x)) == g["output_argmax"][: x.shape[0]]).all()
+    key = "output_softmax_pp" if "output_softmax_pp" in g else "output_softmax_p"
+    assert np.abs(host(P.masked_softmax(x, 11)) - g[key]).max() < PRINT_TOL
+    ident = dev(g["output_identity"].astype(np.int32))
+    assert (host(P.exclusive_scan_sum(ident)) == g["output_sum_exclusive"]).all()
+    assert (host(P.identity(ident)) == g["output_identity"]).all()
+    p = dev(g["output_softmax_scan"][..., 0].copy())
+    cdf = host(P.inclusive_scan_sum(p))
+    assert np.abs(cdf - g["output_softmax_scan"][..., 1]).max() < p.shape[1] * 5e-7 + PRINT_TOL
+
+
+@pytest.mark.parametrize("case", ROW_CASES)
+def test_golden_sampling_with_device_philox(P, golden, case):
+    """The stored sampled indices are reproduced from the stored probabilities with the uniforms
+    generated on the device exactly as the reference does (Philox4_32_10, seed 12344321)."""
+    from ml import _lib
+    announce("golden philox sampling " + case)
+    g = golden(case)
+    mode = _lib.PHILOX_BLOCK if "test2" in case else _lib.PHILOX_GRID
+    p = dev(g["output_softmax_scan"][..., 0].copy())
+    probs, sample, u = P.discrete_sampling(p, rng=P.philox(mode), want_u=True)
+    rows, cols = p.shape
+    want_u = ophilox.row_uniforms_block(rows, cols) if "test2" in case else ophilox.row_uniforms_grid(rows, cols)
+    assert (host(u) == want_u).all()
+    assert (host(probs) == host(p)).all()
+    assert (host(sample) == g["output_sampling"]).all()
+    # masked (j < 11) variant from the first rows of the input
+    x = dev(g["input"])
+    _, sample_m, u_m = P.masked_softmax_and_discrete_sampling(x, 11, rng=P.philox(mode), want_u=True)
+    assert (host(u_m) == want_u[: x.shape[0]]).all()
+    assert (host(sample_m) == g["output_sampling_p"][: x.shape[0]]).all()
+
+
+@pytest.mark.parametrize("case", ["primitives_test3_a", "primitives_test3_b"])
+def test_golden_gather_rows(P, golden, case):
+    from ml import _lib
+    announce("golden gather rows " + case)
+    g = golden(case)
+    x = dev(g["zip_input_output_identity_map"][..., 0].copy())
+    assert np.abs(host(P.masked_regret_matching(x, 3)) - g["output_op_map"]).max() < PRINT_TOL
+    _, sample = P.masked_softmax_and_discrete_sampling(x, 3, rng=P.philox(_lib.PHILOX_GATHER))
+    assert (host(sample) == g["output_sample_reduce"][: x.shape[0]]).all()
+
+
+def test_golden_reduce_and_transpose(P, golden):
+    announce("golden reduce / transpose")
+    g = golden("primitives_test6_a")
+    x = torch.arange(128 * 128, dtype=torch.int64, device="cuda")
+    assert int(P.reduce_sum(x)) == int(g["output_reduce_grid"]) == 134209536
+    xi = torch.arange(1 << 20, dtype=torch.int32, device="cuda") % 1000
+    assert int(P.reduce_sum(xi)) == int(host(xi).sum())
+    xf = dev(np.random.default_rng(0).standard_normal(1 << 20).astype(np.float32))
+    assert abs(float(P.reduce_sum(xf)) - float(host(xf).astype(np.float64).sum())) < 1e-2
+    for case in ("primitives_test5_a", "primitives_test5_b"):
+        t = golden(case)
+        assert (host(P.transpose_snd(dev(t["input"].astype(np.int32)))) == t["output"]).all()
+    y = dev(np.arange(3 * 70 * 130, dtype=np.int32).reshape(3, 70, 130))
+    assert (host(P.transpose_snd(y)) == orow.transpose_inner(host(y))).all()
+
+
+SHAPES = [(1, 4), (3, 12), (5, 16), (130, 64), (64, 128), (257, 256), (33, 260), (9, 512), (1000, 1024), (7, 1000)]
+
+
+@pytest.mark.parametrize("rows,cols", SHAPES)
+def test_row_ops_against_oracle(P, rows, cols):
+    announce("row_ops oracle rows=%d cols=%d" % (rows, cols))
+    rng = np.random.default_rng(rows * 10007 + cols)
+    x = (rng.standard_normal((rows, cols)) * 2).astype(np.float32)
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    out = {k: host(v) for k, v in P.row_ops(dev(x), dev(u)).items()}
+    assert (out["argmax"] == orow.argmax(x)).all()
+    assert (out["rowmax"] == x.max(axis=1)).all()
+    assert ogemm.rel_frobenius(out["probs"], orow.softmax(x)) < FLOAT_TOL
+    assert ogemm.rel_frobenius(out["rowsum"], orow.softmax_stats(x)[1]) < FLOAT_TOL
+    # the prefix sums and the sampled index are bit-exact given the kernel's own probabilities
+    assert (out["cdf"] == orow.inclusive_scan_sum(out["probs"], order="wave")).all()
+    assert (out["sample"] == orow.discrete_sampling(out["probs"], u, order="wave")).all()
+    assert ogemm.rel_frobenius(out["cdf"], orow.inclusive_scan_sum(orow.softmax(x))) < FLOAT_TOL
+    # sequential-order cdf: same index on all but boundary rows
+    seq = orow.discrete_sampling(out["probs"], u, order="sequential")
+    assert (seq != out["sample"]).mean() < 0.01
+
+
+@pytest.mark.parametrize("rows,cols", [(3, 12), (130, 64), (257, 256), (9, 512), (7, 1000)])
+def test_row_maps_against_oracle(P, rows, cols):
+    announce("row maps oracle rows=%d cols=%d" % (rows, cols))
+    rng = np.random.default_rng(rows * 31 + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    x[0] = -np.abs(x[0])  # a row with no positive entry: regret matching falls back to uniform
+    xd = dev(x)
+    size = max(1, cols // 3)
+    assert ogemm.rel_frobenius(host(P.softmax(xd)), orow.softmax(x)) < FLOAT_TOL
+    assert ogemm.rel_frobenius(host(P.masked_softmax(xd, size)), orow.masked_softmax(x, size)) < FLOAT_TOL
+    assert ogemm.rel_frobenius(host(P.ln_l2(xd)), orow.ln_l2(x)) < FLOAT_TOL
+    rm = host(P.regret_matching(xd))
+    assert ogemm.rel_frobenius(rm, orow.regret_matching(x)) < FLOAT_TOL
+    assert (rm[0] == np.float32(1) / np.float32(cols)).all()
+    mrm = host(P.masked_regret_matching(xd, size))
+    assert ogemm.rel_frobenius(mrm, orow.masked_regret_matching(x, size)) < FLOAT_TOL
+    assert (mrm[:, size:] == 0).all()
+    assert (host(P.inclusive_scan_sum(xd)) == orow.inclusive_scan_sum(x, order="wave")).all()
+    assert (host(P.exclusive_scan_sum(xd)) == orow.exclusive_scan(x, order="wave")).all()
+    xi = rng.integers(-2 ** 20, 2 ** 20, size=(rows, cols)).astype(np.int32)
+    assert (host(P.inclusive_scan_sum(dev(xi))) == orow.inclusive_scan_sum(xi)).all()
+    assert (host(P.exclusive_scan_sum(dev(xi))) == orow.exclusive_scan(xi)).all()
+    assert (host(P.map("relu", xd)) == orow.relu(x)).all()
+    assert np.abs(host(P.map("tanh", xd)) - np.tanh(x)).max() < 1e-6
+    assert np.abs(host(P.map("sigmoid", xd)) - 1 / (1 + np.exp(-x))).max() < 1e-6
+    # sampling heads given the same uniforms
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    for fn, args in ((P.softmax_and_discrete_sampling, ()), (P.masked_softmax_and_discrete_sampling, (size,)),
+                     (P.regret_matching_and_discrete_sampling, ()),
+                     (P.masked_regret_matching_and_discrete_sampling, (size,))):
+        probs, sample, cdf = fn(xd, *args, u=dev(u), want_cdf=True)
+        probs, sample, cdf = host(probs), host(sample), host(cdf)
+        assert (cdf == orow.inclusive_scan_sum(probs, order="wave")).all()
+        assert (sample == orow.discrete_sampling(probs, u, cdf=cdf)).all()
+        assert (np.take_along_axis(probs, sample[:, None].astype(np.int64), 1) > 0).all()
+
+
+def test_sampling_edge_cases(P):
+    announce("sampling edge cases")
+    p = np.zeros((4, 8), dtype=np.float32)
+    p[0, 3] = 1.0                      # a single atom
+    p[1, [1, 6]] = 0.5                 # zeros around the atoms
+    p[2, :] = 0.125
+    u = np.array([1.0, 1.0, 1e-30, 0.5], dtype=np.float32)
+    _, sample = P.discrete_sampling(dev(p), u=dev(u))
+    s = host(sample)
+    assert s[0] == 3 and s[1] == 6 and s[2] == 0
+    assert s[3] == 2147483647           # no p > 0: the reduction's neutral element (limit.max)
+
+
+def test_row_ops_full_size(P):
+    """BASELINE config 5: 65536 x 256 f32 logits ~ N(0, sigma=2), one uniform per row."""
+    announce("row_ops full size 65536x256")
+    rng = np.random.default_rng(5)
+    rows, cols = 65536, 256
+    x = (rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(2)).astype(np.float32)
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    out = {k: host(v) for k, v in P.row_ops(dev(x), dev(u)).items()}
+    assert (out["argmax"] == orow.argmax(x)).all()
+    assert (out["rowmax"] == x.max(axis=1)).all()
+    assert ogemm.rel_frobenius(out["probs"], orow.softmax(x)) < FLOAT_TOL
+    assert (out["cdf"] == orow.inclusive_scan_sum(out["probs"], order="wave")).all()
+    assert (out["sample"] == orow.discrete_sampling(out["probs"], u, cdf=out["cdf"])).all()
+    # size-independent properties
+    assert np.abs(out["cdf"][:, -1] - 1).max() < 1e-5
+    assert (np.diff(out["cdf"], axis=1) >= 0).all()
+    assert ((out["sample"] >= 0) & (out["sample"] < cols)).all()
+    # scalar-outputs-only mode gives the same indices
+    lean = P.row_ops(dev(x), dev(u), want=("argmax", "sample", "rowmax", "rowsum"))
+    assert (host(lean["sample"]) == out["sample"]).all() and (host(lean["argmax"]) == out["argmax"]).all()
