@@ -1,0 +1,226 @@
+#!/usr/bin/env python3
+"""Benchmark of the GEMM -> dense-layer -> row-primitive hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-extra] [--no-cpu]
+
+Headline (the JSON line's `value`): TFLOP/s of the bf16 4096^3 GEMM C = A.B^T with f32
+accumulation and f32 output, inputs resident in HBM, whole-job throughput over K launches.
+A "step" is one launch of that GEMM.  The same line carries, under "extra", the other
+configurations (f32 1024^3, f16 / 8192^3, tall-skinny value-net GEMMs, the fused Leduc MLP
+forward in rows/s, the row primitives in GB/s), each with its own roofline fraction, and under
+"cpu_baseline" the NumPy restatement timed on this box's host cores in the same run.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "spiral-s-ml-library_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks
+PEAK_HBM_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--only", default=None, help="run a single extra case by name (profiling aid)")
+    return ap.parse_args()
+
+
+def time_launches(fn, steps, warmup):
+    """W untimed + K timed launches.  Returns (wall ms per step between two full device syncs,
+    HIP-event ms per launch on the launch stream)."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()           # torch's current stream == the stream the library launches on
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3 / steps
+    return wall, start.elapsed_time(stop) / steps
+
+
+def roofline_mfma(flops, ms, dtype):
+    achieved = flops / (ms * 1e-3) / 1e12
+    return {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK_TFLOPS[dtype], "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_TFLOPS[dtype], 4), "traffic": None}
+
+
+def roofline_hbm(nbytes, ms):
+    achieved = nbytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None}
+
+
+def best_of(fn, reps):
+    fn()
+    best = float("inf")
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        best = min(best, time.perf_counter() - t0)
+    return best
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU; --gpus %d is not supported (every GPU box here has one GPU "
+              "and the path has no collective step)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from ml import layers, matmul, primitives
+    from oracle import gemm as ogemm, layers as olayers, row_ops as orow
+
+    torch.cuda.set_device(0)
+    TD = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
+    dev = lambda x, t=None: torch.from_numpy(np.ascontiguousarray(x)).cuda().to(t or torch.from_numpy(x).dtype)
+    K, W = args.steps, args.warmup
+
+    def gemm_inputs(seed, m, n, k, dtype):
+        rng = np.random.default_rng(seed)
+        scale = np.float32(1.0 / np.sqrt(k)) if dtype != "f32" else np.float32(1.0)
+        a = ogemm.round_to(rng.standard_normal((m, k), dtype=np.float32) * scale, dtype)
+        b = ogemm.round_to(rng.standard_normal((n, k), dtype=np.float32) * scale, dtype)
+        return a, b
+
+    def gemm_case(seed, m, n, k, dtype, out="f32", bias_relu=False, steps=K, warmup=W):
+        a, b = gemm_inputs(seed, m, n, k, dtype)
+        ad, bd = dev(a, TD[dtype]), dev(b, TD[dtype])
+        c = torch.empty((m, n), dtype=TD[out], device="cuda")
+        bias = dev(np.random.default_rng(seed + 1).standard_normal(n, dtype=np.float32)) if bias_relu else None
+        fn = lambda: matmul.matmul_abt(ad, bd, c, bias=bias, relu=bias_relu)
+        wall, ev = time_launches(fn, steps, warmup)
+        flops = 2.0 * m * n * k
+        es_in, es_out = (4 if dtype == "f32" else 2), (4 if out == "f32" else 2)
+        nbytes = es_in * (m * k + n * k) + es_out * m * n + (4 * n if bias_relu else 0)
+        t_mfma = flops / (PEAK_TFLOPS[dtype] * 1e12)
+        t_mem = nbytes / (PEAK_HBM_GBS * 1e9)
+        roof = roofline_mfma(flops, ev, dtype) if t_mfma >= t_mem else roofline_hbm(nbytes, ev)
+        res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "tflops": round(flops / (ev * 1e-3) / 1e12, 2),
+               "gbs": round(nbytes / (ev * 1e-3) / 1e9, 1), "roofline": roof, "seed": seed,
+               "tile": matmul.matmul_config_tf32(False, True, m, n, k, TD[dtype])}
+        return res, (a, b)
+
+    # ---------------- headline: bf16 4096^3, f32 accumulate, f32 out ----------------
+    head, (a, b) = gemm_case(2, 4096, 4096, 4096, "bf16")
+    flops = 2.0 * 4096 ** 3
+
+    cpu = None
+    if not args.no_cpu:
+        t = best_of(lambda: np.matmul(a, b.T), 3)
+        cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": len(os.sched_getaffinity(0)),
+               "kind": "port", "sample": "full 4096^3 problem, np.matmul(A32, B32.T) in f32 on the bf16-rounded "
+               "inputs (all BLAS threads), 1 warm-up + best of 3",
+               "os_cpu_count": os.cpu_count()}
+    del a, b
+
+    extra = {}
+    cases = []
+    if not args.no_extra:
+        cases = [
+            ("gemm_f32_1024", lambda: gemm_case(1, 1024, 1024, 1024, "f32")[0]),
+            ("gemm_bf16_4096_bf16out", lambda: gemm_case(2, 4096, 4096, 4096, "bf16", "bf16")[0]),
+            ("gemm_f16_4096", lambda: gemm_case(2, 4096, 4096, 4096, "f16")[0]),
+            ("gemm_bf16_8192", lambda: gemm_case(3, 8192, 8192, 8192, "bf16", steps=max(3, K // 5), warmup=2)[0]),
+            ("gemm_bf16_65536x256x256", lambda: gemm_case(4, 65536, 256, 256, "bf16")[0]),
+            ("gemm_bf16_65536x1024x512", lambda: gemm_case(5, 65536, 1024, 512, "bf16")[0]),
+            ("gemm_bf16_65536x256x2048", lambda: gemm_case(6, 65536, 256, 2048, "bf16")[0]),
+            ("gemm_bf16_65536x256x256_bias_relu", lambda: gemm_case(4, 65536, 256, 256, "bf16", bias_relu=True)[0]),
+        ]
+
+        def mlp_case():
+            rng = np.random.default_rng(7)
+            dims = [32, 256, 256, 256, 3]
+            batch = 16384
+            x = (rng.random((batch, 32)) < 0.2).astype(np.float32)
+            ws = [ogemm.round_to(olayers.weight_init(rng, o, i), "f16") for i, o in zip(dims[:-1], dims[1:])]
+            u = (1 - rng.random(batch, dtype=np.float32)).astype(np.float32)
+            xd, wd, ud = dev(x, torch.float16), [dev(w, torch.float16) for w in ws], dev(u)
+            fn = lambda: layers.mlp_forward(xd, wd, u=ud)
+            wall, ev = time_launches(fn, max(K, 200), W)
+            fl = 2.0 * batch * sum(i * o for i, o in zip(dims[:-1], dims[1:]))
+            res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
+                   "roofline": roofline_mfma(fl, ev, "f16"), "seed": 7,
+                   "timing": "mean over back-to-back launches between two HIP events"}
+            if not args.no_cpu:
+                t = best_of(lambda: olayers.mlp_forward(x, ws, u=u), 3)
+                res["cpu_rows_per_s"] = round(batch / t, 1)
+            return res
+
+        def rows_case(materialise):
+            rng = np.random.default_rng(8)
+            rows, cols = 65536, 256
+            x = (rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(2)).astype(np.float32)
+            u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+            xd, ud = dev(x), dev(u)
+            want = ("rowmax", "rowsum", "argmax", "sample") + (("probs", "cdf") if materialise else ())
+            outs = {}
+            for name in want:
+                shape = (rows, cols) if name in ("probs", "cdf") else (rows,)
+                outs[name] = torch.empty(shape, dtype=torch.int32 if name in ("argmax", "sample") else torch.float32,
+                                         device="cuda")
+            from ml._lib import check, lib, ptr, stream_ptr
+            fn = lambda: check(lib.sp_row_ops(ptr(xd), ptr(ud), ptr(outs["rowmax"]), ptr(outs["rowsum"]),
+                                              ptr(outs.get("probs")), ptr(outs.get("cdf")), ptr(outs["argmax"]),
+                                              ptr(outs["sample"]), rows, cols, 0, stream_ptr()))
+            wall, ev = time_launches(fn, K, W)
+            nbytes = rows * cols * 4 * (3 if materialise else 1) + rows * 4 * 5
+            res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(rows / (ev * 1e-3), 1),
+                   "roofline": roofline_hbm(nbytes, ev), "seed": 8, "sigma": 2.0}
+            if not args.no_cpu and materialise:
+                def cpu_rows():
+                    p = orow.softmax(x)
+                    cdf = orow.inclusive_scan_sum(p)
+                    return orow.argmax(x), orow.discrete_sampling(p, u, cdf=cdf)
+                t = best_of(cpu_rows, 2)
+                res["cpu_gbs"] = round(nbytes / t / 1e9, 2)
+            return res
+
+        cases += [("mlp_leduc_16384", mlp_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
+                  ("row_ops_65536x256_materialised", lambda: rows_case(True))]
+    for name, fn in cases:
+        if args.only and name != args.only:
+            continue
+        extra[name] = fn()
+        torch.cuda.empty_cache()
+
+    info = None
+    try:
+        from ml._lib import device_info
+        info = device_info()
+    except Exception as e:  # the device query is informational only
+        info = {"error": str(e)}
+
+    line = {
+        "metric": "GEMM TFLOP/s (% MFMA peak) at 4096^3 bf16; fused MLP fwd rows/sec",
+        "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": head["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "C = A.B^T, M=N=K=4096, A/B bf16 row-major N(0,1)/sqrt(K) (seed 2), f32 accumulate, "
+                               "f32 output", "tile": head["tile"]},
+        "roofline": head["roofline"], "cpu_baseline": cpu,
+        "mlp_rows_per_s": extra.get("mlp_leduc_16384", {}).get("rows_per_s"),
+        "extra": extra, "device": info,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
