@@ -4,9 +4,11 @@
 // 32x32 MFMA fragment of either one is "32 rows x one 16-byte K-chunk per lane".
 //
 // Data movement per workgroup and K-tile (128 bytes of K per row: 64 bf16/f16 or 32 f32):
-//   global --16-byte loads--> registers --ds_write_b128--> LDS (double buffered, XOR-swizzled
-//   16-byte chunks) --ds_read_b128--> MFMA operands.  One barrier per K-tile; the global loads
-//   of tile k+1 are in flight while tile k is multiplied.
+//   global --global_load_lds_dwordx4 (DMA, no registers)--> LDS (double buffered, XOR-swizzled
+//   16-byte chunks) --ds_read_b128--> MFMA operands.  One barrier per K-tile; the DMA of tile k+1
+//   runs while tile k is multiplied.  A wave-wide DMA instruction fills 1 KiB of LDS linearly
+//   (lane i -> byte 16*i), i.e. 8 tile rows; the swizzle is applied by choosing which global
+//   16-byte chunk each lane fetches.
 //
 // Semantics follow matmul_tf32_template (ml/matmul/kernel.spi:25-240) with a_trans=false,
 // b_trans=true; the f32 path multiplies in full f32 (v_mfma_f32_32x32x2_f32), not TF32.
@@ -69,16 +71,22 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     tn = in_group / gsz;
 }
 
-template <int I>
-__device__ __forceinline__ void load_rows(u32x4 (&r)[I], const unsigned char* src, long row_step) {
-#pragma unroll
-    for (int i = 0; i < I; ++i) r[i] = *reinterpret_cast<const u32x4*>(src + i * row_step);
+// One wave-wide DMA: every lane copies 16 bytes from global memory (uniform base + per-lane
+// 32-bit offset) to LDS byte m0 + 16 * lane.  Completion is tracked by vmcnt; the instruction is
+// issued from inline assembly so that the tile in flight does not make the compiler wait before
+// LDS reads of the tile being multiplied (it cannot tell the two buffers apart).
+__device__ __forceinline__ void dma_to_lds(const unsigned char* base, unsigned lane_offset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
+                 : "memory");
 }
 
-template <int I, int ROW_STRIDE>
-__device__ __forceinline__ void store_rows(const u32x4 (&r)[I], unsigned char* tile, int row, int kc) {
-#pragma unroll
-    for (int i = 0; i < I; ++i) *reinterpret_cast<u32x4*>(tile + lds_offset(row + i * ROW_STRIDE, kc)) = r[i];
+__device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
+    const unsigned long long v = (unsigned long long)p;
+    const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
+    const unsigned hi = __builtin_amdgcn_readfirstlane((unsigned)(v >> 32));
+    return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
 }
 
 template <int DT, int BM, int BN, int WM, int WN>
@@ -88,8 +96,6 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     constexpr int BK = ROW_BYTES / ES;                   // elements of K per tile
     constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile
     constexpr int TM = WTM / 32, TN = WTN / 32;          // 32x32 fragments per wave
-    constexpr int IA = BM * CHUNKS / NT, IB = BN * CHUNKS / NT;
-    static_assert(BM * CHUNKS % NT == 0 && BN * CHUNKS % NT == 0, "tile must be a multiple of the loader footprint");
     static_assert(TM >= 1 && TN >= 1, "wave tile too small");
     constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
 
@@ -105,12 +111,28 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     const long m0 = (long)tm * BM, n0 = (long)tn * BN;
     const long K = g.K;
 
-    // ---- loader: thread -> (row, chunk) of the A and B tiles ----
-    const int ld_row = tid >> 3, ld_kc = tid & 7;
-    const unsigned char* a_src = (const unsigned char*)g.A + ((m0 + ld_row) * K) * ES + ld_kc * 16;
-    const unsigned char* b_src = (const unsigned char*)g.B + ((n0 + ld_row) * K) * ES + ld_kc * 16;
-    const long row_step = (long)(NT / 8) * K * ES;  // bytes between a thread's consecutive rows
-    u32x4 ra[IA], rb[IB];
+    // ---- loader: DMA instruction q of wave w fills the 8 rows of row block q * NW + w of the
+    //      stacked (A rows, then B rows) tile ----
+    constexpr int NW = WM * WN;
+    constexpr int NI = (BM + BN) / 8 / NW;      // DMA instructions per wave and K-tile
+    constexpr int NIA = BM / 8 / NW;            // the first NIA of them fetch A
+    static_assert((BM / 8) % NW == 0 && (BN / 8) % NW == 0, "row blocks must split evenly over the waves");
+    const unsigned lds_base = (unsigned)(size_t)lds;
+    const unsigned char* src[NI];
+    unsigned lane_off[NI];
+    unsigned dst[NI];
+#pragma unroll
+    for (int q = 0; q < NI; ++q) {
+        const bool is_a = q < NIA;
+        const int blk = (is_a ? q : q - NIA) * NW + wave;           // row block inside the A (or B) tile
+        const int r = lane >> 3;                                    // row inside the block
+        const int kc = (lane & 7) ^ ((r ^ blk) & 7);                // global chunk that belongs in slot lane & 7
+        const unsigned char* origin = is_a ? (const unsigned char*)g.A + (m0 + blk * 8) * K * ES
+                                           : (const unsigned char*)g.B + (n0 + blk * 8) * K * ES;
+        src[q] = uniform_ptr(origin);
+        lane_off[q] = (unsigned)(r * K * ES + kc * 16);
+        dst[q] = __builtin_amdgcn_readfirstlane(lds_base + (is_a ? 0 : BM * ROW_BYTES) + blk * 8 * ROW_BYTES);
+    }
 
     f32x16 acc[TM][TN];
 #pragma unroll
@@ -162,25 +184,21 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     };
 
     const int nk = (int)(K / BK);
-    load_rows<IA>(ra, a_src, row_step);
-    load_rows<IB>(rb, b_src, row_step);
-    store_rows<IA, NT / 8>(ra, lds, ld_row, ld_kc);
-    store_rows<IB, NT / 8>(rb, lds + BM * ROW_BYTES, ld_row, ld_kc);
+#pragma unroll
+    for (int q = 0; q < NI; ++q) dma_to_lds(src[q], lane_off[q], dst[q]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     for (int kt = 0; kt < nk; ++kt) {
-        const bool more = kt + 1 < nk;
-        if (more) {
-            a_src += ROW_BYTES;
-            b_src += ROW_BYTES;
-            load_rows<IA>(ra, a_src, row_step);
-            load_rows<IB>(rb, b_src, row_step);
+        if (kt + 1 < nk) {
+            const unsigned stage_off = ((kt + 1) & 1) * STAGE_BYTES;
+#pragma unroll
+            for (int q = 0; q < NI; ++q) {
+                src[q] += ROW_BYTES;
+                dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
+            }
         }
         compute(kt & 1);
-        if (more) {
-            unsigned char* st = lds + ((kt + 1) & 1) * STAGE_BYTES;
-            store_rows<IA, NT / 8>(ra, st, ld_row, ld_kc);
-            store_rows<IB, NT / 8>(rb, st + BM * ROW_BYTES, ld_row, ld_kc);
-        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
     }
 
@@ -308,7 +326,7 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     const int lds_bytes = 2 * (BM + BN) * ROW_BYTES;
     static bool attr_set[64] = {false};
     int dev = 0;
-    hipGetDevice(&dev);
+    (void)hipGetDevice(&dev);
     if (!attr_set[dev & 63]) {
         hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
         if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes,
