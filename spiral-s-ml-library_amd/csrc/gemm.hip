@@ -21,6 +21,7 @@ typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 struct GemmArgs {
     const void* A;
@@ -41,6 +42,20 @@ constexpr int CHUNKS = 8;       // 16-byte chunks per LDS row
 // read at the same kc touch 8 different slots, and rows r, r+8 land in different 128-byte halves.
 __device__ __forceinline__ int lds_offset(int row, int kc) {
     return row * ROW_BYTES + (((kc ^ row ^ (row >> 3)) & 7) << 4);
+}
+
+template <int T>
+__device__ __forceinline__ float half_bits_to_f32(unsigned bits) {
+    if constexpr (T == SP_BF16) return __uint_as_float(bits << 16);
+    else return (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
+}
+
+__device__ __forceinline__ unsigned short f32_to_bf16_rne(float x);
+
+template <int T>
+__device__ __forceinline__ unsigned f32_to_half_bits(float x) {
+    if constexpr (T == SP_BF16) return f32_to_bf16_rne(x);
+    else return __builtin_bit_cast(unsigned short, (_Float16)x);
 }
 
 __device__ __forceinline__ unsigned short f32_to_bf16_rne(float x) {
@@ -89,7 +104,7 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
     return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
 }
 
-template <int DT, int BM, int BN, int WM, int WN>
+template <int DT, int OT, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g) {
     constexpr int NT = WM * WN * 64;
     constexpr int ES = (DT == SP_F32) ? 4 : 2;          // element size
@@ -144,99 +159,163 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
 
     const int frag_row = lane & 31, frag_half = lane >> 5;
 
-    auto compute = [&](int stage) {
+    // Per-lane LDS byte offsets of the fragments.  For fragment 0 the chunk of k-step t sits at
+    // va[t]; fragment i (32 rows further down) has the same low row bits and (row >> 3) + 4 * i, so
+    // its swizzle differs by bit 2 for odd i: its chunk for step ks sits at va[ks ^ 2 * (i & 1)] plus
+    // the constant i * 32 rows.  Only 8 address registers are live and the per-fragment part is an
+    // instruction immediate.  The stage (double buffer) is toggled into the registers once per tile.
+    int va[4], vb[4];
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const int kc = 2 * ks + frag_half;
-            u32x4 fa[TM], fb[TN];
+    for (int t = 0; t < 4; ++t) {
+        va[t] = lds_offset(wm * WTM + frag_row, 2 * t + frag_half);
+        vb[t] = BM * ROW_BYTES + lds_offset(wn * WTN + frag_row, 2 * t + frag_half);
+    }
+    auto load_frags = [&](int ks, u32x4(&fa)[TM], u32x4(&fb)[TN]) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const int row = wm * WTM + i * 32 + frag_row;  // swizzle uses the tile-relative row
-                fa[i] = *reinterpret_cast<const u32x4*>(lds + stage * STAGE_BYTES + lds_offset(row, kc));
-            }
+        for (int i = 0; i < TM; ++i)
+            fa[i] = *reinterpret_cast<const u32x4*>(lds + va[ks ^ (2 * (i & 1))] + i * 32 * ROW_BYTES);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+            fb[j] = *reinterpret_cast<const u32x4*>(lds + vb[ks ^ (2 * (j & 1))] + j * 32 * ROW_BYTES);
+    };
+    int stage_delta = STAGE_BYTES;
+    auto toggle_stage = [&]() {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            va[t] += stage_delta;
+            vb[t] += stage_delta;
+        }
+        stage_delta = -stage_delta;
+    };
+    // The B fragment is the MFMA's first operand, so the result fragment is (n, m): register r of
+    // lane l holds C[m = l % 32][n = 8 * (r / 4) + 4 * (l / 32) + r % 4], 4 consecutive columns per
+    // register quad.
+    auto mma = [&](const u32x4(&fa)[TM], const u32x4(&fb)[TN]) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const int row = wn * WTN + j * 32 + frag_row;
-                fb[j] = *reinterpret_cast<const u32x4*>(lds + stage * STAGE_BYTES + BM * ROW_BYTES +
-                                                        lds_offset(row, kc));
-            }
+                if constexpr (DT == SP_BF16) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                        __builtin_bit_cast(bf16x8, fb[j]), __builtin_bit_cast(bf16x8, fa[i]), acc[i][j], 0, 0, 0);
+                } else if constexpr (DT == SP_F16) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                        __builtin_bit_cast(f16x8, fb[j]), __builtin_bit_cast(f16x8, fa[i]), acc[i][j], 0, 0, 0);
+                } else {
+                    // the chunk holds 4 consecutive k for this half-wave; A and B use the same
+                    // k for the same (half, step), which is all the MFMA needs
+                    const f32x4 pa = __builtin_bit_cast(f32x4, fa[i]);
+                    const f32x4 pb = __builtin_bit_cast(f32x4, fb[j]);
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-#pragma unroll
-                for (int j = 0; j < TN; ++j) {
-                    if constexpr (DT == SP_BF16) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(bf16x8, fa[i]), __builtin_bit_cast(bf16x8, fb[j]), acc[i][j], 0, 0, 0);
-                    } else if constexpr (DT == SP_F16) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                            __builtin_bit_cast(f16x8, fa[i]), __builtin_bit_cast(f16x8, fb[j]), acc[i][j], 0, 0, 0);
-                    } else {
-                        // the chunk holds 4 consecutive k for this half-wave; A and B use the same
-                        // k for the same (half, step), which is all the MFMA needs
-                        const f32x4 pa = __builtin_bit_cast(f32x4, fa[i]);
-                        const f32x4 pb = __builtin_bit_cast(f32x4, fb[j]);
-#pragma unroll
-                        for (int s = 0; s < 4; ++s)
-                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[s], pb[s], acc[i][j], 0, 0, 0);
-                    }
+                    for (int s = 0; s < 4; ++s)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pb[s], pa[s], acc[i][j], 0, 0, 0);
                 }
-        }
+            }
     };
-
+    // Main loop: a continuous stream of k-steps (4 per K-tile).  Before the MFMAs of a step are
+    // issued, the fragments of the next step are requested from LDS, so LDS latency hides behind
+    // 8 * TM * TN / 8 MFMAs.  The K-tile boundary sits in front of the LAST step of a tile: wait
+    // for the next tile's DMA, barrier (every wave has finished reading this tile and everyone's
+    // share of the next tile has landed), request the next tile's first fragments, run the last
+    // step's MFMAs under that latency, then start the DMA of the tile after next into the stage
+    // that was just released.
     const int nk = (int)(K / BK);
+    u32x4 fa[2][TM], fb[2][TN];
 #pragma unroll
     for (int q = 0; q < NI; ++q) dma_to_lds(src[q], lane_off[q], dst[q]);
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (nk > 1) {
+#pragma unroll
+        for (int q = 0; q < NI; ++q) {
+            src[q] += ROW_BYTES;
+            dma_to_lds(src[q], lane_off[q], dst[q] + STAGE_BYTES);
+        }
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");  // tile 0 landed, tile 1 may be in flight
+    } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-        if (kt + 1 < nk) {
-            const unsigned stage_off = ((kt + 1) & 1) * STAGE_BYTES;
+    load_frags(0, fa[0], fb[0]);
+    auto first_three_steps = [&]() {
+#pragma unroll
+        for (int ks = 0; ks < 3; ++ks) {
+            load_frags(ks + 1, fa[(ks + 1) & 1], fb[(ks + 1) & 1]);
+            __builtin_amdgcn_sched_barrier(0);  // keep these reads ahead of the MFMAs below
+            mma(fa[ks & 1], fb[ks & 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    for (int kt = 0; kt + 1 < nk; ++kt) {
+        first_three_steps();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        __syncthreads();
+        toggle_stage();
+        load_frags(0, fa[0], fb[0]);
+        __builtin_amdgcn_sched_barrier(0);
+        mma(fa[1], fb[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (kt + 2 < nk) {
+            const unsigned stage_off = (kt & 1) * STAGE_BYTES;
 #pragma unroll
             for (int q = 0; q < NI; ++q) {
                 src[q] += ROW_BYTES;
                 dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
             }
         }
-        compute(kt & 1);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
     }
+    first_three_steps();
+    mma(fa[1], fb[1]);
 
-    // ---- epilogue: D fragment layout of the 32x32 MFMA: register r of lane l holds
-    //      row 8*(r/4) + 4*(l/32) + r%4, column l%32 ----
+    // ---- epilogue: each wave transposes its accumulators through a private LDS strip, 32 rows at
+    //      a time, so that C is written (and, for beta != 0, read) as whole rows of the wave tile:
+    //      16 bytes per lane, WTN * 4 contiguous bytes per row ----
+    constexpr int EPI_STRIDE = WTN * 4 + 16;       // bytes; the pad keeps the 16-byte column writes conflict free
+    constexpr int LPR = WTN / 4;                   // lanes per output row
+    constexpr int RPP = 64 / LPR;                  // rows per pass
+    static_assert(NW * 32 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
+    __syncthreads();                               // every wave is done reading the tile buffers
+    unsigned char* stg = lds + wave * (32 * EPI_STRIDE);
+    const int er = lane / LPR, ec = (lane % LPR) * 4;
+    const long col = n0 + wn * WTN + ec;
     const float alpha = g.alpha, beta = g.beta;
+    f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+    if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
 #pragma unroll
-    for (int i = 0; i < TM; ++i)
+    for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
-            const long col = n0 + wn * WTN + j * 32 + frag_row;
-            const float bias = g.bias ? g.bias[col] : 0.f;
+        for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const long row = m0 + wm * WTM + i * 32 + (r >> 2) * 8 + frag_half * 4 + (r & 3);
-                const long idx = row * g.N + col;
-                float v = alpha * acc[i][j][r];
-                if (g.out_dtype == SP_F32) {
-                    float* c = (float*)g.C;
-                    if (beta != 0.f) v += beta * c[idx];
-                    v += bias;
-                    if (g.relu) v = fmaxf(v, 0.f);
-                    c[idx] = v;
-                } else if (g.out_dtype == SP_BF16) {
-                    unsigned short* c = (unsigned short*)g.C;
-                    if (beta != 0.f) v += beta * __uint_as_float((unsigned)c[idx] << 16);
-                    v += bias;
-                    if (g.relu) v = fmaxf(v, 0.f);
-                    c[idx] = f32_to_bf16_rne(v);
-                } else {
-                    _Float16* c = (_Float16*)g.C;
-                    if (beta != 0.f) v += beta * (float)c[idx];
-                    v += bias;
-                    if (g.relu) v = fmaxf(v, 0.f);
-                    c[idx] = (_Float16)v;
+            for (int gq = 0; gq < 4; ++gq) {
+                f32x4 v = {acc[i][j][4 * gq], acc[i][j][4 * gq + 1], acc[i][j][4 * gq + 2], acc[i][j][4 * gq + 3]};
+                *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (j * 32 + gq * 8 + frag_half * 4) * 4) = v;
+            }
+#pragma unroll
+        for (int p = 0; p < 32 / RPP; ++p) {
+            const int rl = p * RPP + er;
+            f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
+            const long idx = (m0 + wm * WTM + i * 32 + rl) * g.N + col;
+            v = v * alpha;
+            if constexpr (OT == SP_F32) {
+                f32x4* c = reinterpret_cast<f32x4*>((float*)g.C + idx);
+                if (beta != 0.f) v += beta * *c;
+                v += bias4;
+                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                *c = v;
+            } else {
+                u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)g.C + idx);
+                if (beta != 0.f) {
+                    const u32x2 o = *c;
+                    v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
+                    v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
                 }
+                v += bias4;
+                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                u32x2 o;
+                o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
+                o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
+                *c = o;
             }
         }
+    }
 }
 
 // Shape-agnostic kernel: one thread per output element, 16-byte loads along K.  Used for shapes
@@ -320,9 +399,9 @@ static int choose_cfg(int dtype_in, long M, long N, long K) {
     return smallest;
 }
 
-template <int DT, int BM, int BN, int WM, int WN>
+template <int DT, int OT, int BM, int BN, int WM, int WN>
 static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
-    auto kernel = gemm_abt_kernel<DT, BM, BN, WM, WN>;
+    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN>;
     const int lds_bytes = 2 * (BM + BN) * ROW_BYTES;
     static bool attr_set[64] = {false};
     int dev = 0;
@@ -338,12 +417,12 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     return check_launch("sp_gemm_abt");
 }
 
-template <int DT>
+template <int DT, int OT>
 static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
     switch (cfg) {
-        case 0: return launch_tiled<DT, 256, 256, 2, 4>(g, stream);
-        case 1: return launch_tiled<DT, 128, 128, 2, 2>(g, stream);
-        case 2: return launch_tiled<DT, 64, 64, 2, 2>(g, stream);
+        case 0: return launch_tiled<DT, OT, 256, 256, 2, 4>(g, stream);
+        case 1: return launch_tiled<DT, OT, 128, 128, 2, 2>(g, stream);
+        case 2: return launch_tiled<DT, OT, 64, 64, 2, 2>(g, stream);
     }
     dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16));
     hipLaunchKernelGGL(gemm_abt_generic_kernel<DT>, grid, dim3(256), 0, stream, g);
@@ -407,8 +486,10 @@ extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const voi
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype_in) {
-        case SP_F32: return launch_dtype<SP_F32>(cfg, g, s);
-        case SP_F16: return launch_dtype<SP_F16>(cfg, g, s);
-        default: return launch_dtype<SP_BF16>(cfg, g, s);
+        case SP_F32: return launch_dtype<SP_F32, SP_F32>(cfg, g, s);
+        case SP_F16:
+            return dtype_out == SP_F32 ? launch_dtype<SP_F16, SP_F32>(cfg, g, s) : launch_dtype<SP_F16, SP_F16>(cfg, g, s);
+        default:
+            return dtype_out == SP_F32 ? launch_dtype<SP_BF16, SP_F32>(cfg, g, s) : launch_dtype<SP_BF16, SP_BF16>(cfg, g, s);
     }
 }
