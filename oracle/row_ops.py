@@ -15,8 +15,13 @@ cooperative-groups collectives is not specified by CUDA.  Two orders are offered
                       compared bit for bit:
                         lane t owns columns 4t..4t+3 of each 4*T-column chunk (T lanes per row)
                         s_t   = ((x0 + x1) + x2) + x3
-                        incl  = Hillis-Steele inclusive scan of s over the T lanes
-                                (for d = 1, 2, 4, ...: v_t += v_{t-d} for t >= d)
+                        incl  = inclusive scan of s over the T lanes:
+                                Hillis-Steele inside rows of min(T, 16) lanes
+                                  (for d = 1, 2, 4, 8: v_t += v_{t-d} for t >= d, t in the row);
+                                T >= 32: each lane of an odd 16-lane row adds the last value of
+                                  the row before it;
+                                T == 64: each lane of rows 2 and 3 then adds the value lane 31
+                                  holds after the previous step
                         start = carry + (incl_{t-1} or 0);  out_k = (...(start + x0) + ...) + x_k
                         carry = carry + incl_{T-1}                      (next chunk)
 """
@@ -141,6 +146,23 @@ def relu(x):
 # scans
 # ----------------------------------------------------------------------------------------------
 
+def _lane_scan(s, t):
+    """Inclusive scan of s (rows, t) over the t lanes of a row in the kernels' association."""
+    r = min(t, 16)
+    v = s.reshape(s.shape[0], t // r, r).copy()
+    d = 1
+    while d < r:
+        nxt = v.copy()
+        nxt[..., d:] = v[..., :-d] + v[..., d:]
+        v = nxt
+        d *= 2
+    if t >= 32:
+        v[:, 1::2, :] = v[:, 0::2, 15:16] + v[:, 1::2, :]
+    if t >= 64:
+        v[:, 2:4, :] = v[:, 1:2, 15:16] + v[:, 2:4, :]
+    return v.reshape(s.shape[0], t)
+
+
 def _wave_scan(x, inclusive=True):
     x = np.asarray(x)
     rows, cols = x.shape
@@ -155,13 +177,7 @@ def _wave_scan(x, inclusive=True):
     for c in range(n_chunks):
         v = xp[:, c]                                  # (rows, T, 4)
         s = ((v[..., 0] + v[..., 1]) + v[..., 2]) + v[..., 3]
-        incl = s.copy()
-        d = 1
-        while d < t:
-            nxt = incl.copy()
-            nxt[:, d:] = incl[:, d:] + incl[:, :-d]
-            incl = nxt
-            d *= 2
+        incl = _lane_scan(s, t)
         excl = np.concatenate([np.zeros((rows, 1), dtype=x.dtype), incl[:, :-1]], axis=1)
         run = carry[:, None] + excl
         for k in range(4):

@@ -52,25 +52,64 @@ void register_kernel(const char* name, const void* fn, int threads);
 #ifdef __HIPCC__
 constexpr int WAVE = 64;
 
-// Butterfly all-reduce inside aligned groups of T lanes (T a power of two <= 64).
+// Cross-lane move through the DPP data path (VALU speed, no LDS traffic).  CTRL is a DPP control
+// word: 0xB1 = quad_perm [1,0,3,2], 0x4E = quad_perm [2,3,0,1], 0x141 = row_half_mirror,
+// 0x140 = row_mirror, 0x110 + d = row_shr:d, 0x142 = row_bcast:15, 0x143 = row_bcast:31.
+// Lanes without a source (or masked out by ROW_MASK) receive 0.
+template <int CTRL, int ROW_MASK = 0xf, typename V>
+__device__ __forceinline__ V dpp_move(V v) {
+    static_assert(sizeof(V) == 4, "DPP moves 32-bit values");
+    return __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+
+// The value held by the partner lane of butterfly step D (lane ^ D) for values that are already
+// uniform inside aligned groups of D lanes, which is what an all-reduce produces step by step.
+template <int D, typename V>
+__device__ __forceinline__ V butterfly_partner(V v) {
+    if constexpr (D == 1) return dpp_move<0xB1>(v);
+    else if constexpr (D == 2) return dpp_move<0x4E>(v);
+    else if constexpr (D == 4) return dpp_move<0x141>(v);
+    else if constexpr (D == 8) return dpp_move<0x140>(v);
+    else return __shfl_xor(v, D, WAVE);
+}
+
+// Butterfly all-reduce inside aligned groups of T lanes (T a power of two <= 64).  Every level
+// combines the same two partial results in both partner lanes, so for a commutative f all lanes
+// of the group end with bit-identical values.
 template <int T, typename V, typename F>
 __device__ __forceinline__ V group_allreduce(V v, F f) {
-#pragma unroll
-    for (int d = 1; d < T; d <<= 1) v = f(v, __shfl_xor(v, d, WAVE));
+    if constexpr (T >= 2) v = f(v, butterfly_partner<1>(v));
+    if constexpr (T >= 4) v = f(v, butterfly_partner<2>(v));
+    if constexpr (T >= 8) v = f(v, butterfly_partner<4>(v));
+    if constexpr (T >= 16) v = f(v, butterfly_partner<8>(v));
+    if constexpr (T >= 32) v = f(v, butterfly_partner<16>(v));
+    if constexpr (T >= 64) v = f(v, butterfly_partner<32>(v));
     return v;
 }
 
-// Hillis-Steele inclusive scan inside aligned groups of T lanes: for d = 1, 2, 4, ...:
-// v_t = v_{t-d} + v_t for t >= d.  The association is part of the library's contract (the CPU
-// checker restates it to compare cumulative distributions bit for bit).
+// Inclusive prefix sum inside aligned groups of T lanes.  The association is part of the
+// library's contract (the CPU checker restates it to compare cumulative distributions bit for
+// bit):
+//   1. Hillis-Steele inside rows of min(T, 16) lanes: for d = 1, 2, 4, 8: v_t += v_{t-d} (t >= d);
+//   2. T >= 32: every lane of an odd 16-lane row adds the last value of the row before it;
+//   3. T == 64: every lane of rows 2 and 3 then adds the value lane 31 holds after step 2.
 template <int T, typename V>
 __device__ __forceinline__ V group_inclusive_scan(V v, int lane_in_group) {
-#pragma unroll
-    for (int d = 1; d < T; d <<= 1) {
-        V o = __shfl_up(v, d, T);
-        if (lane_in_group >= d) v = o + v;
-    }
+    constexpr int R = T < 16 ? T : 16;
+    if constexpr (R >= 2) { const V o = dpp_move<0x111>(v); if (R == 16 || lane_in_group >= 1) v = o + v; }
+    if constexpr (R >= 4) { const V o = dpp_move<0x112>(v); if (R == 16 || lane_in_group >= 2) v = o + v; }
+    if constexpr (R >= 8) { const V o = dpp_move<0x114>(v); if (R == 16 || lane_in_group >= 4) v = o + v; }
+    if constexpr (R >= 16) { const V o = dpp_move<0x118>(v); v = o + v; }
+    if constexpr (T >= 32) v = dpp_move<0x142, 0xa>(v) + v;
+    if constexpr (T >= 64) v = dpp_move<0x143, 0xc>(v) + v;
     return v;
+}
+
+// Value of lane `src` of the own group (src < T), broadcast to the group.
+template <int T, typename V>
+__device__ __forceinline__ V group_broadcast(V v, int src) {
+    if constexpr (T == 64) return __builtin_bit_cast(V, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
+    else return __shfl(v, src, T);
 }
 #endif
 

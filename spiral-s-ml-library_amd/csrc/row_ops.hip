@@ -81,6 +81,9 @@ __device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r)
     return philox_uniform_x(a.seed, sub, group);
 }
 
+// exp(x) = 2^(x * log2 e) on the hardware exp2 unit; relative error about 1e-6 for |x| < 20.
+__device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
+
 __device__ __forceinline__ float sum4(const float (&v)[4]) { return ((v[0] + v[1]) + v[2]) + v[3]; }
 
 template <int T, int C>
@@ -126,12 +129,15 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                     const int j = c * 4 * T + 4 * l + k;
                     if (ok[c] && (bi == INT_MAX_ || v[c][k] > bv)) { bv = v[c][k]; bi = j; }
                 }
-#pragma unroll
-            for (int d = 1; d < T; d <<= 1) {
-                const float ov = __shfl_xor(bv, d, WAVE);
-                const int oi = __shfl_xor(bi, d, WAVE);
+            auto better = [&](float ov, int oi) {
                 if (oi != INT_MAX_ && (bi == INT_MAX_ || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
-            }
+            };
+            if constexpr (T >= 2) better(butterfly_partner<1>(bv), butterfly_partner<1>(bi));
+            if constexpr (T >= 4) better(butterfly_partner<2>(bv), butterfly_partner<2>(bi));
+            if constexpr (T >= 8) better(butterfly_partner<4>(bv), butterfly_partner<4>(bi));
+            if constexpr (T >= 16) better(butterfly_partner<8>(bv), butterfly_partner<8>(bi));
+            if constexpr (T >= 32) better(butterfly_partner<16>(bv), butterfly_partner<16>(bi));
+            if constexpr (T >= 64) better(butterfly_partner<32>(bv), butterfly_partner<32>(bi));
         }
 
         // ---- the row map ----
@@ -154,15 +160,16 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 #pragma unroll
             for (int c = 0; c < C; ++c) {
 #pragma unroll
-                for (int k = 0; k < 4; ++k) p[c][k] = (p[c][k] == NEG_INF) ? 0.f : expf(p[c][k] - m);
+                for (int k = 0; k < 4; ++k) p[c][k] = (p[c][k] == NEG_INF) ? 0.f : fast_exp(p[c][k] - m);
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
             s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
             stat_sum = s;
+            const float inv = 1.f / s;   // one correctly rounded reciprocal per row, then multiplies
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] / s;
+                for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
         } else if (op == SP_ROW_REGRET_MATCHING || op == SP_ROW_MASKED_REGRET_MATCHING) {
             float s = 0.f;
 #pragma unroll
@@ -214,7 +221,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             for (int c = 0; c < C; ++c) {
                 const float s = sum4(p[c]);
                 const float incl = group_inclusive_scan<T>(s, l);
-                float prev = __shfl_up(incl, 1, T);
+                float prev = dpp_move<0x138>(incl);   // wave_shr:1 = the lane before
                 if (l == 0) prev = 0.f;
                 float run = carry + prev;
 #pragma unroll
@@ -227,7 +234,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                         cdf[c][k] = run;
                     }
                 }
-                if (C > 1) carry = carry + __shfl(incl, T - 1, T);
+                if (C > 1) carry = carry + group_broadcast<T>(incl, T - 1);
             }
         }
 
@@ -299,7 +306,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel_i32(const int* __restr
             if (ok) v = *reinterpret_cast<const int4*>(x + row * (long)cols + col);
             const int s = ((v.x + v.y) + v.z) + v.w;
             const int incl = group_inclusive_scan<T>(s, l);
-            int prev = __shfl_up(incl, 1, T);
+            int prev = dpp_move<0x138>(incl);
             if (l == 0) prev = 0;
             const int start = carry + prev;
             int4 r;
@@ -311,7 +318,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel_i32(const int* __restr
                 r = v;
             }
             if (ok) *reinterpret_cast<int4*>(out + row * (long)cols + col) = r;
-            if (C > 1) carry = carry + __shfl(incl, T - 1, T);
+            if (C > 1) carry = carry + group_broadcast<T>(incl, T - 1);
         }
     }
 }

@@ -177,7 +177,8 @@ def test_row_ops_full_size(P):
     assert (out["sample"] == orow.discrete_sampling(out["probs"], u, cdf=out["cdf"])).all()
     # size-independent properties
     assert np.abs(out["cdf"][:, -1] - 1).max() < 1e-5
-    assert (np.diff(out["cdf"], axis=1) >= 0).all()
+    # a parallel prefix sum is monotone only up to rounding where two lanes' partial sums meet
+    assert (np.diff(out["cdf"], axis=1) >= -2.5e-7).all()
     assert ((out["sample"] >= 0) & (out["sample"] < cols)).all()
     # scalar-outputs-only mode gives the same indices
     lean = P.row_ops(dev(x), dev(u), want=("argmax", "sample", "rowmax", "rowsum"))
