@@ -105,6 +105,29 @@ __device__ __forceinline__ V group_inclusive_scan(V v, int lane_in_group) {
     return v;
 }
 
+// All-reduce for one row per wave (T == 64) whose result comes back through a scalar register:
+// butterfly inside the 16-lane rows, row_bcast:15 / row_bcast:31 to fold the rows into lane 63,
+// v_readlane to broadcast.  Narrower groups use the butterfly.  Masked-out lanes of the row_bcast
+// steps keep their own value, so any idempotent-or-not f is safe (only lane 63 is read).
+template <int T, typename V, typename F>
+__device__ __forceinline__ V group_reduce(V v, F f) {
+    if constexpr (T < 64) {
+        return group_allreduce<T>(v, f);
+    } else {
+        v = f(v, butterfly_partner<1>(v));
+        v = f(v, butterfly_partner<2>(v));
+        v = f(v, butterfly_partner<4>(v));
+        v = f(v, butterfly_partner<8>(v));
+        const int vi = __builtin_bit_cast(int, v);
+        V o = __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(vi, vi, 0x142, 0xa, 0xf, false));
+        v = f(v, o);   // rows 1 and 3 fold in the row before them (their own value elsewhere: f(v, v))
+        const int vj = __builtin_bit_cast(int, v);
+        o = __builtin_bit_cast(V, __builtin_amdgcn_update_dpp(vj, vj, 0x143, 0xc, 0xf, false));
+        v = f(v, o);   // rows 2 and 3 fold in lane 31
+        return __builtin_bit_cast(V, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+    }
+}
+
 // Value of lane `src` of the own group (src < T), broadcast to the group.
 template <int T, typename V>
 __device__ __forceinline__ V group_broadcast(V v, int src) {

@@ -86,7 +86,9 @@ __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp
 
 __device__ __forceinline__ float sum4(const float (&v)[4]) { return ((v[0] + v[1]) + v[2]) + v[3]; }
 
-template <int T, int C>
+// FUSED = true is the lean instantiation behind sp_row_ops: the op is softmax, uniforms come from
+// a tensor and nothing is masked, so every op/philox/mask decision folds away at compile time.
+template <int T, int C, bool FUSED>
 __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -96,8 +98,10 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
     const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
     const float NEG_INF = -__builtin_inff();
     const int cols = a.cols;
-    const bool masked = (a.op == SP_ROW_MASKED_SOFTMAX || a.op == SP_ROW_MASKED_REGRET_MATCHING);
+    const int op = FUSED ? (int)SP_ROW_SOFTMAX : a.op;
+    const bool masked = (op == SP_ROW_MASKED_SOFTMAX || op == SP_ROW_MASKED_REGRET_MATCHING);
     const int limit = masked ? a.mask_size : cols;
+    const bool want_stats = FUSED || a.want_stats;
 
     for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += n_waves * ROWS_PER_WAVE) {
         const long row = row0 + sub;
@@ -118,32 +122,30 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             }
         }
 
-        // ---- argmax (and the row max of the raw input): lowest index among equal maxima ----
+        // ---- row max of the raw input, then argmax = lowest index holding it ----
         float bv = NEG_INF;
         int bi = INT_MAX_;
-        if (a.argmax != nullptr || a.rowmax != nullptr || a.want_stats) {
+        if (a.argmax != nullptr || a.rowmax != nullptr || want_stats) {
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const int j = c * 4 * T + 4 * l + k;
-                    if (ok[c] && (bi == INT_MAX_ || v[c][k] > bv)) { bv = v[c][k]; bi = j; }
-                }
-            auto better = [&](float ov, int oi) {
-                if (oi != INT_MAX_ && (bi == INT_MAX_ || ov > bv || (ov == bv && oi < bi))) { bv = ov; bi = oi; }
-            };
-            if constexpr (T >= 2) better(butterfly_partner<1>(bv), butterfly_partner<1>(bi));
-            if constexpr (T >= 4) better(butterfly_partner<2>(bv), butterfly_partner<2>(bi));
-            if constexpr (T >= 8) better(butterfly_partner<4>(bv), butterfly_partner<4>(bi));
-            if constexpr (T >= 16) better(butterfly_partner<8>(bv), butterfly_partner<8>(bi));
-            if constexpr (T >= 32) better(butterfly_partner<16>(bv), butterfly_partner<16>(bi));
-            if constexpr (T >= 64) better(butterfly_partner<32>(bv), butterfly_partner<32>(bi));
+                for (int k = 0; k < 4; ++k)
+                    if (ok[c]) bv = fmaxf(bv, v[c][k]);
+            bv = group_reduce<T>(bv, [](float x, float y) { return fmaxf(x, y); });
+            if (a.argmax != nullptr) {
+#pragma unroll
+                for (int c = C - 1; c >= 0; --c)
+#pragma unroll
+                    for (int k = 3; k >= 0; --k)
+                        if (ok[c] && v[c][k] == bv) bi = c * 4 * T + 4 * l + k;
+                bi = group_reduce<T>(bi, [](int x, int y) { return x < y ? x : y; });
+                if (bi == INT_MAX_) bi = 0;   // a row of NaNs: no element equals the max
+            }
         }
 
         // ---- the row map ----
         float p[C][4];
         float stat_sum = 0.f;
-        const int op = a.op;
         if (op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX) {
             float m = NEG_INF;
 #pragma unroll
@@ -155,7 +157,8 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                     p[c][k] = xv;
                     m = fmaxf(m, xv);
                 }
-            m = group_allreduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
+            if (op == SP_ROW_SOFTMAX && want_stats) m = bv;   // same reduction as the row max above
+            else m = group_reduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
             float s = 0.f;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
@@ -163,7 +166,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 for (int k = 0; k < 4; ++k) p[c][k] = (p[c][k] == NEG_INF) ? 0.f : fast_exp(p[c][k] - m);
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
-            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
             stat_sum = s;
             const float inv = 1.f / s;   // one correctly rounded reciprocal per row, then multiplies
 #pragma unroll
@@ -181,7 +184,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 }
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
-            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
             const float inv_len = 1.f / (float)limit;
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -199,7 +202,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 for (int k = 0; k < 4; ++k) q[k] = v[c][k] * v[c][k];
                 s = (c == 0) ? sum4(q) : s + sum4(q);
             }
-            s = group_allreduce<T>(s, [](float x, float y) { return x + y; });
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
@@ -248,15 +251,18 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
                     if (p[c][k] > 0.f) m = fmaxf(m, cdf[c][k]);
-            m = group_allreduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
-            if (row_ok) uu = (a.u != nullptr) ? a.u[row] : reference_row_uniform(a, row);
+            m = group_reduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
+            if (row_ok) {
+                if (FUSED || a.u != nullptr) uu = a.u[row];
+                else uu = reference_row_uniform(a, row);
+            }
             const float thr = uu * m;
 #pragma unroll
             for (int c = C - 1; c >= 0; --c)
 #pragma unroll
                 for (int k = 3; k >= 0; --k)
                     if (p[c][k] > 0.f && cdf[c][k] >= thr) pick = c * 4 * T + 4 * l + k;
-            pick = group_allreduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
+            pick = group_reduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
         }
 
         // ---- stores ----
@@ -367,6 +373,7 @@ static int check_rows_cols(const char* fn, int64_t rows, int64_t cols) {
     return SP_OK;
 }
 
+template <bool FUSED>
 static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
     int rc = require_gfx950(fn);
     if (rc != SP_OK) return rc;
@@ -374,8 +381,8 @@ static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
-        hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
-                           stream, a);
+        hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value, FUSED>), dim3(grid), dim3(ROW_THREADS),
+                           0, stream, a);
     });
     if (rc != SP_OK) return rc;
     return check_launch(fn);
@@ -398,7 +405,7 @@ extern "C" int sp_row_ops(const float* logits, const float* u, float* rowmax, fl
     a.x = logits; a.u = u; a.rowmax = rowmax; a.rowsum = rowsum; a.out = probs; a.cdf = cdf; a.argmax = argmax;
     a.sample = sample; a.rows = rows; a.cols = (int)cols; a.op = SP_ROW_SOFTMAX; a.mask_size = (int)cols;
     a.want_stats = 1; a.philox_mode = -1;
-    return launch_row(a, (hipStream_t)stream, __func__);
+    return launch_row<true>(a, (hipStream_t)stream, __func__);
 }
 
 extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, int64_t cols, int32_t mask_size,
@@ -414,7 +421,7 @@ extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, 
     RowArgs a{};
     a.x = x; a.out = out; a.rows = rows; a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols;
     a.philox_mode = -1;
-    return launch_row(a, (hipStream_t)stream, __func__);
+    return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 
 extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* philox, float* probs_out,
@@ -448,7 +455,7 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
         a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
         a.blocks = philox->blocks_per_grid;
     }
-    return launch_row(a, (hipStream_t)stream, __func__);
+    return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 
 extern "C" int sp_row_map_i32(int op, const int32_t* x, int32_t* out, int64_t rows, int64_t cols, void* stream) {
