@@ -1,9 +1,23 @@
-// Fused dense-stack forward for gfx950: every workgroup pushes a tile of 64 batch rows through all
-// layers.  Activations stay in LDS as 16-bit values (two ping-pong buffers); each layer's weight
-// matrix is streamed from L2 through a double-buffered LDS stage in 64-wide K-chunks; products run
-// on v_mfma_f32_32x32x16_{f16,bf16} with f32 accumulation; ReLU (and bias) are applied in
-// registers; the head (softmax / regret matching / sampling) runs on the last layer's f32
-// outputs without leaving the CU.
+// Fused dense-stack forward for gfx950.
+//
+// A workgroup is 4 waves; every wave owns 16 batch rows and pushes them through ALL layers, so
+// activations never leave the wave's registers: the f32 accumulator fragment of one layer,
+// after bias / ReLU / rounding to 16 bits, is bit-for-bit the MFMA operand fragment of the next
+// layer.  (v_mfma_f32_16x16x32_{f16,bf16}: a lane ends up with 4 consecutive rows of the first
+// operand.  The weight rows are therefore fed in the order 32 u + 8 (i / 4) + i % 4 for an even
+// output tile and + 4 for the odd tile next to it, so that the two quads a lane holds in a pair
+// of tiles are the 8 consecutive columns 32 u + 8 q .. + 7: exactly the K-values lane group q
+// feeds to the next layer's MFMA.)
+//
+// Weights are the shared operand.  All layers' weight matrices are cut into chunks of 64 K-columns
+// and streamed as one flat sequence through a ring of 4 LDS stages by global_load_lds DMA, three
+// chunks ahead of the MFMAs (also across layer boundaries); one barrier per chunk.  Inside a
+// stage a chunk is stored as 128-byte rows (one weight row each) whose eight 16-byte pieces are
+// XOR-swizzled with swz(row) = 2 * ((row >> 3) & 3) + ((row >> 1) & 1): a DMA instruction then fetches 8 whole 128-byte lines (8
+// adjacent lanes per line), and the ds_read_b128 operand fetches of the 16 rows of a tile are
+// bank-conflict free.
+//
+// The head (softmax / regret matching / sampling) runs on the last layer's f32 outputs.
 //
 // Semantics follow the graph interpreter of ml/layers.spi:194-240 (BlockMatmul = x . w^T with w
 // stored (out, in), relu = max 0) and the heads of ml/primitives.spi:711-722,748-798.
@@ -15,16 +29,16 @@ namespace sp {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
 
 constexpr int MLP_MAX_LAYERS = 8;
-constexpr int MLP_ROWS = 64;       // batch rows per workgroup
-constexpr int MLP_THREADS = 256;   // 4 waves; wave w owns output fragments w, w+4, ...
-constexpr int MLP_MAX_DIM = 256;   // widest layer input / hidden width
-constexpr int MLP_MAX_OUT = 64;    // widest head
-constexpr int W_ROW_BYTES = 144;   // 64 16-bit K values + 16 bytes of padding (odd number of 16-byte slots)
+constexpr int MLP_MAX_DIM = 256;       // widest layer input / hidden width
+constexpr int MLP_MAX_OUT = 64;        // widest head
+constexpr int MLP_STAGES = 4;
+constexpr int MLP_STAGE_BYTES = MLP_MAX_DIM * 128;   // 256 weight rows x 64 K-columns x 2 bytes
+constexpr int MLP_DMA_PER_CHUNK = MLP_MAX_DIM / 8;         // 1 KiB DMA instructions per full chunk
 constexpr int INT_MAX_ = 2147483647;
 
 struct MlpArgs {
@@ -40,213 +54,267 @@ struct MlpArgs {
     long batch;
     int head;
     int mask_size;
-    int act_stride_bytes;  // (max width + 8) * 2: odd number of 16-byte slots per row
 };
 
 template <int DT>
-__device__ __forceinline__ unsigned short to_half_bits(float v) {
+__device__ __forceinline__ unsigned to_half_bits(float v) {
     if constexpr (DT == SP_F16) {
         _Float16 h = (_Float16)v;
         return __builtin_bit_cast(unsigned short, h);
     } else {
         unsigned u = __float_as_uint(v);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
+        if ((u & 0x7fffffffu) > 0x7f800000u) return ((u >> 16) | 0x40u);
         u += 0x7fffu + ((u >> 16) & 1u);
-        return (unsigned short)(u >> 16);
+        return u >> 16;
     }
 }
 
-template <int DT>
-__global__ __launch_bounds__(MLP_THREADS) void mlp_forward_kernel(const MlpArgs a) {
+// One wave-wide DMA: lane i copies 16 bytes from base + lane_offset to LDS byte lds_addr + 16 * i.
+// Issued from inline assembly so the chunks in flight do not make the compiler wait before LDS
+// reads of the chunk being multiplied; completion is tracked by vmcnt.
+__device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane_offset, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :
+                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
+                 : "memory");
+}
+
+__device__ __forceinline__ int mlp_swz(int row) { return (((row >> 3) & 3) << 1) | ((row >> 1) & 1); }
+
+// NW waves per workgroup, 16 batch rows per wave.
+template <int DT, int NW>
+__global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
+    constexpr int MLP_THREADS = NW * 64;
+    constexpr int MLP_ROWS = NW * 16;
+    constexpr int MLP_DMA_PER_WAVE = MLP_DMA_PER_CHUNK / NW;
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
-    const int l32 = lane & 31, half = lane >> 5;
-    const long row0 = (long)blockIdx.x * MLP_ROWS;
-    const int stride = a.act_stride_bytes;
-    unsigned char* act0 = lds;
-    unsigned char* act1 = lds + MLP_ROWS * stride;
-    unsigned char* wst = lds + 2 * MLP_ROWS * stride;      // two weight stages of MLP_MAX_DIM rows
-    constexpr int WSTAGE = MLP_MAX_DIM * W_ROW_BYTES;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15;       // batch row inside the wave's 16-row tile; weight row inside a 16-row tile
+    const int q = lane >> 4;       // which 8 of the 32 K-values of an MFMA step this lane feeds
+    const long row = (long)blockIdx.x * MLP_ROWS + wave * 16 + j;
+    const bool row_ok = row < a.batch;
+    const unsigned lds_base = (unsigned)(size_t)lds;
+    const unsigned dummy_dst = lds_base + MLP_STAGES * MLP_STAGE_BYTES;
 
-    // ---- stage the input tile (zero rows past the batch) ----
+    // ---- weight chunk pipeline: chunk = (layer, 64-column slab c) ----
+    int pf_layer = 0, pf_c = 0;    // next chunk to fetch
+    int pf_stage = 0;
+    auto fetch_next_chunk = [&]() {
+        const bool live = pf_layer < a.n_layers;
+        const int layer = live ? pf_layer : 0;
+        const int K = a.dims[layer], N = a.dims[layer + 1];
+        const unsigned char* W = (const unsigned char*)a.w[layer];
+        const int n_instr = live ? (N + 7) / 8 : 0;            // 8 weight rows (128 bytes each) per instruction
+#pragma unroll
+        for (int m = 0; m < MLP_DMA_PER_WAVE; ++m) {
+            const int ii = wave + NW * m;
+            if (ii < n_instr) {
+                int n = ii * 8 + (lane >> 3);
+                const int piece = (lane & 7) ^ mlp_swz(n);        // the K piece that belongs in LDS slot lane & 7
+                n = n < N ? n : N - 1;                             // rows past N: any valid row, never used
+                int k = pf_c * 64 + piece * 8;
+                k = k <= K - 8 ? k : K - 8;                        // pieces past K: multiplied by zero activations
+                mlp_dma(W, (unsigned)((n * K + k) * 2), lds_base + pf_stage * MLP_STAGE_BYTES + ii * 1024);
+            } else {
+                mlp_dma((const unsigned char*)a.w[0], 0u, dummy_dst);  // keeps the per-chunk DMA count fixed
+            }
+        }
+        if (live) {
+            ++pf_c;
+            if (pf_c * 64 >= K) { pf_c = 0; ++pf_layer; }
+        }
+        pf_stage = (pf_stage + 1) & (MLP_STAGES - 1);
+    };
+    fetch_next_chunk();
+    fetch_next_chunk();
+    fetch_next_chunk();
+
+    // ---- the wave's input rows as MFMA operand fragments: for step s (32 K-values) lane (j, q)
+    //      holds x[row][32 s + 8 q .. + 7] ----
+    u32x4 act[MLP_MAX_DIM / 32];
     {
-        const int k0 = a.dims[0];
-        const int chunks_per_row = k0 / 8;
-        const int total = MLP_ROWS * chunks_per_row;
-        for (int id = tid; id < total; id += MLP_THREADS) {
-            const int r = id / chunks_per_row, c = id % chunks_per_row;
+        const int K0 = a.dims[0];
+        const unsigned char* xr = (const unsigned char*)a.x + row * K0 * 2;
+#pragma unroll
+        for (int s = 0; s < MLP_MAX_DIM / 32; ++s) {
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (row0 + r < a.batch)
-                v = *reinterpret_cast<const u32x4*>((const unsigned char*)a.x + ((row0 + r) * k0 + c * 8) * 2);
-            *reinterpret_cast<u32x4*>(act0 + r * stride + c * 16) = v;
+            if (row_ok && 32 * s + 8 * q < K0) v = *reinterpret_cast<const u32x4*>(xr + (32 * s + 8 * q) * 2);
+            act[s] = v;
         }
     }
 
-    unsigned char* act_in = act0;
-    unsigned char* act_out = act1;
+    f32x4 acc[MLP_MAX_DIM / 16];
+    int stage = 0;
+    // LDS byte offset of this lane's 16-byte weight piece for the first tile of a chunk: lane j feeds
+    // weight row n0 = 8 (j / 4) + j % 4 of the 32-row group, K piece 4 sp + q (sp = which 32-wide step
+    // of the chunk).  Tile t adds (t / 2) * 32 + (t % 2) * 4 rows, which leaves swz() unchanged.
+    const int n0 = 8 * (j >> 2) + (j & 3);
+    unsigned frag_off[2];
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) frag_off[sp] = (unsigned)(n0 * 128 + (((4 * sp + q) ^ mlp_swz(n0)) << 4));
+    auto tile_off = [](int t) { return ((t >> 1) * 32 + (t & 1) * 4) * 128; };
+    auto tile_col = [&](int t) { return 32 * (t >> 1) + 4 * (t & 1) + 8 * q; };  // first of this lane's 4 columns
+    // per-wave f32 staging of the last layer's outputs; it reuses the first weight stage once every
+    // wave is done with the weights
+    float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
+    static_assert(NW * 16 * MLP_MAX_OUT * 4 <= MLP_STAGE_BYTES, "head staging must fit one weight stage");
 
     for (int layer = 0; layer < a.n_layers; ++layer) {
         const int K = a.dims[layer], N = a.dims[layer + 1];
-        const int nf = (N + 31) / 32;              // 32-wide output fragments
-        const int wrows = nf * 32;
+        const int nt = 2 * ((N + 31) / 32);   // output tiles come in pairs covering 32 columns
         const bool last = layer + 1 == a.n_layers;
-        const unsigned char* W = (const unsigned char*)a.w[layer];
-        const int nchunks = (K + 63) / 64;
-        const int loads = wrows * 8 / MLP_THREADS;  // 16-byte pieces per thread and chunk (1..8)
+#pragma unroll
+        for (int t = 0; t < MLP_MAX_DIM / 16; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-        u32x4 rw[8];
-        auto fetch = [&](int kc, u32x4(&dst)[8]) {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if (i < loads) {
-                    const int id = i * MLP_THREADS + tid;
-                    const int n = id >> 3, c = id & 7;
-                    const int k = kc * 64 + c * 8;
-                    u32x4 v = {0u, 0u, 0u, 0u};
-                    if (n < N && k < K) v = *reinterpret_cast<const u32x4*>(W + ((long)n * K + k) * 2);
-                    dst[i] = v;
-                }
-            }
-        };
-        auto stash = [&](int stage, const u32x4(&src)[8]) {
+        for (int c = 0; c < MLP_MAX_DIM / 64; ++c) {
+            if (c * 64 < K) {
+                // the two newer chunks may still be in flight; everything older has landed
+                asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * MLP_DMA_PER_WAVE) : "memory");
+                __syncthreads();
+                fetch_next_chunk();   // into the stage every wave finished reading before this barrier
+                const unsigned char* st = lds + stage * MLP_STAGE_BYTES;
+                // Output tiles are walked in groups of 4 (64 columns) with one uniform branch per
+                // group, so that the 8 or 16 LDS reads and the MFMAs of a group form one straight
+                // line the scheduler can overlap.  A partly filled last group multiplies whatever
+                // the stage holds past row N; those columns are never used.
+                const bool two_steps = c * 64 + 32 < K;
+                auto mma = [&](int t, int sp, const u32x4& w) {
+                    // weights are the first operand: the result fragment is (n, batch row)
+                    if constexpr (DT == SP_F16)
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            __builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, act[2 * c + sp]), acc[t], 0, 0, 0);
+                    else
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                            __builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, act[2 * c + sp]), acc[t], 0, 0, 0);
+                };
+                auto read = [&](int t, int sp) {
+                    return *reinterpret_cast<const u32x4*>(st + frag_off[sp] + tile_off(t));
+                };
+                if (nt == MLP_MAX_DIM / 16 && two_steps) {
+                    // full-width chunk: 8 groups of (4 tiles, one 32-wide step), software pipelined by
+                    // hand: the weight pieces of group g + 2 are requested before the MFMAs of group g
+                    // (with one wave per SIMD nothing else hides the LDS latency)
+                    u32x4 w[3][4];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if (i < loads) {
-                    const int id = i * MLP_THREADS + tid;
-                    const int n = id >> 3, c = id & 7;
-                    *reinterpret_cast<u32x4*>(wst + stage * WSTAGE + n * W_ROW_BYTES + c * 16) = src[i];
-                }
-            }
-        };
-
-        f32x16 acc[2][2];  // [output fragment slot][batch-row fragment]
+                    for (int t = 0; t < 4; ++t) w[0][t] = read(t, 0);
 #pragma unroll
-        for (int s = 0; s < 2; ++s)
+                    for (int t = 0; t < 4; ++t) w[1][t] = read(t, 1);
 #pragma unroll
-            for (int m = 0; m < 2; ++m)
+                    for (int g = 0; g < 8; ++g) {
+                        if (g + 2 < 8) {
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[s][m][r] = 0.f;
-
-        fetch(0, rw);
-        __syncthreads();  // previous layer's readers of the weight stages and writers of act_in are done
-        stash(0, rw);
-        __syncthreads();
-        for (int kc = 0; kc < nchunks; ++kc) {
-            const bool more = kc + 1 < nchunks;
-            if (more) fetch(kc + 1, rw);
-            const int ksteps = (K - kc * 64) >= 64 ? 4 : (K - kc * 64) / 16;
-            const unsigned char* ws = wst + (kc & 1) * WSTAGE;
-            for (int ks = 0; ks < ksteps; ++ks) {
-                u32x4 fa[2];
+                            for (int t = 0; t < 4; ++t) w[(g + 2) % 3][t] = read(((g + 2) >> 1) * 4 + t, (g + 2) & 1);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int m = 0; m < 2; ++m)
-                    fa[m] = *reinterpret_cast<const u32x4*>(act_in + (m * 32 + l32) * stride +
-                                                            (kc * 64 + ks * 16 + half * 8) * 2);
+                        for (int t = 0; t < 4; ++t) mma((g >> 1) * 4 + t, g & 1, w[g % 3][t]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
 #pragma unroll
-                for (int s = 0; s < 2; ++s) {
-                    const int f = wave + 4 * s;
-                    if (f < nf) {
-                        const u32x4 fw = *reinterpret_cast<const u32x4*>(ws + (f * 32 + l32) * W_ROW_BYTES +
-                                                                         (ks * 16 + half * 8) * 2);
+                    for (int g4 = 0; g4 < MLP_MAX_DIM / 64; ++g4) {
+                        if (g4 * 4 < nt) {
+                            u32x4 w0[4], w1[4];
 #pragma unroll
-                        for (int m = 0; m < 2; ++m) {
-                            // weights as the first operand: the result fragment is (n, batch row), so a
-                            // lane ends up with 4 consecutive n of one row -> one 8-byte store
-                            if constexpr (DT == SP_F16)
-                                acc[s][m] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                                    __builtin_bit_cast(f16x8, fw), __builtin_bit_cast(f16x8, fa[m]), acc[s][m], 0, 0, 0);
-                            else
-                                acc[s][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                    __builtin_bit_cast(bf16x8, fw), __builtin_bit_cast(bf16x8, fa[m]), acc[s][m], 0, 0, 0);
+                            for (int t = 0; t < 4; ++t) w0[t] = read(g4 * 4 + t, 0);
+                            if (two_steps) {
+#pragma unroll
+                                for (int t = 0; t < 4; ++t) w1[t] = read(g4 * 4 + t, 1);
+                            }
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) mma(g4 * 4 + t, 0, w0[t]);
+                            if (two_steps) {
+#pragma unroll
+                                for (int t = 0; t < 4; ++t) mma(g4 * 4 + t, 1, w1[t]);
+                            }
                         }
                     }
                 }
+                stage = (stage + 1) & (MLP_STAGES - 1);
             }
-            if (more) stash((kc + 1) & 1, rw);
-            __syncthreads();
         }
 
-        // ---- layer epilogue: lane holds rows m*32 + l32, columns f*32 + 8*g + 4*half + 0..3 ----
+        // ---- layer epilogue: in tile t lane (j, q) holds columns tile_col(t) + 0..3 of batch row j;
+        //      tiles 2 s and 2 s + 1 together give it columns 32 s + 8 q .. + 7 ----
         const float* bias = a.b[layer];
-        float* lg = reinterpret_cast<float*>(wst);  // f32 staging of the last layer's outputs [64][wrows]
 #pragma unroll
-        for (int s = 0; s < 2; ++s) {
-            const int f = wave + 4 * s;
-            if (f >= nf) continue;
+        for (int t = 0; t < MLP_MAX_DIM / 16; ++t) {
+            if (t < nt && bias != nullptr) {
+                const int n = tile_col(t);
 #pragma unroll
-            for (int m = 0; m < 2; ++m) {
-                const int r_loc = m * 32 + l32;
+                for (int r = 0; r < 4; ++r)
+                    if (n + r < N) acc[t][r] += bias[n + r];
+            }
+        }
+        if (!last) {
 #pragma unroll
-                for (int gq = 0; gq < 4; ++gq) {
-                    const int n = f * 32 + gq * 8 + half * 4;
-                    float v[4];
+            for (int s = 0; s < MLP_MAX_DIM / 32; ++s) {
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (32 * s < N) {
+                    const f32x4 lo = acc[2 * s], hi = acc[2 * s + 1];
+                    v.x = to_half_bits<DT>(fmaxf(lo[0], 0.f)) | (to_half_bits<DT>(fmaxf(lo[1], 0.f)) << 16);
+                    v.y = to_half_bits<DT>(fmaxf(lo[2], 0.f)) | (to_half_bits<DT>(fmaxf(lo[3], 0.f)) << 16);
+                    v.z = to_half_bits<DT>(fmaxf(hi[0], 0.f)) | (to_half_bits<DT>(fmaxf(hi[1], 0.f)) << 16);
+                    v.w = to_half_bits<DT>(fmaxf(hi[2], 0.f)) | (to_half_bits<DT>(fmaxf(hi[3], 0.f)) << 16);
+                }
+                act[s] = v;
+            }
+        } else {
+            __syncthreads();   // all waves have read their last weight chunk: the stage can be reused
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        v[q] = acc[s][m][gq * 4 + q];
-                        if (bias != nullptr && n + q < N) v[q] += bias[n + q];
-                    }
-                    if (!last) {
+            for (int t = 0; t < MLP_MAX_OUT / 16; ++t) {
+                if (t < nt) {
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) v[q] = fmaxf(v[q], 0.f);
-                        u32x2 packed;
-                        packed.x = (unsigned)to_half_bits<DT>(v[0]) | ((unsigned)to_half_bits<DT>(v[1]) << 16);
-                        packed.y = (unsigned)to_half_bits<DT>(v[2]) | ((unsigned)to_half_bits<DT>(v[3]) << 16);
-                        *reinterpret_cast<u32x2*>(act_out + r_loc * stride + n * 2) = packed;
-                    } else {
-#pragma unroll
-                        for (int q = 0; q < 4; ++q) lg[r_loc * wrows + n + q] = v[q];
-                    }
+                    for (int r = 0; r < 4; ++r) head_rows[j * MLP_MAX_OUT + tile_col(t) + r] = acc[t][r];
                 }
             }
         }
-        unsigned char* t = act_in; act_in = act_out; act_out = t;
     }
-    __syncthreads();
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the dummy DMAs before the LDS is released
 
-    // ---- head: one thread per batch row ----
-    if (tid < MLP_ROWS && row0 + tid < a.batch) {
+    // ---- head: lanes 0..15 of every wave own one batch row each (the staging is wave private) ----
+    if (lane < 16 && row_ok) {
         const int N = a.dims[a.n_layers];
-        const int wrows = ((N + 31) / 32) * 32;
-        float* p = reinterpret_cast<float*>(wst) + tid * wrows;  // this row's outputs, updated in place
-        const long row = row0 + tid;
+        float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs, updated in place
         const int limit = a.mask_size > 0 ? a.mask_size : N;
         if (a.logits != nullptr)
-            for (int j = 0; j < N; ++j) a.logits[row * N + j] = p[j];
+            for (int n = 0; n < N; ++n) a.logits[row * N + n] = p[n];
         if (a.head == SP_HEAD_SOFTMAX || a.head == SP_HEAD_SOFTMAX_RM) {
             float m = -__builtin_inff();
-            for (int j = 0; j < limit; ++j) m = fmaxf(m, p[j]);
+            for (int n = 0; n < limit; ++n) m = fmaxf(m, p[n]);
             float s = 0.f;
-            for (int j = 0; j < N; ++j) {
-                p[j] = j < limit ? expf(p[j] - m) : 0.f;
-                s = s + p[j];
+            for (int n = 0; n < N; ++n) {
+                p[n] = n < limit ? expf(p[n] - m) : 0.f;
+                s = s + p[n];
             }
-            for (int j = 0; j < N; ++j) p[j] = p[j] / s;
+            for (int n = 0; n < N; ++n) p[n] = p[n] / s;
         }
         if (a.head == SP_HEAD_REGRET_MATCHING || a.head == SP_HEAD_SOFTMAX_RM) {
             float s = 0.f;
-            for (int j = 0; j < N; ++j) {
-                p[j] = j < limit ? fmaxf(p[j], 0.f) : 0.f;
-                s = s + p[j];
+            for (int n = 0; n < N; ++n) {
+                p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
+                s = s + p[n];
             }
             const float inv_len = 1.f / (float)limit;
-            for (int j = 0; j < N; ++j) p[j] = j < limit ? (s != 0.f ? p[j] / s : inv_len) : 0.f;
+            for (int n = 0; n < N; ++n) p[n] = n < limit ? (s != 0.f ? p[n] / s : inv_len) : 0.f;
         }
-        for (int j = 0; j < N; ++j) a.policy[row * N + j] = p[j];
+        for (int n = 0; n < N; ++n) a.policy[row * N + n] = p[n];
         if (a.action != nullptr) {
             // local_discrete_sampling (ml/primitives.spi:782-798), sequential prefix sums
             float run = 0.f, m = -__builtin_inff();
-            for (int j = 0; j < N; ++j) {
-                run = run + p[j];
-                if (p[j] > 0.f) m = fmaxf(m, run);
+            for (int n = 0; n < N; ++n) {
+                run = run + p[n];
+                if (p[n] > 0.f) m = fmaxf(m, run);
             }
             const float thr = a.u[row] * m;
             int pick = INT_MAX_;
             run = 0.f;
-            for (int j = 0; j < N; ++j) {
-                run = run + p[j];
-                if (pick == INT_MAX_ && p[j] > 0.f && run >= thr) pick = j;
+            for (int n = 0; n < N; ++n) {
+                run = run + p[n];
+                if (pick == INT_MAX_ && p[n] > 0.f && run >= thr) pick = n;
             }
             a.action[row] = pick;
         }
@@ -272,7 +340,6 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     if (head < SP_HEAD_NONE || head > SP_HEAD_SOFTMAX_RM) return fail(SP_ERR_ARG, "sp_mlp_forward: unknown head %d", head);
     if (action_out != nullptr && u == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward: action requested but u is NULL");
     MlpArgs a{};
-    int maxw = 0;
     for (int i = 0; i <= n_layers; ++i) {
         const int d = dims[i];
         if (d <= 0) return fail(SP_ERR_SHAPE, "sp_mlp_forward: dims[%d] must be positive", i);
@@ -282,7 +349,6 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
                             MLP_MAX_DIM);
             if (i > 0 && d % 32 != 0)
                 return fail(SP_ERR_SHAPE, "sp_mlp_forward: hidden width dims[%d] = %d must be a multiple of 32", i, d);
-            if (d > maxw) maxw = d;
         } else if (d > MLP_MAX_OUT) {
             return fail(SP_ERR_SHAPE, "sp_mlp_forward: output width %d must be <= %d", d, MLP_MAX_OUT);
         }
@@ -300,12 +366,20 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     if (rc != SP_OK) return rc;
     a.x = x; a.n_layers = n_layers; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size;
-    a.act_stride_bytes = (maxw + 8) * 2;
-    const int lds_bytes = 2 * MLP_ROWS * a.act_stride_bytes + 2 * MLP_MAX_DIM * W_ROW_BYTES;
-    auto kernel = dtype == SP_F16 ? mlp_forward_kernel<SP_F16> : mlp_forward_kernel<SP_BF16>;
-    hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    // 8 waves (128 rows) per workgroup halve the L2 -> LDS weight traffic and put two waves on every
+    // SIMD; taken once such workgroups still cover half the compute units
+    const int cus = device_cu_count();
+    const bool wide = (batch + 127) / 128 * 2 >= cus;
+    const int nw = wide ? 8 : 4;
+    const void* kernel;
+    if (dtype == SP_F16) kernel = wide ? (const void*)mlp_forward_kernel<SP_F16, 8> : (const void*)mlp_forward_kernel<SP_F16, 4>;
+    else kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
+    const int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-    const long blocks = (batch + MLP_ROWS - 1) / MLP_ROWS;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(MLP_THREADS), lds_bytes, (hipStream_t)stream, a);
+    const long blocks = (batch + nw * 16 - 1) / (nw * 16);
+    void* args[] = {(void*)&a};
+    e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(nw * 64), args, lds_bytes, (hipStream_t)stream);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward: launch failed: %s", hipGetErrorString(e));
     return check_launch(__func__);
 }

@@ -34,7 +34,10 @@ def check(LY, x, ws, u, dtype, head="softmax_regret_matching", mask=0, biases=No
     policy, action, logits = LY.mlp_forward(dev(x, t), [dev(w, t) for w in ws], bd, head, dev(u), mask, True)
     policy, action, logits = host(policy), host(action), host(logits)
     want_p, _, want_l = olayers.mlp_forward(x, ws, biases, HEAD_CODE[head], u, None, mask or None)
-    assert ogemm.rel_frobenius(logits, want_l) < 3e-3
+    # hidden activations are rounded to the storage dtype before they feed the next MFMA: f16 keeps
+    # 11 significant bits, bf16 only 8 (2^-9 relative rounding per activation and layer), so the raw
+    # last-layer outputs of a bf16 stack get a looser bound; the policy keeps the 3e-3 contract
+    assert ogemm.rel_frobenius(logits, want_l) < (3e-3 if dtype == "f16" else 1e-2)
     assert ogemm.rel_frobenius(policy, want_p) < 3e-3
     # against the oracle that rounds hidden activations to the storage dtype like the kernel does:
     # only summation order differs, which now and then flips a rounded activation by one ulp
