@@ -56,17 +56,19 @@ struct MlpArgs {
     int mask_size;
 };
 
+// max(x, 0) and rounding of two f32 values to the 16-bit storage type, packed into one register
+// (v_max_f32 + v_cvt_pk_{f16,bf16}_f32: round to nearest even in hardware).  The max is issued from
+// assembly because fmaxf() would first canonicalise its operand with a second v_max.
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 template <int DT>
-__device__ __forceinline__ unsigned to_half_bits(float v) {
-    if constexpr (DT == SP_F16) {
-        _Float16 h = (_Float16)v;
-        return __builtin_bit_cast(unsigned short, h);
-    } else {
-        unsigned u = __float_as_uint(v);
-        if ((u & 0x7fffffffu) > 0x7f800000u) return ((u >> 16) | 0x40u);
-        u += 0x7fffu + ((u >> 16) & 1u);
-        return u >> 16;
-    }
+__device__ __forceinline__ unsigned relu_pack2(float a, float b) {
+    float ra, rb;
+    asm("v_max_f32 %0, 0, %1" : "=v"(ra) : "v"(a));
+    asm("v_max_f32 %0, 0, %1" : "=v"(rb) : "v"(b));
+    if constexpr (DT == SP_F16) return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{ra, rb}, f16x2));
+    else return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{ra, rb}, bf16x2));
 }
 
 // One wave-wide DMA: lane i copies 16 bytes from base + lane_offset to LDS byte lds_addr + 16 * i.
@@ -77,6 +79,65 @@ __device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane
                  :
                  : "v"(lane_offset), "s"(base), "s"(lds_addr)
                  : "memory");
+}
+
+// Head of one batch row: optional softmax and/or regret matching over the columns j < limit, then
+// local_discrete_sampling (ml/primitives.spi:782-798) with sequential prefix sums.  `src` holds the
+// row's N last-layer outputs; MAXN bounds N at compile time so that narrow heads stay in registers.
+template <int MAXN>
+__device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, long row, int N, int limit) {
+    float p[MAXN];
+#pragma unroll
+    for (int n = 0; n < MAXN; ++n) p[n] = n < N ? src[n] : 0.f;
+    if (a.logits != nullptr) {
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n)
+            if (n < N) a.logits[row * N + n] = p[n];
+    }
+    if (a.head == SP_HEAD_SOFTMAX || a.head == SP_HEAD_SOFTMAX_RM) {
+        float m = -__builtin_inff();
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n)
+            if (n < limit) m = fmaxf(m, p[n]);
+        float s = 0.f;
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n) {
+            p[n] = n < limit ? expf(p[n] - m) : 0.f;
+            if (n < N) s = s + p[n];
+        }
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n) p[n] = p[n] / s;
+    }
+    if (a.head == SP_HEAD_REGRET_MATCHING || a.head == SP_HEAD_SOFTMAX_RM) {
+        float s = 0.f;
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n) {
+            p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
+            if (n < N) s = s + p[n];
+        }
+        const float inv_len = 1.f / (float)limit;
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n) p[n] = n < limit ? (s != 0.f ? p[n] / s : inv_len) : 0.f;
+    }
+#pragma unroll
+    for (int n = 0; n < MAXN; ++n)
+        if (n < N) a.policy[row * N + n] = p[n];
+    if (a.action != nullptr) {
+        float run = 0.f, m = -__builtin_inff();
+        float cdf[MAXN];
+#pragma unroll
+        for (int n = 0; n < MAXN; ++n) {
+            if (n < N) run = run + p[n];
+            cdf[n] = run;
+            if (n < N && p[n] > 0.f) m = fmaxf(m, run);
+        }
+        const float thr = a.u[row] * m;
+        int pick = INT_MAX_;
+#pragma unroll
+        for (int n = MAXN - 1; n >= 0; --n)
+            if (n < N && p[n] > 0.f && cdf[n] >= thr) pick = n;
+        a.action[row] = pick;
+    }
 }
 
 __device__ __forceinline__ int mlp_swz(int row) { return (((row >> 3) & 3) << 1) | ((row >> 1) & 1); }
@@ -255,10 +316,10 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
                 u32x4 v = {0u, 0u, 0u, 0u};
                 if (32 * s < N) {
                     const f32x4 lo = acc[2 * s], hi = acc[2 * s + 1];
-                    v.x = to_half_bits<DT>(fmaxf(lo[0], 0.f)) | (to_half_bits<DT>(fmaxf(lo[1], 0.f)) << 16);
-                    v.y = to_half_bits<DT>(fmaxf(lo[2], 0.f)) | (to_half_bits<DT>(fmaxf(lo[3], 0.f)) << 16);
-                    v.z = to_half_bits<DT>(fmaxf(hi[0], 0.f)) | (to_half_bits<DT>(fmaxf(hi[1], 0.f)) << 16);
-                    v.w = to_half_bits<DT>(fmaxf(hi[2], 0.f)) | (to_half_bits<DT>(fmaxf(hi[3], 0.f)) << 16);
+                    v.x = relu_pack2<DT>(lo[0], lo[1]);
+                    v.y = relu_pack2<DT>(lo[2], lo[3]);
+                    v.z = relu_pack2<DT>(hi[0], hi[1]);
+                    v.w = relu_pack2<DT>(hi[2], hi[3]);
                 }
                 act[s] = v;
             }
@@ -278,46 +339,10 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
     // ---- head: lanes 0..15 of every wave own one batch row each (the staging is wave private) ----
     if (lane < 16 && row_ok) {
         const int N = a.dims[a.n_layers];
-        float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs, updated in place
         const int limit = a.mask_size > 0 ? a.mask_size : N;
-        if (a.logits != nullptr)
-            for (int n = 0; n < N; ++n) a.logits[row * N + n] = p[n];
-        if (a.head == SP_HEAD_SOFTMAX || a.head == SP_HEAD_SOFTMAX_RM) {
-            float m = -__builtin_inff();
-            for (int n = 0; n < limit; ++n) m = fmaxf(m, p[n]);
-            float s = 0.f;
-            for (int n = 0; n < N; ++n) {
-                p[n] = n < limit ? expf(p[n] - m) : 0.f;
-                s = s + p[n];
-            }
-            for (int n = 0; n < N; ++n) p[n] = p[n] / s;
-        }
-        if (a.head == SP_HEAD_REGRET_MATCHING || a.head == SP_HEAD_SOFTMAX_RM) {
-            float s = 0.f;
-            for (int n = 0; n < N; ++n) {
-                p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
-                s = s + p[n];
-            }
-            const float inv_len = 1.f / (float)limit;
-            for (int n = 0; n < N; ++n) p[n] = n < limit ? (s != 0.f ? p[n] / s : inv_len) : 0.f;
-        }
-        for (int n = 0; n < N; ++n) a.policy[row * N + n] = p[n];
-        if (a.action != nullptr) {
-            // local_discrete_sampling (ml/primitives.spi:782-798), sequential prefix sums
-            float run = 0.f, m = -__builtin_inff();
-            for (int n = 0; n < N; ++n) {
-                run = run + p[n];
-                if (p[n] > 0.f) m = fmaxf(m, run);
-            }
-            const float thr = a.u[row] * m;
-            int pick = INT_MAX_;
-            run = 0.f;
-            for (int n = 0; n < N; ++n) {
-                run = run + p[n];
-                if (pick == INT_MAX_ && p[n] > 0.f && run >= thr) pick = n;
-            }
-            a.action[row] = pick;
-        }
+        float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs
+        if (N <= 8) head_row<8>(a, p, row, N, limit);      // narrow heads run in registers
+        else head_row<MLP_MAX_OUT>(a, p, row, N, limit);
     }
 }
 
