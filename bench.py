@@ -28,18 +28,32 @@ PEAK_HBM_GBS = 8000.0
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--prewarm-ms", type=float, default=300.0,
+                    help="untimed device warm-up before the W warm-up steps (the clocks of an idle GPU need tens of "
+                         "milliseconds of load to ramp up)")
     ap.add_argument("--no-extra", action="store_true", help="only the headline GEMM")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default=None, help="run a single extra case by name (profiling aid)")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain copy of 1 GiB (sp_map_f32 copy: 1 GiB read, 1 GiB written) so that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command holds a kernel of known traffic")
     return ap.parse_args()
 
 
+PREWARM_MS = 300.0
+
+
 def time_launches(fn, steps, warmup):
-    """W untimed + K timed launches.  Returns (wall ms per step between two full device syncs,
-    HIP-event ms per launch on the launch stream)."""
+    """Untimed device warm-up, W untimed + K timed launches.  Returns (wall ms per step between two
+    full device syncs, HIP-event ms per launch on the launch stream)."""
     import torch
+    t_end = time.perf_counter() + PREWARM_MS * 1e-3
+    while time.perf_counter() < t_end:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -88,6 +102,8 @@ def main():
     from ml import layers, matmul, primitives
     from oracle import gemm as ogemm, layers as olayers, row_ops as orow
 
+    global PREWARM_MS
+    PREWARM_MS = args.prewarm_ms
     torch.cuda.set_device(0)
     TD = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
     dev = lambda x, t=None: torch.from_numpy(np.ascontiguousarray(x)).cuda().to(t or torch.from_numpy(x).dtype)
@@ -118,12 +134,22 @@ def main():
                "tile": matmul.matmul_config_tf32(False, True, m, n, k, TD[dtype])}
         return res, (a, b)
 
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        primitives.map("copy", src)
+        torch.cuda.synchronize()
+        del src
+        torch.cuda.empty_cache()
+
     # ---------------- headline: bf16 4096^3, f32 accumulate, f32 out ----------------
-    head, (a, b) = gemm_case(2, 4096, 4096, 4096, "bf16")
     flops = 2.0 * 4096 ** 3
+    if args.only:   # profiling aid: only the named extra case runs, the headline fields stay empty
+        head, a, b = {"tflops": None, "wall_ms": None, "roofline": None, "tile": None}, None, None
+    else:
+        head, (a, b) = gemm_case(2, 4096, 4096, 4096, "bf16")
 
     cpu = None
-    if not args.no_cpu:
+    if not args.no_cpu and not args.only:
         t = best_of(lambda: np.matmul(a, b.T), 3)
         cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": len(os.sched_getaffinity(0)),
                "kind": "port", "sample": "full 4096^3 problem, np.matmul(A32, B32.T) in f32 on the bf16-rounded "
@@ -133,7 +159,7 @@ def main():
 
     extra = {}
     cases = []
-    if not args.no_extra:
+    if not args.no_extra or args.only:
         cases = [
             ("gemm_f32_1024", lambda: gemm_case(1, 1024, 1024, 1024, "f32")[0]),
             ("gemm_bf16_4096_bf16out", lambda: gemm_case(2, 4096, 4096, 4096, "bf16", "bf16")[0]),
@@ -153,8 +179,18 @@ def main():
             ws = [ogemm.round_to(olayers.weight_init(rng, o, i), "f16") for i, o in zip(dims[:-1], dims[1:])]
             u = (1 - rng.random(batch, dtype=np.float32)).astype(np.float32)
             xd, wd, ud = dev(x, torch.float16), [dev(w, torch.float16) for w in ws], dev(u)
-            fn = lambda: layers.mlp_forward(xd, wd, u=ud)
+            policy = torch.empty((batch, 3), dtype=torch.float32, device="cuda")
+            action = torch.empty((batch,), dtype=torch.int32, device="cuda")
+            import ctypes as C
+            from ml import _lib
+            wp = (C.c_void_p * 4)(*[w.data_ptr() for w in wd])
+            dp = (C.c_int32 * 5)(*dims)
+            call = (_lib.SP_F16, _lib.ptr(xd), 4, wp, None, dp, _lib.ptr(ud), _lib.ptr(policy), _lib.ptr(action), None,
+                    batch, _lib.HEAD_SOFTMAX_RM, 0)
+            fn = lambda: _lib.check(_lib.lib.sp_mlp_forward(*call, _lib.stream_ptr()))
             wall, ev = time_launches(fn, max(K, 200), W)
+            want_p, want_a, _ = olayers.mlp_forward(x, ws, u=u)
+            assert ogemm.rel_frobenius(policy.cpu().numpy(), want_p) < 3e-3, "bench MLP output drifted from the oracle"
             fl = 2.0 * batch * sum(i * o for i, o in zip(dims[:-1], dims[1:]))
             res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
                    "roofline": roofline_mfma(fl, ev, "f16"), "seed": 7,
@@ -207,6 +243,15 @@ def main():
         info = device_info()
     except Exception as e:  # the device query is informational only
         info = {"error": str(e)}
+
+    # HBM-side traffic of the headline kernel, measured separately with rocprofv3 --pmc (the counters
+    # cannot be read from inside this process); profiles/traffic.json holds the scaled figure
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            if head["roofline"] is not None:
+                head["roofline"]["traffic"] = json.load(f)["headline"]["traffic_bytes"]
+    except (OSError, KeyError, ValueError):
+        pass
 
     line = {
         "metric": "GEMM TFLOP/s (% MFMA peak) at 4096^3 bf16; fused MLP fwd rows/sec",

@@ -61,9 +61,10 @@ typedef struct {
  * ml/max_blocks_per_sm.py:2-31 (device attribute queries). */
 int sp_device_info(sp_device_info_t* out);
 
-/* Occupancy report for a named kernel family of this library ("gemm_bf16_256x256", "row_ops",
- * "mlp_forward", ...): registers, LDS bytes and resident workgroups per CU.  Stands in for
- * ml/max_blocks_per_sm.py:2-31.  Returns SP_ERR_ARG for an unknown name. */
+/* Occupancy report for a named kernel of this library: "gemm_bf16_256x256", "gemm_f16_256x256",
+ * "gemm_bf16_128x128", "gemm_f32_64x64", "row_ops", "row_map", "mlp_forward", "mlp_forward_wide".
+ * Registers, static LDS bytes and resident workgroups per CU (dynamic LDS not included).  Stands in
+ * for ml/max_blocks_per_sm.py:2-31.  Returns SP_ERR_ARG for an unknown name. */
 typedef struct {
     int32_t vgprs;              /* architected + accumulation VGPRs per lane (from the code object) */
     int32_t sgprs;
@@ -125,7 +126,7 @@ int sp_row_ops(const float* logits, const float* u, float* rowmax, float* rowsum
                int32_t* argmax, int32_t* sample, int64_t rows, int64_t cols, uint32_t flags, void* stream);
 
 typedef enum {
-    SP_ROW_IDENTITY = 0,                /* row_map (fun config x i j_tns => x)          primitives.spi:929 */
+    SP_ROW_IDENTITY = 0,                /* row_map (fun config x i j_tns => x)          primitives.spi:930 */
     SP_ROW_SOFTMAX = 1,                 /* local_softmax                                primitives.spi:711-716 */
     SP_ROW_MASKED_SOFTMAX = 2,          /* local_masked_softmax, mask j < mask_size     primitives.spi:748-759 */
     SP_ROW_LN_L2 = 3,                   /* local_ln_l2                                  primitives.spi:701-703 */
@@ -192,8 +193,8 @@ int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int
 
 typedef enum {
     SP_HEAD_NONE = 0,            /* policy_out receives the last layer's outputs */
-    SP_HEAD_SOFTMAX = 1,         /* softmax                          ml/layers.spi:374-380 */
-    SP_HEAD_REGRET_MATCHING = 2, /* regret_matching                  ml/layers.spi:382-388 */
+    SP_HEAD_SOFTMAX = 1,         /* softmax                          ml/layers.spi:370-375 */
+    SP_HEAD_REGRET_MATCHING = 2, /* regret_matching                  ml/layers.spi:377-382 */
     SP_HEAD_SOFTMAX_RM = 3       /* softmax, then regret matching of the probabilities */
 } sp_head;
 
@@ -212,13 +213,13 @@ typedef enum {
  *   weights[i]   (dims[i+1], dims[i]) row-major = the B operand of A.B^T (ml/layers.spi:467);
  *                `weights` is a HOST array of n_layers device pointers
  *   biases       NULL, or a host array of n_layers device pointers to f32 (dims[i+1],) (entries may be NULL)
- *   dims         host array of n_layers + 1 layer widths; dims[0..n_layers-1] multiples of 16 and <= 512,
- *                hidden widths multiples of 32 and <= 512, dims[n_layers] <= 64
+ *   dims         host array of n_layers + 1 layer widths; dims[0] a multiple of 16, hidden widths
+ *                multiples of 32, all <= 256; dims[n_layers] <= 64
  *   u            (batch,) f32 in (0, 1], or NULL when action_out is NULL
  *   policy_out   (batch, dims[n_layers]) f32
  *   action_out   (batch,) i32 or NULL
  *   logits_out   (batch, dims[n_layers]) f32 or NULL
- *   mask_size    0 = no mask, else the head only considers columns j < mask_size (ml/layers.spi:409-424)
+ *   mask_size    0 = no mask, else the head only considers columns j < mask_size (ml/layers.spi:408-432)
  */
 int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights, const float* const* biases,
                    const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,

@@ -3,7 +3,7 @@
 Follows the graph interpreter of ml/layers.spi:194-240: `BlockMatmul(x, w)` is
 `matmul_tf32' false true 1 x w 0 out`, i.e. out = x . w^T with the weight stored
 (out_features, in_features) row-major (`matmul (b,a) x = BlockMatmul(x, weight (a,b))`, :467);
-`relu = max 0` (:355); the heads are the row primitives (:365-424).  There is no bias in the
+`relu = max 0` (:355); the heads are the row primitives (:367-432).  There is no bias in the
 reference; `bias` here is this build's extension.
 
 PARITY UNPINNED end to end against the reference: its layer goldens
@@ -16,8 +16,8 @@ import numpy as np
 from . import gemm, row_ops
 
 HEAD_NONE = 0               # raw last-layer outputs
-HEAD_SOFTMAX = 1            # softmax (ml/layers.spi:374-380)
-HEAD_REGRET_MATCHING = 2    # regret_matching (:382-388)
+HEAD_SOFTMAX = 1            # softmax (ml/layers.spi:370-375)
+HEAD_REGRET_MATCHING = 2    # regret_matching (:377-382)
 HEAD_SOFTMAX_RM = 3         # softmax, then regret matching of the probabilities
 
 

@@ -445,6 +445,17 @@ static int validate_gemm(int dtype_in, int dtype_out, int64_t M, int64_t N, int6
     return SP_OK;
 }
 
+namespace {
+struct GemmKernelNames {
+    GemmKernelNames() {
+        register_kernel("gemm_bf16_256x256", (const void*)gemm_abt_kernel<SP_BF16, SP_F32, 256, 256, 2, 4>, 512);
+        register_kernel("gemm_f16_256x256", (const void*)gemm_abt_kernel<SP_F16, SP_F32, 256, 256, 2, 4>, 512);
+        register_kernel("gemm_bf16_128x128", (const void*)gemm_abt_kernel<SP_BF16, SP_F32, 128, 128, 2, 2>, 256);
+        register_kernel("gemm_f32_64x64", (const void*)gemm_abt_kernel<SP_F32, SP_F32, 64, 64, 2, 2>, 256);
+    }
+} gemm_kernel_names;
+}  // namespace
+
 }  // namespace sp
 
 using namespace sp;

@@ -346,6 +346,15 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
     }
 }
 
+namespace {
+struct MlpKernelNames {
+    MlpKernelNames() {
+        register_kernel("mlp_forward", (const void*)mlp_forward_kernel<SP_F16, 4>, 256);
+        register_kernel("mlp_forward_wide", (const void*)mlp_forward_kernel<SP_F16, 8>, 512);
+    }
+} mlp_kernel_names;
+}  // namespace
+
 }  // namespace sp
 
 using namespace sp;

@@ -388,6 +388,15 @@ static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
     return check_launch(fn);
 }
 
+namespace {
+struct RowKernelNames {
+    RowKernelNames() {
+        register_kernel("row_ops", (const void*)row_kernel<64, 1, true>, ROW_THREADS);
+        register_kernel("row_map", (const void*)row_kernel<64, 1, false>, ROW_THREADS);
+    }
+} row_kernel_names;
+}  // namespace
+
 }  // namespace sp
 
 using namespace sp;

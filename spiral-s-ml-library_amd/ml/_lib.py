@@ -112,3 +112,10 @@ def device_info():
     check(lib.sp_device_info(C.byref(info)))
     return {f: (getattr(info, f).decode() if isinstance(getattr(info, f), bytes) else getattr(info, f))
             for f, _ in DeviceInfo._fields_}
+
+
+def kernel_info(name):
+    """Registers / LDS / resident workgroups of a named kernel (ml/max_blocks_per_sm.py counterpart)."""
+    info = KernelInfo()
+    check(lib.sp_kernel_info(name.encode(), C.byref(info)))
+    return {f: getattr(info, f) for f, _ in KernelInfo._fields_}

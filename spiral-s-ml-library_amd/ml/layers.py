@@ -30,7 +30,7 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
     ml/layers.spi:227-240,467); biases: optional list of f32 (out_i,) or None entries (build
     extension, the reference has no bias); u: (batch,) f32 uniforms in (0, 1] or None (no action).
     head: None | "softmax" | "regret_matching" | "softmax_regret_matching"; mask_size > 0 restricts
-    the head to columns j < mask_size (masked_* layers, ml/layers.spi:409-424)."""
+    the head to columns j < mask_size (masked_* layers, ml/layers.spi:408-432)."""
     n = len(weights)
     dims = [x.shape[1]] + [w.shape[0] for w in weights]
     for i, w in enumerate(weights):

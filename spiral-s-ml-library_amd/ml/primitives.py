@@ -42,7 +42,7 @@ def _row_map(op, x, out=None, mask_size=0):
 
 
 def identity(x, out=None):
-    """row_map (fun config x i j_tns => x) (ml/primitives.spi:929)."""
+    """row_map (fun config x i j_tns => x) (ml/primitives.spi:930)."""
     return _row_map(_lib.ROW_IDENTITY, x, out)
 
 

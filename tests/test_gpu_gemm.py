@@ -183,3 +183,14 @@ def test_reference_self_test(MM):
     diff = float(MM.main_body(1024, 1024, 512))
     torch.cuda.synchronize()
     assert diff < 1e-3
+
+
+def test_device_and_kernel_info():
+    announce("device / kernel info")
+    from ml import _lib
+    info = _lib.device_info()
+    assert info["arch"].startswith("gfx950") and info["compute_units"] >= 64 and info["wavefront_size"] == 64
+    k = _lib.kernel_info("gemm_bf16_256x256")
+    assert k["threads_per_block"] == 512 and k["vgprs"] > 64
+    with pytest.raises(_lib.SpiralError):
+        _lib.kernel_info("no_such_kernel")
