@@ -33,6 +33,7 @@ struct GemmArgs {
     int relu;
     int out_dtype;
     int tiles_m, tiles_n;
+    int group_m;   // tile rows per group of the block -> tile walk (4: an XCD's 32 concurrent tiles form a 4 x 8 patch)
 };
 
 constexpr int ROW_BYTES = 128;  // bytes of K per LDS row and K-tile
@@ -69,9 +70,8 @@ __device__ __forceinline__ unsigned short f32_to_bf16_rne(float x) {
 // (each with a private L2), so id % 8 selects the XCD; each XCD gets a contiguous range of the
 // tile sequence, and the sequence walks the tile grid in column-major groups of GROUP_M tile rows
 // so that an XCD's concurrent tiles share A and B panels.
-__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int& tm, int& tn) {
+__device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n, int GROUP_M, int& tm, int& tn) {
     constexpr int XCDS = 8;
-    constexpr int GROUP_M = 4;
     const int n = tiles_m * tiles_n;
     const int xcd = pid % XCDS;
     const int idx = pid / XCDS;
@@ -122,7 +122,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     const int wm = wave / WN, wn = wave % WN;
 
     int tm, tn;
-    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, tm, tn);
+    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
     const long m0 = (long)tm * BM, n0 = (long)tn * BN;
     const long K = g.K;
 
@@ -265,54 +265,60 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     first_three_steps();
     mma(fa[1], fb[1]);
 
-    // ---- epilogue: each wave transposes its accumulators through a private LDS strip, 32 rows at
-    //      a time, so that C is written (and, for beta != 0, read) as whole rows of the wave tile:
-    //      16 bytes per lane, WTN * 4 contiguous bytes per row ----
-    constexpr int EPI_STRIDE = WTN * 4 + 16;       // bytes; the pad keeps the 16-byte column writes conflict free
-    constexpr int LPR = WTN / 4;                   // lanes per output row
+    // ---- epilogue: each wave transposes its accumulators through a private LDS strip of 32 rows x
+    //      up to 64 columns, so that C is written (and, for beta != 0, read) as whole row segments:
+    //      16 bytes per lane, up to 256 contiguous bytes per row ----
+    constexpr int SW = WTN < 64 ? WTN : 64;        // columns per strip
+    constexpr int SF = SW / 32;                    // fragments per strip
+    constexpr int EPI_STRIDE = SW * 4 + 16;        // bytes; the pad keeps the 16-byte column writes conflict free
+    constexpr int LPR = SW / 4;                    // lanes per output row
     constexpr int RPP = 64 / LPR;                  // rows per pass
     static_assert(NW * 32 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
     __syncthreads();                               // every wave is done reading the tile buffers
     unsigned char* stg = lds + wave * (32 * EPI_STRIDE);
     const int er = lane / LPR, ec = (lane % LPR) * 4;
-    const long col = n0 + wn * WTN + ec;
     const float alpha = g.alpha, beta = g.beta;
-    f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
-    if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
+        for (int js = 0; js < TN / SF; ++js) {
+            const long col = n0 + wn * WTN + js * SW + ec;
+            f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+            if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
 #pragma unroll
-            for (int gq = 0; gq < 4; ++gq) {
-                f32x4 v = {acc[i][j][4 * gq], acc[i][j][4 * gq + 1], acc[i][j][4 * gq + 2], acc[i][j][4 * gq + 3]};
-                *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (j * 32 + gq * 8 + frag_half * 4) * 4) = v;
-            }
+            for (int jj = 0; jj < SF; ++jj)
 #pragma unroll
-        for (int p = 0; p < 32 / RPP; ++p) {
-            const int rl = p * RPP + er;
-            f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
-            const long idx = (m0 + wm * WTM + i * 32 + rl) * g.N + col;
-            v = v * alpha;
-            if constexpr (OT == SP_F32) {
-                f32x4* c = reinterpret_cast<f32x4*>((float*)g.C + idx);
-                if (beta != 0.f) v += beta * *c;
-                v += bias4;
-                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                *c = v;
-            } else {
-                u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)g.C + idx);
-                if (beta != 0.f) {
-                    const u32x2 o = *c;
-                    v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
-                    v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
+                for (int gq = 0; gq < 4; ++gq) {
+                    const f32x16& c16 = acc[i][js * SF + jj];
+                    f32x4 v = {c16[4 * gq], c16[4 * gq + 1], c16[4 * gq + 2], c16[4 * gq + 3]};
+                    *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (jj * 32 + gq * 8 + frag_half * 4) * 4) = v;
                 }
-                v += bias4;
-                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                u32x2 o;
-                o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
-                o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
-                *c = o;
+#pragma unroll
+            for (int p = 0; p < 32 / RPP; ++p) {
+                const int rl = p * RPP + er;
+                f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
+                const long idx = (m0 + wm * WTM + i * 32 + rl) * g.N + col;
+                v = v * alpha;
+                if constexpr (OT == SP_F32) {
+                    f32x4* c = reinterpret_cast<f32x4*>((float*)g.C + idx);
+                    if (beta != 0.f) v += beta * *c;
+                    v += bias4;
+                    if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                    *c = v;
+                } else {
+                    u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)g.C + idx);
+                    if (beta != 0.f) {
+                        const u32x2 o = *c;
+                        v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
+                        v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
+                    }
+                    v += bias4;
+                    if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                    u32x2 o;
+                    o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
+                    o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
+                    *c = o;
+                }
             }
         }
     }
@@ -491,6 +497,7 @@ extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const voi
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.relu = (flags & SP_GEMM_RELU) ? 1 : 0;
     g.out_dtype = dtype_out;
+    g.group_m = 4;
     if (cfg >= 0) {
         g.tiles_m = (int)(M / kTileCfgs[cfg].bm);
         g.tiles_n = (int)(N / kTileCfgs[cfg].bn);
