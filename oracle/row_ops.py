@@ -36,9 +36,13 @@ def _f32(x):
 
 
 def lanes_per_row(cols):
-    """Lanes that share one row: one lane per 4 columns, rounded up to a power of two, at most 64."""
+    """Lanes that share one row in the kernels.  Up to 64 columns: one lane per 4 columns, rounded
+    up to a power of two.  Up to 256 columns: 16 lanes, each with one 4-column piece of every
+    64-column chunk.  Wider rows: 64 lanes, one piece per 256-column chunk."""
+    if cols > 256:
+        return 64
     t = 1
-    while t * 4 < cols and t < 64:
+    while t * 4 < cols and t < 16:
         t *= 2
     return t
 

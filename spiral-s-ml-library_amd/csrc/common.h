@@ -128,11 +128,61 @@ __device__ __forceinline__ V group_reduce(V v, F f) {
     }
 }
 
-// Value of lane `src` of the own group (src < T), broadcast to the group.
+// Value of lane `src` of the own group (src < T), broadcast to the group.  A 16-lane group is a
+// DPP row, whose lanes can all read one lane of the row directly (control 0x150 + lane).
 template <int T, typename V>
 __device__ __forceinline__ V group_broadcast(V v, int src) {
     if constexpr (T == 64) return __builtin_bit_cast(V, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), src));
     else return __shfl(v, src, T);
+}
+template <int T, typename V>
+__device__ __forceinline__ V group_broadcast_last(V v) {
+    if constexpr (T == 16) return dpp_move<0x15F>(v);
+    else return group_broadcast<T>(v, T - 1);
+}
+
+// max(x, y) as the single hardware instruction: fmaxf() first canonicalises operands that come
+// straight from memory, which doubles the instruction count of a max over freshly loaded data.
+__device__ __forceinline__ float vmax(float x, float y) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
+
+// One butterfly step of a max all-reduce, the cross-lane read folded into the v_max (the
+// compiler does this by itself for add and min, not for max).  The s_nop covers the two wait
+// states a DPP read needs after a VALU write of the same register.
+template <int D>
+__device__ __forceinline__ float max_with_partner(float v) {
+    float r;
+    if constexpr (D == 1)
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));
+    else if constexpr (D == 2)
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));
+    else if constexpr (D == 4)
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 row_half_mirror row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));
+    else
+        asm("s_nop 1\n\tv_max_f32_dpp %0, %1, %1 row_mirror row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));
+    return r;
+}
+
+// Row max for every lane of an aligned group of T lanes.
+template <int T>
+__device__ __forceinline__ float group_max(float v) {
+    if constexpr (T >= 2) v = max_with_partner<1>(v);
+    if constexpr (T >= 4) v = max_with_partner<2>(v);
+    if constexpr (T >= 8) v = max_with_partner<4>(v);
+    if constexpr (T >= 16) v = max_with_partner<8>(v);
+    if constexpr (T == 64) {
+        const int vi = __builtin_bit_cast(int, v);
+        float o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vi, vi, 0x142, 0xa, 0xf, false));
+        v = vmax(v, o);
+        const int vj = __builtin_bit_cast(int, v);
+        o = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(vj, vj, 0x143, 0xc, 0xf, false));
+        v = vmax(v, o);
+        v = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+    }
+    return v;
 }
 #endif
 

@@ -12,6 +12,8 @@
 
 namespace sp {
 
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+
 constexpr int ROW_THREADS = 256;
 constexpr int INT_MAX_ = 2147483647;
 
@@ -86,9 +88,7 @@ __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp
 
 __device__ __forceinline__ float sum4(const float (&v)[4]) { return ((v[0] + v[1]) + v[2]) + v[3]; }
 
-// FUSED = true is the lean instantiation behind sp_row_ops: the op is softmax, uniforms come from
-// a tensor and nothing is masked, so every op/philox/mask decision folds away at compile time.
-template <int T, int C, bool FUSED>
+template <int T, int C>
 __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -98,10 +98,10 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
     const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
     const float NEG_INF = -__builtin_inff();
     const int cols = a.cols;
-    const int op = FUSED ? (int)SP_ROW_SOFTMAX : a.op;
+    const int op = a.op;
     const bool masked = (op == SP_ROW_MASKED_SOFTMAX || op == SP_ROW_MASKED_REGRET_MATCHING);
     const int limit = masked ? a.mask_size : cols;
-    const bool want_stats = FUSED || a.want_stats;
+    const bool want_stats = a.want_stats;
 
     for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += n_waves * ROWS_PER_WAVE) {
         const long row = row0 + sub;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                     if (p[c][k] > 0.f) m = fmaxf(m, cdf[c][k]);
             m = group_reduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
             if (row_ok) {
-                if (FUSED || a.u != nullptr) uu = a.u[row];
+                if (a.u != nullptr) uu = a.u[row];
                 else uu = reference_row_uniform(a, row);
             }
             const float thr = uu * m;
@@ -286,6 +286,130 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             if (a.argmax != nullptr) a.argmax[row] = bi;
             if (a.sample != nullptr) a.sample[row] = pick;
             if (a.u_out != nullptr) a.u_out[row] = uu;
+        }
+    }
+}
+
+// The fused pipeline behind sp_row_ops: softmax of every row plus, each optional, the row max and
+// argmax of the input, the sum of exponentials, the probabilities, their running sums and one
+// inverse-CDF sample per row.  Same results as row_kernel (the probabilities and running sums
+// are computed by the same operations in the same order); what differs is the instruction count:
+// padding lanes hold -inf, whose exponential is 0, so no per-element validity tests remain, full
+// waves load and store without predicates, and the max reductions are single DPP instructions.
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs a) {
+    constexpr int ROWS_PER_WAVE = WAVE / T;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int l = lane % T;
+    const int sub = lane / T;
+    const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
+    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    const float NEG_INF = -__builtin_inff();
+    const int cols = a.cols;
+    const bool full_cols = cols == C * 4 * T;
+
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += n_waves * ROWS_PER_WAVE) {
+        const long row = row0 + sub;
+        const bool row_ok = row < a.rows;
+        const bool full = full_cols && row0 + ROWS_PER_WAVE <= a.rows;   // wave-uniform
+        const long base = row * (long)cols + 4 * l;
+
+        f32x4 v[C];
+        if (full) {
+#pragma unroll
+            for (int c = 0; c < C; ++c) v[c] = *reinterpret_cast<const f32x4*>(a.x + base + c * 4 * T);
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                v[c] = f32x4{NEG_INF, NEG_INF, NEG_INF, NEG_INF};
+                if (row_ok && c * 4 * T + 4 * l < cols) v[c] = *reinterpret_cast<const f32x4*>(a.x + base + c * 4 * T);
+            }
+        }
+
+        float bv = vmax(vmax(v[0][0], v[0][1]), vmax(v[0][2], v[0][3]));
+#pragma unroll
+        for (int c = 1; c < C; ++c) bv = vmax(bv, vmax(vmax(v[c][0], v[c][1]), vmax(v[c][2], v[c][3])));
+        bv = group_max<T>(bv);
+
+        int bi = INT_MAX_;
+        if (a.argmax != nullptr) {
+#pragma unroll
+            for (int c = C - 1; c >= 0; --c)
+#pragma unroll
+                for (int k = 3; k >= 0; --k)
+                    if (v[c][k] == bv) bi = c * 4 * T + 4 * l + k;
+            bi = group_reduce<T>(bi, [](int x, int y) { return x < y ? x : y; });
+            if (bi == INT_MAX_) bi = 0;   // a row of NaNs: no element equals the max
+        }
+
+        float p[C][4];
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(v[c][k] - bv);
+            s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+        }
+        s = group_reduce<T>(s, [](float x, float y) { return x + y; });
+        const float inv = 1.f / s;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
+
+        const bool want_sample = a.sample != nullptr;
+        float cdf[C][4];
+        int pick = INT_MAX_;
+        if (want_sample || a.cdf != nullptr) {
+            float carry = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float incl = group_inclusive_scan<T>(sum4(p[c]), l);
+                float prev = dpp_move<0x138>(incl);   // wave_shr:1 = the lane before
+                if (l == 0) prev = 0.f;
+                float run = carry + prev;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    run = run + p[c][k];
+                    cdf[c][k] = run;
+                }
+                if (C > 1) carry = carry + group_broadcast_last<T>(incl);
+            }
+            if (want_sample) {
+                // local_discrete_sampling (ml/primitives.spi:782-798): the first index with p > 0 whose
+                // running sum reaches u * (largest running sum over p > 0).  Inside one lane and chunk
+                // the four running sums never decrease and are > 0 only if some p is (p >= 0), so
+                // the largest of them over p > 0 is the last one, provided the chunk's sum is positive.
+                float m = NEG_INF;
+#pragma unroll
+                for (int c = 0; c < C; ++c) m = vmax(m, sum4(p[c]) > 0.f ? cdf[c][3] : NEG_INF);
+                m = group_max<T>(m);
+                const float uu = row_ok ? a.u[row] : 1.f;
+                const float thr = uu * m;
+#pragma unroll
+                for (int c = C - 1; c >= 0; --c)
+#pragma unroll
+                    for (int k = 3; k >= 0; --k)
+                        if (p[c][k] > 0.f && cdf[c][k] >= thr) pick = c * 4 * T + 4 * l + k;
+                pick = group_reduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
+            }
+        }
+
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (full || (row_ok && c * 4 * T + 4 * l < cols)) {
+                if (a.out != nullptr)
+                    *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) = f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
+                if (a.cdf != nullptr)
+                    *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) =
+                        f32x4{cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]};
+            }
+        }
+        if (row_ok && l == 0) {
+            if (a.rowmax != nullptr) a.rowmax[row] = bv;
+            if (a.rowsum != nullptr) a.rowsum[row] = s;
+            if (a.argmax != nullptr) a.argmax[row] = bi;
+            if (a.sample != nullptr) a.sample[row] = pick;
         }
     }
 }
@@ -329,16 +453,21 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel_i32(const int* __restr
     }
 }
 
+// Lanes that share a row.  Up to 64 columns: one lane per 4 columns (rounded up to a power of two).
+// Up to 256 columns: 16 lanes (one DPP row), each holding one 4-column piece of every 64-column
+// chunk, so a wave works on 4 rows at once and no reduction leaves its DPP row.  Wider rows: the
+// whole wave, one 4-column piece per 256-column chunk.
 static int lanes_per_row(long cols) {
+    if (cols > 256) return 64;
     int t = 1;
-    while (t * 4 < cols && t < 64) t *= 2;
+    while (t * 4 < cols && t < 16) t *= 2;
     return t;
 }
 
 static int row_grid(long rows, int t) {
     const long rows_per_block = (long)(WAVE / t) * (ROW_THREADS / WAVE);
     long blocks = (rows + rows_per_block - 1) / rows_per_block;
-    const long cap = (long)device_cu_count() * 8;  // 8 workgroups of 4 waves = 8 waves per SIMD
+    const long cap = (long)device_cu_count() * 32;  // several rounds of short workgroups: the dispatcher evens out the tail
     if (blocks > cap) blocks = cap;
     return (int)(blocks < 1 ? 1 : blocks);
 }
@@ -350,8 +479,14 @@ static int dispatch_tc(int t, int c, F&& f) {
         case 2: f(std::integral_constant<int, 2>{}, std::integral_constant<int, 1>{}); return SP_OK;
         case 4: f(std::integral_constant<int, 4>{}, std::integral_constant<int, 1>{}); return SP_OK;
         case 8: f(std::integral_constant<int, 8>{}, std::integral_constant<int, 1>{}); return SP_OK;
-        case 16: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 1>{}); return SP_OK;
-        case 32: f(std::integral_constant<int, 32>{}, std::integral_constant<int, 1>{}); return SP_OK;
+        case 16:
+            switch (c) {
+                case 1: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 1>{}); return SP_OK;
+                case 2: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 2>{}); return SP_OK;
+                case 3: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 3>{}); return SP_OK;
+                case 4: f(std::integral_constant<int, 16>{}, std::integral_constant<int, 4>{}); return SP_OK;
+            }
+            break;
         case 64:
             switch (c) {
                 case 1: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 1>{}); return SP_OK;
@@ -359,6 +494,7 @@ static int dispatch_tc(int t, int c, F&& f) {
                 case 3: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 3>{}); return SP_OK;
                 case 4: f(std::integral_constant<int, 64>{}, std::integral_constant<int, 4>{}); return SP_OK;
             }
+            break;
     }
     return fail(SP_ERR_SHAPE, "row kernels: unsupported lanes/chunks %d/%d", t, c);
 }
@@ -381,8 +517,12 @@ static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
-        hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value, FUSED>), dim3(grid), dim3(ROW_THREADS),
-                           0, stream, a);
+        if (FUSED)
+            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid),
+                               dim3(ROW_THREADS), 0, stream, a);
+        else
+            hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
+                               stream, a);
     });
     if (rc != SP_OK) return rc;
     return check_launch(fn);
@@ -391,8 +531,8 @@ static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
 namespace {
 struct RowKernelNames {
     RowKernelNames() {
-        register_kernel("row_ops", (const void*)row_kernel<64, 1, true>, ROW_THREADS);
-        register_kernel("row_map", (const void*)row_kernel<64, 1, false>, ROW_THREADS);
+        register_kernel("row_ops", (const void*)row_softmax_kernel<16, 4>, ROW_THREADS);
+        register_kernel("row_map", (const void*)row_kernel<16, 4>, ROW_THREADS);
     }
 } row_kernel_names;
 }  // namespace

@@ -149,6 +149,32 @@ def test_row_maps_against_oracle(P, rows, cols):
         assert (np.take_along_axis(probs, sample[:, None].astype(np.int64), 1) > 0).all()
 
 
+@pytest.mark.parametrize("cols", [8, 64, 100, 256, 768])
+def test_row_ops_zero_probabilities_and_extreme_uniforms(P, cols):
+    """Rows whose softmax underflows to exact zeros (also in whole lanes and chunks), with u = 1, tiny u and
+    u = 0: the index must still be the first one with p > 0 whose running sum reaches u * max."""
+    announce("row_ops zeros/extreme u cols=%d" % cols)
+    rng = np.random.default_rng(cols)
+    rows = 67
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    x[::3, : cols // 2] -= 300                      # leading zeros
+    x[1::3, cols // 4:] -= 300                      # trailing zeros
+    x[5, :] = -300; x[5, cols - 1] = 0              # a single atom at the end
+    x[6, :] = -300; x[6, 0] = 0                     # ... and at the start
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    u[::4] = 1.0
+    u[1::4] = 1e-30
+    u[2::8] = 0.0
+    out = {k: host(v) for k, v in P.row_ops(dev(x), dev(u)).items()}
+    assert (out["probs"] == 0).any()
+    assert (out["cdf"] == orow.inclusive_scan_sum(out["probs"], order="wave")).all()
+    expect = orow.discrete_sampling(out["probs"], u, cdf=out["cdf"])
+    assert (out["sample"] == expect).all()
+    assert (np.take_along_axis(out["probs"], out["sample"][:, None].astype(np.int64), 1) > 0).all()
+    assert out["sample"][5] == cols - 1 and out["sample"][6] == 0
+    assert (out["argmax"] == orow.argmax(x)).all()
+
+
 def test_sampling_edge_cases(P):
     announce("sampling edge cases")
     p = np.zeros((4, 8), dtype=np.float32)
