@@ -150,15 +150,20 @@ int sp_row_map_i32(int op, const int32_t* x, int32_t* out, int64_t rows, int64_t
 typedef enum {
     SP_PHILOX_BLOCK = 0,   /* row_map_reduce: subsequence = thread-in-block        primitives.spi:927 */
     SP_PHILOX_GRID = 1,    /* grid_row_map_reduce: subsequence = thread-in-grid    primitives.spi:1014,493 */
-    SP_PHILOX_GATHER = 2   /* row_gather_reduce: one row per thread                primitives.spi:409-413 */
+    SP_PHILOX_GATHER = 2,  /* row_gather_reduce: one row per thread                primitives.spi:409-413 */
+    SP_PHILOX_LAYER = 3    /* graph_run_host: the tensor is (blocks, rows_per_block, cols), block b works
+                              through its own slice, subsequence = thread-in-grid       layers.spi:339-344 */
 } sp_philox_mode;
 
 typedef struct {
     uint64_t seed;               /* reference: 12344321 (corecuda/cupy.spi:6) */
+    uint64_t offset;             /* 32-bit draws every thread has already consumed: the reference keeps one
+                                    generator state per thread for a whole graph run, and every sampling
+                                    node advances it by 4 draws per row-iteration (layers.spi:341) */
     int32_t mode;                /* sp_philox_mode */
     int32_t threads_per_block;   /* reference: 256 */
     int32_t blocks_per_grid;     /* reference: 24 (RTX 4060) or 112 (H100), corecuda/base.spi:14-42 */
-    int32_t reserved;
+    int32_t rows_per_block;      /* SP_PHILOX_LAYER only: rows of one block's slice */
 } sp_philox_t;
 
 /*
@@ -166,10 +171,29 @@ typedef struct {
  * then sample = local_discrete_sampling(probs).  Replaces `row_map_reduce
  * (local_softmax_and_discrete_sampling rng) x probs sample` and its masked / regret-matching
  * siblings (ml/primitives.spi:528-536,800-814).  Exactly one of `u` (rows,) f32 in (0,1] and
- * `philox` must be given.  probs_out, cdf_out and u_out (the uniform each row used) may be NULL.
+ * `philox` must be given.  probs_out, cdf_out, u_out (the uniform each row used) and prob_out may be
+ * NULL.  prob_out (rows,) receives the probability of the sampled index, which is what
+ * `local_get_prob config action_id (zip probs j_tns)` returns next to the action in the agents'
+ * `get_action` (ml/cem.spi:152-164, ml/cfr.spi:117-129); 0 for a row without positive mass.
  */
 int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* philox, float* probs_out, float* cdf_out,
-                  float* u_out, int32_t* sample_out, int64_t rows, int64_t cols, int32_t mask_size, void* stream);
+                  float* u_out, int32_t* sample_out, float* prob_out, int64_t rows, int64_t cols, int32_t mask_size,
+                  void* stream);
+
+/*
+ * prob_out[r] = op(x)[r, action[r]]: `row_gather_reduce` of `local_get_prob` after an optional
+ * (masked) softmax / regret matching (ml/primitives.spi:824-830; callers ml/cfr.spi:97-107).  The
+ * reference asserts that the action id is a column of the row; here an id outside [0, cols) gives 0.
+ */
+int sp_row_get_prob(int op, const float* x, const int32_t* action, float* prob_out, int64_t rows, int64_t cols,
+                    int32_t mask_size, void* stream);
+
+/*
+ * out[r] = (OR over j of (x[r, j] > 0) << j) mod modulo: `local_binarize` (ml/primitives.spi:817-821), the
+ * hash head `binarize` of ml/layers.spi:439-446.  The shift is the device's 32-bit shift: columns
+ * j >= 32 contribute nothing.  modulo must be positive.
+ */
+int sp_row_binarize(const float* x, uint32_t* out, int64_t rows, int64_t cols, uint32_t modulo, void* stream);
 
 typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID = 3 } sp_map_op;
 

@@ -98,3 +98,23 @@ def row_uniforms_gather(n_threads, cols, seed=CONSTANT_SEED, threads_per_block=2
     lt = t % threads_per_block
     sub = (t // threads_per_block) * threads_per_block + (lt % d) * t_per_row
     return curand_uniform(curand_words(seed, sub, 4 * (lt // d)))
+
+
+def row_uniforms_layer(blocks, rows_per_block, cols, seed=CONSTANT_SEED, threads_per_block=256, offset=0):
+    """Same for a sampling node of a layer graph run by `graph_run_host` (ml/layers.spi:339-344):
+    the tensor is (blocks, rows_per_block, cols), block b works through its own slice with the
+    block-level `row_map_reduce`, the generator is seeded once per thread with subsequence =
+    thread-in-grid and keeps its state for the whole run, so a node starts `offset` draws in
+    (4 per row-iteration of every earlier sampling node).  Returns (blocks * rows_per_block,)."""
+    t = cols // 4
+    r_per_iter = threads_per_block // t
+    b = np.repeat(np.arange(blocks), rows_per_block)
+    r = np.tile(np.arange(rows_per_block), blocks)
+    sub = b * threads_per_block + (r % r_per_iter) * t
+    return curand_uniform(curand_words(seed, sub, offset + 4 * (r // r_per_iter)))
+
+
+def draws_per_sampling_node(rows_per_block, cols, threads_per_block=256):
+    """32-bit draws one sampling node takes from every thread's generator: 4 per row-iteration."""
+    r_per_iter = threads_per_block // (cols // 4)
+    return 4 * ((rows_per_block + r_per_iter - 1) // r_per_iter)

@@ -27,6 +27,10 @@ struct RowArgs {
     float* u_out;
     int* argmax;
     int* sample;
+    const int* action;     // get_prob: the column whose mapped value goes to prob_out (nullptr: the sampled one)
+    float* prob_out;
+    unsigned* bits_out;    // binarize
+    unsigned modulo;
     long rows;
     int cols;
     int op;                // sp_row_op
@@ -37,13 +41,15 @@ struct RowArgs {
     int philox_mode;       // -1: none
     int tpb;
     int blocks;
+    int rows_per_block;
+    unsigned long long draw_offset;
 };
 
 // Philox4x32-10 (Salmon et al., SC'11) with cuRAND's counter layout: key = seed, counter =
-// (group, 0, subsequence_lo, subsequence_hi); returns the first word of the group, mapped to (0, 1]
+// (group, 0, subsequence_lo, subsequence_hi); returns word `word` of the group, mapped to (0, 1]
 // like curand_uniform (corecuda/random.spi:22-32,84).
-__device__ __forceinline__ float philox_uniform_x(unsigned long long seed, unsigned long long subsequence,
-                                                  unsigned long long group) {
+__device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigned long long subsequence,
+                                                unsigned long long group, int word) {
     unsigned c0 = (unsigned)group, c1 = (unsigned)(group >> 32), c2 = (unsigned)subsequence,
              c3 = (unsigned)(subsequence >> 32);
     unsigned k0 = (unsigned)seed, k1 = (unsigned)(seed >> 32);
@@ -58,7 +64,8 @@ __device__ __forceinline__ float philox_uniform_x(unsigned long long seed, unsig
         unsigned n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
         c0 = n0; c1 = n1; c2 = n2; c3 = n3;
     }
-    return (float)c0 * 2.3283064e-10f + 1.1641532e-10f;
+    const unsigned w = word == 0 ? c0 : word == 1 ? c1 : word == 2 ? c2 : c3;
+    return (float)w * 2.3283064e-10f + 1.1641532e-10f;
 }
 
 // Which (subsequence, 4-word group) the reference's sampling op uses for row r: every thread of
@@ -75,12 +82,17 @@ __device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r)
         const long it = r / per_iter;
         sub = (it % a.blocks) * a.tpb + (r % per_iter) * t;
         group = it / a.blocks;
-    } else {  // SP_PHILOX_GATHER: row r belongs to thread r
+    } else if (a.philox_mode == SP_PHILOX_GATHER) {  // row r belongs to thread r
         const long lt = r % a.tpb;
         sub = (r / a.tpb) * a.tpb + (lt % per_iter) * t;
         group = lt / per_iter;
+    } else {  // SP_PHILOX_LAYER: block b = r / rows_per_block walks its own slice (ml/layers.spi:339-344)
+        const long b = r / a.rows_per_block, rb = r % a.rows_per_block;
+        sub = b * a.tpb + (rb % per_iter) * t;
+        group = rb / per_iter;
     }
-    return philox_uniform_x(a.seed, sub, group);
+    // the generator is `draw_offset` draws in; this row uses the first draw of its 4-draw group
+    return philox_uniform(a.seed, sub, group + a.draw_offset / 4, (int)(a.draw_offset % 4));
 }
 
 // exp(x) = 2^(x * log2 e) on the hardware exp2 unit; relative error about 1e-6 for |x| < 20.
@@ -265,6 +277,31 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             pick = group_reduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
         }
 
+        // ---- local_get_prob (ml/primitives.spi:824-830): the mapped value at one column ----
+        float got = 0.f;
+        if (a.prob_out != nullptr) {
+            const int id = a.action != nullptr ? (row_ok ? a.action[row] : 0) : pick;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (ok[c] && c * 4 * T + 4 * l + k == id) got = p[c][k];
+            got = group_reduce<T>(got, [](float x, float y) { return x + y; });   // one non-zero term: exact
+        }
+
+        // ---- local_binarize (ml/primitives.spi:817-821) ----
+        unsigned bits = 0;
+        if (a.bits_out != nullptr) {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int j = c * 4 * T + 4 * l + k;
+                    if (ok[c] && j < 32 && v[c][k] > 0.f) bits |= 1u << j;
+                }
+            bits = group_reduce<T>(bits, [](unsigned x, unsigned y) { return x | y; });
+        }
+
         // ---- stores ----
         float* out_ptr = is_scan ? nullptr : a.out;
         float* cdf_ptr = is_scan ? a.out : a.cdf;
@@ -286,6 +323,8 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             if (a.argmax != nullptr) a.argmax[row] = bi;
             if (a.sample != nullptr) a.sample[row] = pick;
             if (a.u_out != nullptr) a.u_out[row] = uu;
+            if (a.prob_out != nullptr) a.prob_out[row] = got;
+            if (a.bits_out != nullptr) a.bits_out[row] = bits % a.modulo;
         }
     }
 }
@@ -574,11 +613,12 @@ extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, 
 }
 
 extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* philox, float* probs_out,
-                             float* cdf_out, float* u_out, int32_t* sample_out, int64_t rows, int64_t cols,
-                             int32_t mask_size, void* stream) {
+                             float* cdf_out, float* u_out, int32_t* sample_out, float* prob_out, int64_t rows,
+                             int64_t cols, int32_t mask_size, void* stream) {
     SP_REQUIRE_PTR(x);
     SP_REQUIRE_PTR(sample_out);
     SP_OPTIONAL_PTR(u); SP_OPTIONAL_PTR(probs_out); SP_OPTIONAL_PTR(cdf_out); SP_OPTIONAL_PTR(u_out);
+    SP_OPTIONAL_PTR(prob_out);
     int rc = check_rows_cols(__func__, rows, cols);
     if (rc != SP_OK) return rc;
     if (!(op == SP_ROW_IDENTITY || op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX ||
@@ -591,9 +631,10 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
         return fail(SP_ERR_ARG, "sp_row_sample: exactly one of u and philox must be given");
     RowArgs a{};
     a.x = x; a.u = u; a.out = probs_out; a.cdf = cdf_out; a.u_out = u_out; a.sample = sample_out; a.rows = rows;
+    a.prob_out = prob_out;
     a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols; a.philox_mode = -1;
     if (philox != nullptr) {
-        if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_GATHER)
+        if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_LAYER)
             return fail(SP_ERR_ARG, "sp_row_sample: unknown philox mode %d", philox->mode);
         const int64_t t = cols / 4;
         if (philox->threads_per_block <= 0 || philox->threads_per_block % t != 0)
@@ -601,8 +642,12 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
                         philox->threads_per_block, (long long)t);
         if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
             return fail(SP_ERR_ARG, "sp_row_sample: blocks_per_grid must be positive");
+        if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || rows % philox->rows_per_block != 0))
+            return fail(SP_ERR_ARG, "sp_row_sample: rows_per_block (%d) must be positive and divide rows (%lld)",
+                        philox->rows_per_block, (long long)rows);
         a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
-        a.blocks = philox->blocks_per_grid;
+        a.blocks = philox->blocks_per_grid; a.rows_per_block = philox->rows_per_block;
+        a.draw_offset = philox->offset;
     }
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
@@ -625,4 +670,36 @@ extern "C" int sp_row_map_i32(int op, const int32_t* x, int32_t* out, int64_t ro
     });
     if (rc != SP_OK) return rc;
     return check_launch(__func__);
+}
+
+extern "C" int sp_row_get_prob(int op, const float* x, const int32_t* action, float* prob_out, int64_t rows,
+                               int64_t cols, int32_t mask_size, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(action);
+    SP_REQUIRE_PTR(prob_out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (!(op == SP_ROW_IDENTITY || op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX ||
+          op == SP_ROW_REGRET_MATCHING || op == SP_ROW_MASKED_REGRET_MATCHING || op == SP_ROW_LN_L2))
+        return fail(SP_ERR_ARG, "sp_row_get_prob: op %d is not a row map", op);
+    const bool masked = (op == SP_ROW_MASKED_SOFTMAX || op == SP_ROW_MASKED_REGRET_MATCHING);
+    if (masked && (mask_size < 1 || mask_size > cols))
+        return fail(SP_ERR_ARG, "sp_row_get_prob: mask_size must be in [1, cols], got %d", mask_size);
+    RowArgs a{};
+    a.x = x; a.action = action; a.prob_out = prob_out; a.rows = rows; a.cols = (int)cols; a.op = op;
+    a.mask_size = masked ? mask_size : (int)cols; a.philox_mode = -1;
+    return launch_row<false>(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_row_binarize(const float* x, uint32_t* out, int64_t rows, int64_t cols, uint32_t modulo,
+                               void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (modulo == 0) return fail(SP_ERR_ARG, "sp_row_binarize: modulo must be positive");
+    RowArgs a{};
+    a.x = x; a.bits_out = out; a.modulo = modulo; a.rows = rows; a.cols = (int)cols; a.op = SP_ROW_IDENTITY;
+    a.mask_size = (int)cols; a.philox_mode = -1;
+    return launch_row<false>(a, (hipStream_t)stream, __func__);
 }

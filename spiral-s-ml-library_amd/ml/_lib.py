@@ -11,7 +11,7 @@ SP_F32, SP_F16, SP_BF16 = 0, 1, 2
 GEMM_RELU, GEMM_FORCE_GENERIC = 0x1, 0x100
 (ROW_IDENTITY, ROW_SOFTMAX, ROW_MASKED_SOFTMAX, ROW_LN_L2, ROW_REGRET_MATCHING, ROW_MASKED_REGRET_MATCHING,
  ROW_INCLUSIVE_SCAN, ROW_EXCLUSIVE_SCAN) = range(8)
-PHILOX_BLOCK, PHILOX_GRID, PHILOX_GATHER = 0, 1, 2
+PHILOX_BLOCK, PHILOX_GRID, PHILOX_GATHER, PHILOX_LAYER = 0, 1, 2, 3
 MAP_COPY, MAP_RELU, MAP_TANH, MAP_SIGMOID = 0, 1, 2, 3
 HEAD_NONE, HEAD_SOFTMAX, HEAD_REGRET_MATCHING, HEAD_SOFTMAX_RM = 0, 1, 2, 3
 
@@ -28,8 +28,8 @@ class SpiralError(RuntimeError):
 
 
 class PhiloxConfig(C.Structure):
-    _fields_ = [("seed", C.c_uint64), ("mode", C.c_int32), ("threads_per_block", C.c_int32),
-                ("blocks_per_grid", C.c_int32), ("reserved", C.c_int32)]
+    _fields_ = [("seed", C.c_uint64), ("offset", C.c_uint64), ("mode", C.c_int32), ("threads_per_block", C.c_int32),
+                ("blocks_per_grid", C.c_int32), ("rows_per_block", C.c_int32)]
 
 
 class DeviceInfo(C.Structure):
@@ -54,7 +54,9 @@ SIGNATURES = {
     "sp_row_ops": (C.c_int, [_P] * 8 + [_I64, _I64, _U32, _P]),
     "sp_row_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _I64, _I32, _P]),
     "sp_row_map_i32": (C.c_int, [C.c_int, _P, _P, _I64, _I64, _P]),
-    "sp_row_sample": (C.c_int, [C.c_int, _P, _P, C.POINTER(PhiloxConfig), _P, _P, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_row_sample": (C.c_int, [C.c_int, _P, _P, C.POINTER(PhiloxConfig), _P, _P, _P, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_row_get_prob": (C.c_int, [C.c_int, _P, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_row_binarize": (C.c_int, [_P, _P, _I64, _I64, C.c_uint32, _P]),
     "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
     "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),
     "sp_reduce_workspace_bytes": (C.c_int64, []),

@@ -110,28 +110,36 @@ def argmax(x):
 
 
 def philox(mode=_lib.PHILOX_BLOCK, seed=CONSTANT_SEED, threads_per_block=THREADS_PER_BLOCK,
-           blocks_per_grid=BLOCKS_PER_GRID):
+           blocks_per_grid=BLOCKS_PER_GRID, rows_per_block=0, offset=0):
     """The reference's device RNG: Philox4_32_10 seeded like `random.init {seed subsequence offset=0}`
-    (ml/primitives.spi:927,1014; corecuda/random.spi:22-32)."""
-    return PhiloxConfig(seed, mode, threads_per_block, blocks_per_grid, 0)
+    (ml/primitives.spi:927,1014; corecuda/random.spi:22-32).  `offset` = draws every thread's generator
+    has already handed out (a graph run keeps one state per thread across its sampling nodes)."""
+    return PhiloxConfig(seed, offset, mode, threads_per_block, blocks_per_grid, rows_per_block)
 
 
-def _sample(op, x, u=None, rng=None, mask_size=0, want_cdf=False, want_u=False):
+def _sample(op, x, u=None, rng=None, mask_size=0, want_cdf=False, want_u=False, want_prob=False, probs_out=None,
+            sample_out=None):
     rows, cols = _rows_cols(x)
-    probs = torch.empty_like(x)
-    sample = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device)
+    probs = torch.empty_like(x) if probs_out is None else probs_out
+    sample = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device) if sample_out is None else sample_out
     cdf = torch.empty_like(x) if want_cdf else None
     u_out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if want_u else None
+    prob = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if want_prob else None
     if (u is None) == (rng is None):
         raise ValueError("give exactly one of u (a tensor of uniforms in (0, 1]) and rng (a PhiloxConfig)")
+    if probs.shape != x.shape or sample.shape != x.shape[:-1]:
+        raise ValueError("the output tensors do not have the input's dimensions")
     check(lib.sp_row_sample(op, ptr(x, torch.float32, "x"), ptr(u, torch.float32, "u"),
-                            C.byref(rng) if rng is not None else None, ptr(probs), ptr(cdf), ptr(u_out), ptr(sample),
-                            rows, cols, mask_size, stream_ptr()))
+                            C.byref(rng) if rng is not None else None, ptr(probs, torch.float32, "probs"), ptr(cdf),
+                            ptr(u_out), ptr(sample, torch.int32, "sample"), ptr(prob), rows, cols, mask_size,
+                            stream_ptr()))
     res = (probs, sample)
     if want_cdf:
         res += (cdf,)
     if want_u:
         res += (u_out,)
+    if want_prob:
+        res += (prob,)
     return res
 
 
@@ -158,6 +166,42 @@ def regret_matching_and_discrete_sampling(x, u=None, rng=None, **kw):
 def masked_regret_matching_and_discrete_sampling(x, size, u=None, rng=None, **kw):
     """row_map_reduce local_masked_regret_matching_and_discrete_sampling (ml/primitives.spi:812-814)."""
     return _sample(_lib.ROW_MASKED_REGRET_MATCHING, x, u, rng, mask_size=size, **kw)
+
+
+_ROW_OPS = {"identity": _lib.ROW_IDENTITY, "softmax": _lib.ROW_SOFTMAX, "masked_softmax": _lib.ROW_MASKED_SOFTMAX,
+            "ln_l2": _lib.ROW_LN_L2, "regret_matching": _lib.ROW_REGRET_MATCHING,
+            "masked_regret_matching": _lib.ROW_MASKED_REGRET_MATCHING}
+
+
+def get_prob(x, action_id, op="identity", size=0):
+    """row_gather_reduce of `local_get_prob config action_id (zip probs j_tns)` (ml/primitives.spi:824-830):
+    the value of op(x) at column action_id[r] of every row, e.g. `get_policy_probs` of the CFR agent with
+    op="masked_regret_matching" (ml/cfr.spi:97-107)."""
+    rows, cols = _rows_cols(x)
+    if action_id.shape != x.shape[:-1]:
+        raise ValueError("one action id per row expected")
+    out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device)
+    check(lib.sp_row_get_prob(_ROW_OPS[op], ptr(x, torch.float32, "x"), ptr(action_id, torch.int32, "action_id"),
+                              ptr(out), rows, cols, size, stream_ptr()))
+    return out
+
+
+def get_action(x, u=None, rng=None, op="identity", size=0):
+    """The agents' `get_action` (ml/cem.spi:152-164, ml/cfr.spi:117-129): row_gather_reduce of a discrete
+    sample from op(x) together with the probability it was drawn with.  With `rng` the default stream is the
+    gather mapping (one row per thread).  Returns (prob, action_id)."""
+    if u is None and rng is None:
+        rng = philox(_lib.PHILOX_GATHER)
+    _, action, prob = _sample(_ROW_OPS[op], x, u, rng, mask_size=size, want_prob=True)
+    return prob, action
+
+
+def binarize(x, modulo):
+    """row_reduce local_binarize (ml/primitives.spi:817-821; layer head ml/layers.spi:439-446)."""
+    rows, cols = _rows_cols(x)
+    out = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device)   # holds the reference's u32
+    check(lib.sp_row_binarize(ptr(x, torch.float32, "x"), ptr(out), rows, cols, modulo, stream_ptr()))
+    return out
 
 
 def map(op, x, out=None):  # noqa: A001  (the reference's name, ml/primitives.spi:128)

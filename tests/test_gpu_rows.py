@@ -175,6 +175,54 @@ def test_row_ops_zero_probabilities_and_extreme_uniforms(P, cols):
     assert (out["argmax"] == orow.argmax(x)).all()
 
 
+@pytest.mark.parametrize("cols", [4, 12, 64, 256])
+def test_get_prob_get_action_binarize(P, cols):
+    """row_gather_reduce users (ml/cem.spi:152-164, ml/cfr.spi:97-129) and the binarize head."""
+    announce("get_prob / get_action / binarize cols=%d" % cols)
+    rng = np.random.default_rng(cols + 77)
+    rows = 301
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    ids = rng.integers(0, cols, size=rows).astype(np.int32)
+    size = max(1, cols // 2)
+    assert (host(P.get_prob(dev(x), dev(ids))) == orow.get_prob(x, ids)).all()
+    mrm = host(P.masked_regret_matching(dev(x), size))
+    assert (host(P.get_prob(dev(x), dev(ids), op="masked_regret_matching", size=size)) == orow.get_prob(mrm, ids)).all()
+    sm = host(P.softmax(dev(x)))
+    assert (host(P.get_prob(dev(x), dev(ids), op="softmax")) == orow.get_prob(sm, ids)).all()
+    bad = ids.copy(); bad[::2] = cols + 3; bad[1::4] = -1
+    got = host(P.get_prob(dev(x), dev(bad)))
+    assert (got[::2] == 0).all() and (got[1::4] == 0).all()
+    # sample + probability of the sample, from given uniforms and from the device stream
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    prob, action = P.get_action(dev(x), u=dev(u), op="masked_softmax", size=size)
+    msm = host(P.masked_softmax(dev(x), size))
+    assert (host(action) == orow.discrete_sampling(msm, u, order="wave")).all()
+    assert (host(prob) == orow.get_prob(msm, host(action))).all() and (host(prob) > 0).all()
+    if cols >= 4 and 256 % (cols // 4) == 0:
+        prob2, action2 = P.get_action(dev(x), op="masked_softmax", size=size)
+        u2 = ophilox.row_uniforms_gather(rows, cols)
+        assert (host(action2) == orow.discrete_sampling(msm, u2, order="wave")).all()
+        assert (host(prob2) == orow.get_prob(msm, host(action2))).all()
+    for modulo in (1, 7, 2 ** 31 - 1, 2 ** 32 - 1):
+        assert (host(P.binarize(dev(x), modulo)).view(np.uint32) == orow.binarize(x, modulo)).all()
+
+
+def test_layer_stream_uniforms(P):
+    """The uniforms a sampling node of a layer graph sees (ml/layers.spi:339-344), with a draw offset."""
+    from ml import _lib
+    announce("philox layer stream")
+    blocks, m, n = 6, 64, 64
+    x = dev(np.random.default_rng(3).standard_normal((blocks * m, n)).astype(np.float32))
+    for offset in (0, 16, 6):
+        rng = P.philox(_lib.PHILOX_LAYER, blocks_per_grid=blocks, rows_per_block=m, offset=offset)
+        _, _, u = P.softmax_and_discrete_sampling(x, rng=rng, want_u=True)
+        assert (host(u) == ophilox.row_uniforms_layer(blocks, m, n, offset=offset)).all()
+    # one block: the layer stream is the block-level stream
+    rng = P.philox(_lib.PHILOX_LAYER, blocks_per_grid=1, rows_per_block=blocks * m)
+    _, _, u = P.softmax_and_discrete_sampling(x, rng=rng, want_u=True)
+    assert (host(u) == ophilox.row_uniforms_block(blocks * m, n)).all()
+
+
 def test_sampling_edge_cases(P):
     announce("sampling edge cases")
     p = np.zeros((4, 8), dtype=np.float32)

@@ -159,3 +159,29 @@ def test_mlp_forward_composition():
     assert ((action >= 0) & (action < 3)).all()
     pol16, _, _ = layers.mlp_forward(x, ws, u=u, act_dtype="f16")
     assert gemm.rel_frobenius(pol16, policy) < 3e-3
+
+
+def test_binarize_and_get_prob_by_hand():
+    x = np.array([[0.5, -1.0, 0.0, 2.0], [-1, -1, -1, -1], [1, 1, 1, 1]], dtype=np.float32)
+    assert row_ops.binarize(x, 100).tolist() == [0b1001, 0, 0b1111]
+    assert row_ops.binarize(x, 4).tolist() == [0b1001 % 4, 0, 0b1111 % 4]
+    wide = np.ones((1, 40), dtype=np.float32)          # columns 32.. are shifted out
+    assert row_ops.binarize(wide, 2 ** 32 - 1).tolist() == [0]   # 0xFFFFFFFF mod 0xFFFFFFFF
+    assert row_ops.binarize(wide, 2 ** 31).tolist() == [2 ** 31 - 1]
+    p = np.array([[0.1, 0.2, 0.7], [0.3, 0.3, 0.4]], dtype=np.float32)
+    assert row_ops.get_prob(p, [2, 0]).tolist() == [np.float32(0.7), np.float32(0.3)]
+
+
+def test_layer_stream_reduces_to_block_stream_and_shifts_by_offset():
+    one_block = philox.row_uniforms_layer(1, 96, 64)
+    assert (one_block == philox.row_uniforms_block(96, 64)).all()
+    # every block restarts the row walk and uses its own 256 subsequences
+    u = philox.row_uniforms_layer(3, 32, 64)
+    want = philox.curand_uniform(philox.curand_words(philox.CONSTANT_SEED,
+                                                     np.repeat(np.arange(3), 32) * 256 + (np.tile(np.arange(32), 3) % 16) * 16,
+                                                     4 * (np.tile(np.arange(32), 3) // 16)))
+    assert (u == want).all()
+    # a node that starts 8 draws in sees what a fresh node sees two row-iterations later
+    fresh = philox.row_uniforms_layer(2, 64, 64)
+    later = philox.row_uniforms_layer(2, 32, 64, offset=philox.draws_per_sampling_node(32, 64))
+    assert (later.reshape(2, 32) == fresh.reshape(2, 64)[:, 32:]).all()
