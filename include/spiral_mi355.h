@@ -181,6 +181,13 @@ int sp_row_sample(int op, const float* x, const float* u, const sp_philox_t* phi
                   void* stream);
 
 /*
+ * u_out[r] = the uniform in (0, 1] that row r of a (rows, cols) sampling op draws from the stream
+ * `philox` describes: the reference's `random.init` + `random.uniform` (corecuda/random.spi:22-32,84)
+ * without the op around it, for callers that feed the uniforms to sp_mlp_forward or sp_row_ops.
+ */
+int sp_philox_uniforms(const sp_philox_t* philox, float* u_out, int64_t rows, int64_t cols, void* stream);
+
+/*
  * prob_out[r] = op(x)[r, action[r]]: `row_gather_reduce` of `local_get_prob` after an optional
  * (masked) softmax / regret matching (ml/primitives.spi:824-830; callers ml/cfr.spi:97-107).  The
  * reference asserts that the action id is a column of the row; here an id outside [0, cols) gives 0.

@@ -492,6 +492,12 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel_i32(const int* __restr
     }
 }
 
+// One thread per row: just the uniform the row would draw.
+__global__ __launch_bounds__(ROW_THREADS) void philox_uniforms_kernel(const RowArgs a) {
+    const long r = (long)blockIdx.x * ROW_THREADS + threadIdx.x;
+    if (r < a.rows) a.u_out[r] = reference_row_uniform(a, r);
+}
+
 // Lanes that share a row.  Up to 64 columns: one lane per 4 columns (rounded up to a power of two).
 // Up to 256 columns: 16 lanes (one DPP row), each holding one 4-column piece of every 64-column
 // chunk, so a wave works on 4 rows at once and no reduction leaves its DPP row.  Wider rows: the
@@ -580,6 +586,41 @@ struct RowKernelNames {
 
 using namespace sp;
 
+static int set_philox(RowArgs& a, const sp_philox_t* philox, int64_t rows, int64_t cols, const char* fn) {
+    if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_LAYER)
+        return fail(SP_ERR_ARG, "%s: unknown philox mode %d", fn, philox->mode);
+    const int64_t t = cols / 4;
+    if (philox->threads_per_block <= 0 || philox->threads_per_block % t != 0)
+        return fail(SP_ERR_ARG, "%s: threads_per_block (%d) must be a positive multiple of cols/4 (%lld)", fn,
+                    philox->threads_per_block, (long long)t);
+    if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
+        return fail(SP_ERR_ARG, "%s: blocks_per_grid must be positive", fn);
+    if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || rows % philox->rows_per_block != 0))
+        return fail(SP_ERR_ARG, "%s: rows_per_block (%d) must be positive and divide rows (%lld)", fn,
+                    philox->rows_per_block, (long long)rows);
+    a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
+    a.blocks = philox->blocks_per_grid; a.rows_per_block = philox->rows_per_block;
+    a.draw_offset = philox->offset;
+    return SP_OK;
+}
+
+extern "C" int sp_philox_uniforms(const sp_philox_t* philox, float* u_out, int64_t rows, int64_t cols, void* stream) {
+    SP_REQUIRE_PTR(u_out);
+    if (philox == nullptr) return fail(SP_ERR_NULL, "sp_philox_uniforms: philox is NULL");
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    RowArgs a{};
+    a.rows = rows; a.cols = (int)cols; a.u_out = u_out;
+    rc = set_philox(a, philox, rows, cols, __func__);
+    if (rc != SP_OK) return rc;
+    const long blocks = (rows + ROW_THREADS - 1) / ROW_THREADS;
+    if (blocks > 0x7fffffffL) return fail(SP_ERR_SHAPE, "sp_philox_uniforms: rows too large");
+    hipLaunchKernelGGL(philox_uniforms_kernel, dim3((unsigned)blocks), dim3(ROW_THREADS), 0, (hipStream_t)stream, a);
+    return check_launch(__func__);
+}
+
 extern "C" int sp_row_ops(const float* logits, const float* u, float* rowmax, float* rowsum, float* probs, float* cdf,
                           int32_t* argmax, int32_t* sample, int64_t rows, int64_t cols, uint32_t flags, void* stream) {
     (void)flags;
@@ -634,20 +675,8 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
     a.prob_out = prob_out;
     a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols; a.philox_mode = -1;
     if (philox != nullptr) {
-        if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_LAYER)
-            return fail(SP_ERR_ARG, "sp_row_sample: unknown philox mode %d", philox->mode);
-        const int64_t t = cols / 4;
-        if (philox->threads_per_block <= 0 || philox->threads_per_block % t != 0)
-            return fail(SP_ERR_ARG, "sp_row_sample: threads_per_block (%d) must be a positive multiple of cols/4 (%lld)",
-                        philox->threads_per_block, (long long)t);
-        if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
-            return fail(SP_ERR_ARG, "sp_row_sample: blocks_per_grid must be positive");
-        if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || rows % philox->rows_per_block != 0))
-            return fail(SP_ERR_ARG, "sp_row_sample: rows_per_block (%d) must be positive and divide rows (%lld)",
-                        philox->rows_per_block, (long long)rows);
-        a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
-        a.blocks = philox->blocks_per_grid; a.rows_per_block = philox->rows_per_block;
-        a.draw_offset = philox->offset;
+        rc = set_philox(a, philox, rows, cols, __func__);
+        if (rc != SP_OK) return rc;
     }
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }

@@ -1,29 +1,43 @@
 """Host surface of the dense layers (reference: ml/layers.spi, generated ml/layers.py).
 
-The reference builds a static graph (`matmul`, `relu`, `softmax`, ... ml/layers.spi:353-484) and
-interprets it inside one kernel with every node's output going through a global-memory workspace
-(graph_extract_, :181-252).  Here a dense stack with ReLU between layers and a row head is ONE
-fused kernel (sp_mlp_forward): activations never leave the compute unit.
+Two levels:
+
+* `mlp_forward`: a dense stack with ReLU between layers and a row head as ONE fused kernel
+  (sp_mlp_forward); activations never leave the compute unit.
+* the reference's static layer graph (ml/layers.spi:24-55): the same node constructors
+  (`input`, `weight`, `matmul`, `matmul_ensemble`, `tanh`/`sigmoid`/`relu`, `ln_l2`, `softmax`,
+  `regret_matching`, `argmax`, `discrete_sample`, `softmax_and_discrete_sample`, `masked_*`,
+  `binarize`, `copy`, `pair`, `apply`, `key_graph`), the same byte-arena layout (`create_model`,
+  `pass_calculate_partitions`: three arenas -- weights, workspace, weight adjoints -- every tensor at
+  a 16-byte aligned offset in depth-first order, :127-179 and corebase/partitionm.spi:53-67) so a
+  `model_ptrs` triple can be exchanged with code that lays the arenas out like the reference, and
+  `graph_run_host`, which runs every node through the C ABI.  The reference interprets the graph
+  inside one kernel (:181-252); here each node is one library call on the caller's stream, and a
+  relu-MLP with a sampling head collapses into the fused kernel when its shapes allow.
+
+A primed constructor of the reference (`softmax' out x`) is the underscore form here with a graph
+for `out` (`softmax_(out, x)`); every constructor also curries on its last argument so that
+`pipe(input(...), matmul((64, 64)), ln_l2, relu)` reads like the reference's `|>` chains.
 """
+import builtins
 import ctypes as C
+import itertools
 
 import torch
 
-from . import _lib
+from . import _console, _lib, matmul as _matmul, primitives as _prim
 from ._lib import check, lib, ptr, stream_ptr
 
 HEADS = {None: _lib.HEAD_NONE, "none": _lib.HEAD_NONE, "softmax": _lib.HEAD_SOFTMAX,
          "regret_matching": _lib.HEAD_REGRET_MATCHING, "softmax_regret_matching": _lib.HEAD_SOFTMAX_RM}
 
 
-def weight_init(out_features, in_features, std=0.1, dtype=torch.float16, generator=None, device="cuda"):
-    """`weight_init` (ml/layers.spi:460-463): N(0, std), std = 0.1 in the reference; stored
-    (out_features, in_features) like `weight (a, b)` (:467)."""
-    w = torch.randn((out_features, in_features), generator=generator, device=device, dtype=torch.float32) * std
-    return w.to(dtype)
+# ----------------------------------------------------------------------------------------------
+# fused dense stack
+# ----------------------------------------------------------------------------------------------
 
-
-def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None, mask_size=0, want_logits=False):
+def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None, mask_size=0, want_logits=False,
+                policy_out=None, action_out=None):
     """policy, action[, logits] = fused forward of relu-MLP + head + discrete sampling.
 
     x: (batch, in) f16/bf16; weights[i]: (out_i, in_i) of the same dtype (the B operand of A.B^T,
@@ -38,8 +52,11 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
             raise TypeError("weights[%d] must have the dtype of x" % i)
         assert w.shape[1] == dims[i], "The K dimension of the A and B tensors must match."
     batch = x.shape[0]
-    policy = torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device)
-    action = torch.empty((batch,), dtype=torch.int32, device=x.device) if u is not None else None
+    policy = policy_out if policy_out is not None else \
+        torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device)
+    action = action_out
+    if action is None and u is not None:
+        action = torch.empty((batch,), dtype=torch.int32, device=x.device)
     logits = torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device) if want_logits else None
     wp = (C.c_void_p * n)(*[ptr(w, name="weights[%d]" % i) for i, w in enumerate(weights)])
     bp = None
@@ -48,6 +65,927 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
                                 for i, b in enumerate(biases)])
     dp = (C.c_int32 * (n + 1))(*dims)
     check(lib.sp_mlp_forward(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, bp, dp, ptr(u, torch.float32, "u"),
-                             ptr(policy), ptr(action), ptr(logits), batch, HEADS[head], mask_size, stream_ptr()))
+                             ptr(policy, torch.float32, "policy_out"), ptr(action, torch.int32, "action_out"),
+                             ptr(logits), batch, HEADS[head], mask_size, stream_ptr()))
     out = (policy, action)
     return out + (logits,) if want_logits else out
+
+
+# ----------------------------------------------------------------------------------------------
+# the layer graph (ml/layers.spi:6-55)
+# ----------------------------------------------------------------------------------------------
+
+def weight_id():
+    return 0
+
+
+def workspace_id():
+    """For input layers and intermediates."""
+    return 1
+
+
+def weight_adjoint_id():
+    return 2
+
+
+def num_spaces():
+    return 3
+
+
+THREADS_PER_BLOCK = 256
+_blocks_per_grid = None
+_generator = {}
+
+DTYPES = {"float": torch.float32, "f32": torch.float32, "int": torch.int32, "i32": torch.int32,
+          "uint": torch.int32,   # u32 bit patterns; torch has no arithmetic-free u32 views on all builds
+          "f16": torch.float16, "bf16": torch.bfloat16}
+
+
+def _dtype(t):
+    return DTYPES[t] if isinstance(t, str) else t
+
+
+def blocks_per_grid():
+    """The leading dimension every workspace tensor of a graph must have (ml/layers.spi:81-106).  In
+    the reference it is the number of SMs, because block b of its one kernel owns slice b; here it
+    is a free batch split, by default the number of compute units."""
+    global _blocks_per_grid
+    if _blocks_per_grid is None:
+        _blocks_per_grid = _lib.device_info()["compute_units"] if torch.cuda.is_available() else 24
+    return _blocks_per_grid
+
+
+def set_blocks_per_grid(n):
+    global _blocks_per_grid
+    _blocks_per_grid = int(n)
+
+
+def set_random_seed(seed=_prim.CONSTANT_SEED, device="cuda"):
+    """`cupy.set_random_seed` (corecuda/cupy.spi:9): reseeds the generator the initialisers draw from."""
+    g = torch.Generator(device=device)
+    g.manual_seed(seed)
+    _generator[torch.device(device).type] = g
+    return g
+
+
+def _gen(device):
+    key = torch.device(device).type
+    return _generator[key] if key in _generator else set_random_seed(device=device)
+
+
+class TensorSpec:
+    """Dimensions and element type of one tensor: the `D_D dim` leaf of `dim_of` (ml/layers.spi:56-58)."""
+    __slots__ = ("dim", "dtype")
+
+    def __init__(self, dim, dtype):
+        self.dim, self.dtype = tuple(int(d) for d in dim), dtype
+
+    def __eq__(self, o):
+        return isinstance(o, TensorSpec) and self.dim == o.dim
+
+    def __repr__(self):
+        return "TensorSpec(%r, %s)" % (self.dim, self.dtype)
+
+    @property
+    def nbytes(self):
+        n = 1
+        for d in self.dim:
+            n *= d
+        return n * torch.empty((), dtype=self.dtype).element_size()
+
+
+class Graph:
+    """Base of the node types of `union rec graph t` (ml/layers.spi:24-55).  Nodes compare by identity."""
+
+
+class Layer(Graph):
+    def __init__(self, space_id, dim, init=None, dtype="float"):
+        self.space_id, self.spec, self.init = space_id, TensorSpec(dim, _dtype(dtype)), init
+
+
+class KeyGraph(Graph):
+    def __init__(self, key, x):
+        self.key, self.x = key, x
+
+
+class KeyScalar(Graph):
+    def __init__(self, key):
+        self.key = key
+
+
+class Apply(Graph):
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+
+
+class Pair(Graph):
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+
+
+class Zip(Graph):
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+
+
+class Fst(Graph):
+    def __init__(self, x):
+        self.x = x
+
+
+class Snd(Graph):
+    def __init__(self, x):
+        self.x = x
+
+
+class BlockMap(Graph):
+    def __init__(self, f, a, out=None):
+        self.f, self.a, self.out = f, a, out
+
+
+class BlockRowMap(Graph):
+    def __init__(self, f, a, out=None, size=0):
+        self.f, self.a, self.out, self.size = f, a, out, size
+
+
+class BlockRowReduce(Graph):
+    def __init__(self, f, a, out=None, arg=0):
+        self.f, self.a, self.out, self.arg = f, a, out, arg
+
+
+class BlockRowMapReduce(Graph):
+    def __init__(self, f, a, out=None, size=0):
+        self.f, self.a, self.out, self.size = f, a, out, size
+
+
+class BlockMatmul(Graph):
+    def __init__(self, a, b):
+        self.a, self.b = a, b
+
+
+_REDUCE_DTYPE = {"argmax": torch.int32, "discrete_sample": torch.int32, "binarize": torch.int32, "max": None}
+
+
+def _row_dtype(t):
+    return torch.float32 if t in (torch.float16, torch.bfloat16) else t
+
+
+def get_dim_pair(h, x):
+    """Top-level dimensions of a node, memoised in `h` (ml/layers.spi:75-125): a TensorSpec or a pair of
+    them.  The asserts are the reference's."""
+    if x in h:
+        return h[x]
+    q_msg = "The batch dimension in the %s node needs to equal the number of blocks per grid."
+
+    def check_out(spec, out):
+        if out is not None:
+            assert spec == get_dim_pair(h, out), \
+                "The dimensions coming from the input and the dimensions of the output have to match."
+
+    if isinstance(x, BlockRowMapReduce):
+        a = get_dim(h, x.a)
+        q, w, e = a.dim
+        assert q == blocks_per_grid(), q_msg % "row reduce"
+        # the row heads compute and store f32 whatever the stack above them is stored in
+        r = (TensorSpec((q, w, e), _row_dtype(a.dtype)), TensorSpec((q, w), torch.int32))
+        if x.out is not None:
+            oa, ob = get_dim_pair(h, x.out)
+            assert r[0] == oa, "The dimensions coming from the input and the dimensions of the first output have to match."
+            assert r[1] == ob, "The dimensions coming from the input and the dimensions of the second output have to match."
+    elif isinstance(x, Pair):
+        r = (get_dim_pair(h, x.a), get_dim_pair(h, x.b))
+    elif isinstance(x, Zip):
+        a, b = get_dim(h, x.a), get_dim(h, x.b)
+        assert a == b, "The dimensions of the two inputs to the Zip node have to be equal."
+        r = a
+    elif isinstance(x, BlockMap):
+        r = get_dim(h, x.a)
+        assert r.dim[0] == blocks_per_grid(), q_msg % "map"
+        check_out(r, x.out)
+    elif isinstance(x, BlockRowMap):
+        r = get_dim(h, x.a)
+        assert r.dim[0] == blocks_per_grid(), q_msg % "row map"
+        check_out(r, x.out)
+    elif isinstance(x, BlockRowReduce):
+        a = get_dim(h, x.a)
+        q, w, _ = a.dim
+        assert q == blocks_per_grid(), q_msg % "row reduce"
+        r = TensorSpec((q, w), _REDUCE_DTYPE[x.f] or a.dtype)
+        check_out(r, x.out)
+    elif isinstance(x, BlockMatmul):
+        a = get_dim(h, x.a)
+        q, m, k = a.dim
+        assert q == blocks_per_grid(), q_msg % "matmul"
+        n, k2 = get_dim(h, x.b).dim
+        assert k == k2, "The inner dimensions of the matrix multiplication node have to be equal."
+        r = TensorSpec((q, m, n), a.dtype)
+    elif isinstance(x, Layer):
+        r = x.spec
+    elif isinstance(x, KeyGraph):
+        r = get_dim_pair(h, x.x)
+    elif isinstance(x, Apply):
+        a = get_dim(h, x.a)
+        r = TensorSpec(a.dim[1:], a.dtype)
+    elif isinstance(x, Fst):
+        r = get_dim_pair(h, x.x)[0]
+    elif isinstance(x, Snd):
+        r = get_dim_pair(h, x.x)[1]
+    else:
+        raise TypeError("Cannot get the dimension of %r." % (x,))
+    h[x] = r
+    return r
+
+
+def get_dim(h, x):
+    r = get_dim_pair(h, x)
+    if not isinstance(r, TensorSpec):
+        raise TypeError("The node holds a pair of tensors, not one tensor.")
+    return r
+
+
+def _align(s):
+    """`partitionm.align` (corebase/partitionm.spi:3-4)."""
+    return (s + 15) // 16 * 16
+
+
+class Offsets:
+    """Where one tensor lives in its arena: `partitionm.offsets` (corebase/partitionm.spi:13-16)."""
+    __slots__ = ("spec", "offset")
+
+    def __init__(self, spec, offset):
+        self.spec, self.offset = spec, offset
+
+
+def pass_calculate_partitions(x, dims):
+    """Byte offsets of every layer and node output (ml/layers.spi:127-179): depth-first, inputs before the
+    node's own output, each tensor aligned to 16 bytes (corebase/partitionm.spi:53-67); node outputs without an
+    explicit `out` graph go to the workspace.  Returns [{partition: {node: offsets}, size}] per arena."""
+    h_data = [dict() for _ in range(num_spaces())]
+    ends = [0] * num_spaces()
+    seen = set()
+
+    def place(sid, spec):
+        if isinstance(spec, TensorSpec):
+            start = _align(ends[sid])
+            ends[sid] = start + spec.nbytes
+            return Offsets(spec, start)
+        return tuple(place(sid, s) for s in spec)
+
+    def g(k, out):
+        if out is not None:
+            f(out)
+        else:
+            h_data[workspace_id()][k] = place(workspace_id(), get_dim_pair(dims, k))
+
+    def f(k):
+        if k in seen:
+            return
+        seen.add(k)
+        if isinstance(k, (BlockMap, BlockRowMap, BlockRowReduce, BlockRowMapReduce)):
+            f(k.a)
+            g(k, k.out)
+        elif isinstance(k, BlockMatmul):
+            f(k.a)
+            f(k.b)
+            g(k, None)
+        elif isinstance(k, (Pair, Zip, Apply)):
+            f(k.a)
+            f(k.b)
+        elif isinstance(k, (Fst, Snd, KeyGraph)):
+            f(k.x)
+        elif isinstance(k, Layer):
+            h_data[k.space_id][k] = place(k.space_id, k.spec)
+        elif isinstance(k, KeyScalar):
+            pass
+        else:
+            raise TypeError("unknown graph node %r" % (k,))
+
+    f(x)
+    return [{"partition": h, "size": e} for h, e in zip(h_data, ends)]
+
+
+def create_graph_data(partitions, device="cuda"):
+    """One uint8 array per arena (ml/layers.spi:173-179)."""
+    return [dict(p, array=torch.empty(p["size"], dtype=torch.uint8, device=device)) for p in partitions]
+
+
+class Model:
+    """`nominal model t = {graph; dims; data}` (ml/layers.spi:60-65)."""
+
+    def __init__(self, graph, dims, data):
+        self.graph, self.dims, self.data = graph, dims, data
+
+
+def create_model(graph, device="cuda"):
+    """ml/layers.spi:486-490."""
+    dims = {}
+    return Model(graph, dims, create_graph_data(pass_calculate_partitions(graph, dims), device))
+
+
+def model_to_model_ptrs(model):
+    """The three arenas, weights / workspace / weight adjoints (ml/layers.spi:495)."""
+    return tuple(x["array"] for x in model.data)
+
+
+def model_ptrs_to_model(graph, ptrs):
+    """Rebuild a model around arenas laid out elsewhere (ml/layers.spi:496-502)."""
+    dims = {}
+    parts = pass_calculate_partitions(graph, dims)
+    for p, a in zip(parts, ptrs):
+        assert a.dtype == torch.uint8 and a.numel() >= p["size"], \
+            "The length of the partition has to be less than or equal to the length of the base array."
+    return Model(graph, dims, [dict(p, array=a) for p, a in zip(parts, ptrs)])
+
+
+def _from_offsets(array, o):
+    """`partitionm.from_partition_offsets` (corebase/partitionm.spi:96-105)."""
+    if isinstance(o, Offsets):
+        return array[o.offset:o.offset + o.spec.nbytes].view(o.spec.dtype).view(o.spec.dim)
+    return tuple(_from_offsets(array, x) for x in o)
+
+
+class LayerState:
+    """`nominal layer_state = {rng}` (ml/layers.spi:19-22).  The reference seeds one Philox generator per
+    thread for a whole graph run (:339-344); `draws` counts what each of them has handed out so far."""
+
+    def __init__(self, seed=_prim.CONSTANT_SEED):
+        self.seed, self.draws = seed, 0
+
+    def rng(self, q, w, cols):
+        cfg = _prim.philox(_lib.PHILOX_LAYER, seed=self.seed, threads_per_block=THREADS_PER_BLOCK, blocks_per_grid=q,
+                           rows_per_block=w, offset=self.draws)
+        rows_per_iteration = THREADS_PER_BLOCK // (cols // 4)
+        self.draws += 4 * ((w + rows_per_iteration - 1) // rows_per_iteration)
+        return cfg
+
+
+_MAPS = ("tanh", "sigmoid", "relu", "copy")
+_ROW_MAPS = ("ln_l2", "softmax", "regret_matching", "masked_softmax", "masked_regret_matching", "identity")
+_ROW_MAP_REDUCES = {"softmax_and_discrete_sample": _lib.ROW_SOFTMAX,
+                    "masked_softmax_and_discrete_sample": _lib.ROW_MASKED_SOFTMAX,
+                    "regret_matching_and_discrete_sample": _lib.ROW_REGRET_MATCHING,
+                    "masked_regret_matching_and_discrete_sample": _lib.ROW_MASKED_REGRET_MATCHING}
+
+
+def _flat(t):
+    return t.reshape(-1, t.shape[-1])
+
+
+def graph_extract_(layer_state, model, indices):
+    """ml/layers.spi:181-252.  With a layer state the nodes are computed on the way; without one the
+    tensors are only looked up."""
+    data = model.data
+
+    def extract_current(node):
+        for x in data:
+            if node in x["partition"]:
+                return _from_offsets(x["array"], x["partition"][node])
+        raise KeyError("Cannot find the offset in the dictionaries for node %r." % (node,))
+
+    def try_out(node):
+        return loop(node.out) if node.out is not None else extract_current(node)
+
+    def loop(graph):
+        if isinstance(graph, BlockMap):
+            out = try_out(graph)
+            if layer_state is not None:
+                _prim.map(graph.f, loop(graph.a), out)
+            return out
+        if isinstance(graph, BlockRowMap):
+            out = try_out(graph)
+            if layer_state is not None:
+                a = loop(graph.a)
+                _prim._row_map(_prim._ROW_OPS[graph.f], _flat(a), _flat(out), graph.size)
+            return out
+        if isinstance(graph, BlockRowReduce):
+            out = try_out(graph)
+            if layer_state is not None:
+                a = loop(graph.a)
+                if graph.f == "argmax":
+                    _prim.row_ops(_flat(a), want=("argmax",), into={"argmax": out.reshape(-1)})
+                elif graph.f == "max":
+                    _prim.row_ops(_flat(a), want=("rowmax",), into={"rowmax": out.reshape(-1)})
+                elif graph.f == "binarize":
+                    _prim.binarize(_flat(a), graph.arg, out=out.reshape(-1))
+                else:   # discrete_sample
+                    q, w, cols = a.shape
+                    _prim._sample(_lib.ROW_IDENTITY, _flat(a), rng=layer_state.rng(q, w, cols), want_probs=False,
+                                  sample_out=out.reshape(-1))
+            return out
+        if isinstance(graph, BlockRowMapReduce):
+            out_map, out_reduce = try_out(graph)
+            if layer_state is not None:
+                a = loop(graph.a)
+                q, w, cols = a.shape
+                _prim._sample(_ROW_MAP_REDUCES[graph.f], _flat(a), rng=layer_state.rng(q, w, cols),
+                              mask_size=graph.size, probs_out=_flat(out_map), sample_out=out_reduce.reshape(-1))
+            return out_map, out_reduce
+        if isinstance(graph, BlockMatmul):
+            a, b, out = loop(graph.a), loop(graph.b), extract_current(graph)
+            if layer_state is not None:
+                # matmul_tf32' false true 1 a b 0 out (ml/layers.spi:227-240)
+                _matmul.matmul_abt(_flat(a), b, c=_flat(out), alpha=1.0, beta=0.0)
+            return out
+        if isinstance(graph, (Zip, Pair)):
+            return loop(graph.a), loop(graph.b)
+        if isinstance(graph, Fst):
+            return loop(graph.x)[0]
+        if isinstance(graph, Snd):
+            return loop(graph.x)[1]
+        if isinstance(graph, Layer):
+            return extract_current(graph)
+        if isinstance(graph, Apply):
+            return loop(graph.a)[loop(graph.b)]
+        if isinstance(graph, KeyGraph):
+            return loop(graph.x)
+        if isinstance(graph, KeyScalar):
+            if graph.key not in indices:
+                raise KeyError("Cannot extract the node for the graph due to the missing (scalar) key in the "
+                               "environment.")
+            return indices[graph.key]
+        raise TypeError("unknown graph node %r" % (graph,))
+
+    return loop(model.graph)
+
+
+def graph_extract(model, indices=None):
+    """Extracts the tensor at the top level node (ml/layers.spi:255)."""
+    return graph_extract_(None, model, indices or {})
+
+
+def graph_run(model, ls, indices):
+    """ml/layers.spi:260."""
+    return graph_extract_(ls, model, indices)
+
+
+def extract_layers_(model, space_id=-1, key=None):
+    """All `Layer` nodes of one arena (-1: of all), or the graphs under `key_graph key`, as tensors, in
+    graph order (ml/layers.spi:268-307)."""
+    found, seen = [], set()
+
+    def f(k):
+        if k in seen:
+            return
+        seen.add(k)
+        if isinstance(k, (BlockMap, BlockRowMap, BlockRowReduce, BlockRowMapReduce)):
+            f(k.a)
+            if k.out is not None:
+                f(k.out)
+        elif isinstance(k, (BlockMatmul, Apply, Pair, Zip)):
+            f(k.a)
+            f(k.b)
+        elif isinstance(k, (Fst, Snd)):
+            f(k.x)
+        elif isinstance(k, Layer):
+            if key is None and (space_id == -1 or space_id == k.space_id):
+                found.append((k.space_id, graph_extract(Model(k, model.dims, model.data)), k.init))
+        elif isinstance(k, KeyGraph):
+            if key is not None and k.key == key:
+                found.append(graph_extract(Model(k.x, model.dims, model.data)))
+            else:
+                f(k.x)
+
+    f(model.graph)
+    return found
+
+
+def extract_layers(model):
+    return extract_layers_(model, -1)
+
+
+def pass_init(model):
+    """Initializes the layers on the host (ml/layers.spi:313)."""
+    for _, t, init in extract_layers(model):
+        if init is not None:
+            init(t)
+
+
+def _format(t, limit=100):
+    if isinstance(t, tuple):
+        return ", ".join(_format(x, limit) for x in t)
+    return _console.format_tensor(limit, t.detach().cpu().numpy())
+
+
+def print_layers(model, write=print):
+    for _, t, _ in extract_layers(model):
+        write(_format(t))
+
+
+def print_weights(model, write=print):
+    for _, t, _ in extract_layers_(model, weight_id()):
+        write(_format(t))
+
+
+def key_extract_list(model, key):
+    return extract_layers_(model, key=key)
+
+
+def key_extract(model, key):
+    """The tensor under `key_graph key` (ml/layers.spi:325-330)."""
+    found = key_extract_list(model, key)
+    if not found:
+        raise KeyError("Cannot find the input tensor with the given key.")
+    if len(found) > 1:
+        raise KeyError("More than one tensor with the given key found.")
+    return found[0]
+
+
+def create_layer_state(seed=_prim.CONSTANT_SEED):
+    return LayerState(seed)
+
+
+def graph_run_device(model, ls, indices):
+    graph_run(model, ls, indices)
+
+
+def _fused_plan(model):
+    """A `matmul -> relu -> ... -> matmul -> head` chain over 16-bit tensors that sp_mlp_forward can run:
+    returns (input node, [weight nodes], head node) or None."""
+    top = model.graph
+    head_ops = {"softmax_and_discrete_sample": "softmax", "masked_softmax_and_discrete_sample": "softmax",
+                "regret_matching_and_discrete_sample": "regret_matching",
+                "masked_regret_matching_and_discrete_sample": "regret_matching"}
+    if not isinstance(top, BlockRowMapReduce) or top.f not in head_ops:
+        return None
+    weights, node = [], top.a
+    while True:
+        if not isinstance(node, BlockMatmul) or not isinstance(node.b, Layer):
+            return None
+        weights.append(node.b)
+        node = node.a
+        if isinstance(node, BlockMap) and node.f == "relu" and node.out is None:
+            node = node.a
+            continue
+        break
+    while isinstance(node, KeyGraph):
+        node = node.x
+    if not isinstance(node, Layer):
+        return None
+    weights.reverse()
+    dims = [node.spec.dim[-1]] + [w.spec.dim[0] for w in weights]
+    ok = node.spec.dtype in (torch.float16, torch.bfloat16) and all(w.spec.dtype == node.spec.dtype for w in weights)
+    ok = ok and builtins.max(dims) <= 256   # `max` is a node constructor in this module and dims[0] % 16 == 0 and all(d % 32 == 0 for d in dims[1:-1]) and dims[-1] <= 64
+    return (node, weights, top, head_ops[top.f]) if ok else None
+
+
+def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True):
+    """Runs the graph for every combination of the key indices in `sizes`, e.g. {"ensemble": 16}
+    (ml/layers.spi:336-344).  Uniforms come from the reference's per-thread Philox streams."""
+    ls = create_layer_state(seed)
+    sizes = sizes or {}
+    plan = _fused_plan(model) if fuse and not sizes else None
+    if plan is not None:
+        x_node, w_nodes, top, head = plan
+        x = graph_extract(Model(x_node, model.dims, model.data))
+        ws = [graph_extract(Model(w, model.dims, model.data)) for w in w_nodes]
+        probs, action = graph_extract(model)
+        q, w, cols = probs.shape
+        u = _prim.philox_uniforms(ls.rng(q, w, cols), q * w, cols)
+        mlp_forward(_flat(x), ws, head=head, u=u, mask_size=top.size, policy_out=_flat(probs),
+                    action_out=action.reshape(-1))
+        return
+    keys = list(sizes)
+    for combo in itertools.product(*[range(sizes[k]) for k in keys]):
+        graph_run_device(model, ls, dict(zip(keys, combo)))
+
+
+# ---- node constructors (ml/layers.spi:346-484) ------------------------------------------------
+
+def _curried(f):
+    """f(args..., x) -> also callable without x, giving the function of x (for `pipe`)."""
+    def g(*args):
+        if args and isinstance(args[-1], Graph):
+            return f(*args)
+        return lambda x: f(*(args + (x,)))
+    g.__name__, g.__doc__ = f.__name__, f.__doc__
+    return g
+
+
+def pipe(x, *fs):
+    """x |> f1 |> f2 ..."""
+    for f in fs:
+        x = f(x)
+    return x
+
+
+def tanh(x):
+    return BlockMap("tanh", x)
+
+
+def sigmoid(x):
+    return BlockMap("sigmoid", x)
+
+
+def relu(x):
+    """relu = max 0 (ml/layers.spi:355)."""
+    return BlockMap("relu", x)
+
+
+@_curried
+def max_(out, x):
+    return BlockRowReduce("max", x, out)
+
+
+def max(x):  # noqa: A001  (the reference's name, ml/layers.spi:361)
+    return BlockRowReduce("max", x)
+
+
+def ln_l2(x):
+    return BlockRowMap("ln_l2", x)
+
+
+def argmax(x):
+    return BlockRowReduce("argmax", x)
+
+
+@_curried
+def softmax_(out, x):
+    return BlockRowMap("softmax", x, out)
+
+
+def softmax(x):
+    return BlockRowMap("softmax", x)
+
+
+@_curried
+def regret_matching_(out, x):
+    return BlockRowMap("regret_matching", x, out)
+
+
+def regret_matching(x):
+    return BlockRowMap("regret_matching", x)
+
+
+@_curried
+def discrete_sample_(out, x):
+    return BlockRowReduce("discrete_sample", x, out)
+
+
+def discrete_sample(x):
+    return BlockRowReduce("discrete_sample", x)
+
+
+@_curried
+def softmax_and_discrete_sample_(out, x):
+    return BlockRowMapReduce("softmax_and_discrete_sample", x, out)
+
+
+def softmax_and_discrete_sample(x):
+    return BlockRowMapReduce("softmax_and_discrete_sample", x)
+
+
+@_curried
+def copy_(out, x):
+    return BlockMap("copy", x, out)
+
+
+def copy(x):
+    return BlockMap("copy", x)
+
+
+@_curried
+def masked_softmax_(size, out, x):
+    return BlockRowMap("masked_softmax", x, out, size)
+
+
+@_curried
+def masked_softmax(size, x):
+    return BlockRowMap("masked_softmax", x, None, size)
+
+
+@_curried
+def masked_regret_matching_(size, out, x):
+    return BlockRowMap("masked_regret_matching", x, out, size)
+
+
+@_curried
+def masked_regret_matching(size, x):
+    return BlockRowMap("masked_regret_matching", x, None, size)
+
+
+@_curried
+def masked_softmax_and_discrete_sample_(size, out, x):
+    return BlockRowMapReduce("masked_softmax_and_discrete_sample", x, out, size)
+
+
+@_curried
+def masked_softmax_and_discrete_sample(size, x):
+    return BlockRowMapReduce("masked_softmax_and_discrete_sample", x, None, size)
+
+
+@_curried
+def binarize_(modulo, out, x):
+    return BlockRowReduce("binarize", x, out, modulo)
+
+
+@_curried
+def binarize(modulo, x):
+    return BlockRowReduce("binarize", x, None, modulo)
+
+
+def key_scalar(key):
+    return KeyScalar(key)
+
+
+def key_graph(key, x):
+    return KeyGraph(key, x)
+
+
+def apply(b, a):  # noqa: A001  (the reference's name, ml/layers.spi:450)
+    """Index the leading dimension of `a` with the run-time value of key `b`."""
+    return Apply(a, key_scalar(b))
+
+
+def pair(a, b):
+    return Pair(a, b)
+
+
+def fst_(x):
+    return Fst(x)
+
+
+def snd_(x):
+    return Snd(x)
+
+
+def layer(space_id, dim, init=None, dtype="float"):
+    return Layer(space_id, dim, init, dtype)
+
+
+tensor = layer
+
+
+def init_const(t, v):
+    t.fill_(v)
+
+
+def init_zero(t):
+    t.zero_()
+
+
+def weight_init(t, std=0.1):
+    """`weight_init` (ml/layers.spi:460-463): N(0, 0.1) in the current source."""
+    t.copy_(torch.randn(t.shape, generator=_gen(t.device), device=t.device, dtype=torch.float32) * std)
+
+
+def weight_(dim, init, dtype="float"):
+    return Layer(weight_id(), dim, init, dtype)
+
+
+def weight(dim, dtype="float"):
+    return weight_(dim, weight_init, dtype)
+
+
+@_curried
+def matmul(ba, x):
+    """`matmul (in, out) x = BlockMatmul(x, weight (out, in))` (ml/layers.spi:467): the weight is stored
+    (out_features, in_features) row-major, the B operand of A.B^T."""
+    b, a = ba
+    return BlockMatmul(x, weight((a, b), _input_dtype(x)))
+
+
+@_curried
+def matmul_ensemble(cba, x):
+    """E weight matrices (E, out, in) under the key "weights", indexed by the run-time key "ensemble"
+    (ml/layers.spi:468-471)."""
+    c, b, a = cba
+    weights = key_graph("weights", Layer(weight_id(), (c, a, b), weight_init, _input_dtype(x)))
+    return BlockMatmul(x, apply("ensemble", weights))
+
+
+def _input_dtype(x):
+    return get_dim({}, x).dtype
+
+
+def input_(dim, dtype="float"):
+    """Creates a layer in the workspace.  Doesn't initialize it (ml/layers.spi:481)."""
+    return Layer(workspace_id(), dim, None, dtype)
+
+
+def input(key, dim, dtype="float"):  # noqa: A001  (the reference's name, ml/layers.spi:482-484)
+    return key_graph(key, input_(dim, dtype))
+
+
+# ----------------------------------------------------------------------------------------------
+# the reference's self-tests (ml/layers.spi:510-668), same files, same text format
+# ----------------------------------------------------------------------------------------------
+
+def _redirect(root, name):
+    import os
+    d = os.path.join(root, name)
+    os.makedirs(d, exist_ok=True)
+    return open(os.path.join(d, "layers.txt"), "w")
+
+
+def _fill_normal(t):
+    t.copy_(torch.randn(t.shape, generator=_gen(t.device), device=t.device, dtype=torch.float32))
+
+
+def test1(root="test_text_outputs/layers/"):
+    """Tests whether randomly initializing the params of the graph works."""
+    set_random_seed()
+    with _redirect(root, "test1") as f:
+        w = lambda s: f.write(s + "\n")
+        graph = pipe(input("input", (blocks_per_grid(), 1, 4)), matmul((4, 4)), tanh, matmul((4, 4)), tanh,
+                     matmul((4, 2)), tanh)
+        model = create_model(graph)
+        for x in model.data:
+            x["array"].zero_()
+        w("---")
+        print_weights(model, w)
+        pass_init(model)
+        w("Done initing.")
+        print_weights(model, w)
+    return model
+
+
+def test2(root="test_text_outputs/layers/"):
+    """Tests whether extracting the inputs of the graph works.  Also randomly inits them."""
+    set_random_seed()
+    with _redirect(root, "test2") as f:
+        w = lambda s: f.write(s + "\n")
+        graph = pipe(input("input", (blocks_per_grid(), 1, 2)), matmul((2, 4)), tanh, matmul((4, 4)), tanh,
+                     matmul((4, 2)), tanh)
+        model = create_model(graph)
+        w("---")
+        pass_init(model)
+        w("Here are the weight matrices.")
+        print_weights(model, w)
+        w("Here is the input tensor.")
+        x = key_extract(model, "input")
+        _fill_normal(x)
+        w(_format(x))
+    return model
+
+
+def test3(root="test_text_outputs/layers/"):
+    """Tests running a feedforward model which outputs the sampling indices."""
+    set_random_seed()
+    with _redirect(root, "test3") as f:
+        w = lambda s: f.write(s + "\n")
+        graph = pipe(input("input", (blocks_per_grid(), 64, 64)), matmul((64, 64)), ln_l2, relu, matmul((64, 64)),
+                     ln_l2, relu, matmul((64, 64)), softmax_and_discrete_sample)
+        model = create_model(graph)
+        pass_init(model)
+        w("Here are the weight matrices.")
+        print_weights(model, w)
+        x = key_extract(model, "input")
+        _fill_normal(x)
+        w(_format(x))
+        w("Here is the output tensor.")
+        graph_run_host(model, {})
+        w(_format(graph_extract(model, {})))
+        w("====")
+    return model
+
+
+def _ensemble_test(name, ensemble, size, deep, root):
+    set_random_seed()
+    with _redirect(root, name) as f:
+        w = lambda s: f.write(s + "\n")
+        q = blocks_per_grid()
+        out = pair(apply("ensemble", input("output_probs", (ensemble, q, 64, 64))),
+                   apply("ensemble", input("output_indices", (ensemble, q, 64), "int")))
+        x = pipe(input("input", (q, 64, 64)), matmul_ensemble((ensemble, 64, 64)))
+        if deep:
+            x = pipe(x, ln_l2, relu, matmul_ensemble((ensemble, 64, 64)), ln_l2, relu,
+                     matmul_ensemble((ensemble, 64, 64)))
+        graph = softmax_and_discrete_sample_(out, x) if size is None else \
+            masked_softmax_and_discrete_sample_(size, out, x)
+        model = create_model(graph)
+        pass_init(model)
+        if deep:
+            w("Here are the weight matrices.")
+            print_weights(model, w)
+        inp = key_extract(model, "input")
+        _fill_normal(inp)
+        if deep:
+            w(_format(inp))
+            w("Here is the output tensor.")
+        graph_run_host(model, {"ensemble": ensemble})
+        w(_format(key_extract(model, "output_indices"), limit=2 ** 31 - 1))
+    return model
+
+
+def test4(root="test_text_outputs/layers/"):
+    """Tests running a feedforward ensemble model which keeps around the sampling probabilities."""
+    return _ensemble_test("test4", 16, None, True, root)
+
+
+def test5(root="test_text_outputs/layers/"):
+    """... with masking."""
+    return _ensemble_test("test5", 4, 11, False, root)
+
+
+def main_body(root="test_text_outputs/layers/"):
+    test1(root)
+    test2(root)
+    test3(root)
+    test4(root)
+    test5(root)
+
+
+def main():
+    main_body()
+    torch.cuda.synchronize()
+    return 0

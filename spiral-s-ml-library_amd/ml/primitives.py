@@ -81,16 +81,18 @@ def exclusive_scan_sum(x, out=None):
     return _row_map(_lib.ROW_EXCLUSIVE_SCAN, x, out)
 
 
-def row_ops(logits, u=None, want=("rowmax", "rowsum", "probs", "cdf", "argmax", "sample")):
+def row_ops(logits, u=None, want=("rowmax", "rowsum", "probs", "cdf", "argmax", "sample"), into=None):
     """The fused pipeline of one pass over the logits: row max, sum of exp(x - max), softmax,
     inclusive prefix sum, argmax and inverse-CDF sampling (sp_row_ops).  Returns a dict with the
-    requested outputs."""
+    requested outputs; `into` may hold preallocated tensors for some of them."""
     rows, cols = _rows_cols(logits)
     lead = logits.shape[:-1]
     dev = logits.device
     out = {}
     for name in want:
-        if name in ("probs", "cdf"):
+        if into is not None and name in into:
+            out[name] = into[name]
+        elif name in ("probs", "cdf"):
             out[name] = torch.empty_like(logits)
         elif name in ("rowmax", "rowsum"):
             out[name] = torch.empty(lead, dtype=torch.float32, device=dev)
@@ -117,20 +119,31 @@ def philox(mode=_lib.PHILOX_BLOCK, seed=CONSTANT_SEED, threads_per_block=THREADS
     return PhiloxConfig(seed, offset, mode, threads_per_block, blocks_per_grid, rows_per_block)
 
 
+def philox_uniforms(rng, rows, cols, out=None):
+    """The uniform each of `rows` rows of width `cols` would draw from the reference's device stream `rng`."""
+    if out is None:
+        out = torch.empty((rows,), dtype=torch.float32, device="cuda")
+    check(lib.sp_philox_uniforms(C.byref(rng), ptr(out, torch.float32, "out"), rows, cols, stream_ptr()))
+    return out
+
+
 def _sample(op, x, u=None, rng=None, mask_size=0, want_cdf=False, want_u=False, want_prob=False, probs_out=None,
-            sample_out=None):
+            sample_out=None, want_probs=True):
     rows, cols = _rows_cols(x)
-    probs = torch.empty_like(x) if probs_out is None else probs_out
+    probs = probs_out
+    if probs is None and want_probs:
+        probs = torch.empty_like(x)
     sample = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device) if sample_out is None else sample_out
     cdf = torch.empty_like(x) if want_cdf else None
     u_out = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if want_u else None
     prob = torch.empty(x.shape[:-1], dtype=torch.float32, device=x.device) if want_prob else None
     if (u is None) == (rng is None):
         raise ValueError("give exactly one of u (a tensor of uniforms in (0, 1]) and rng (a PhiloxConfig)")
-    if probs.shape != x.shape or sample.shape != x.shape[:-1]:
+    if (probs is not None and probs.shape != x.shape) or sample.shape != x.shape[:-1]:
         raise ValueError("the output tensors do not have the input's dimensions")
     check(lib.sp_row_sample(op, ptr(x, torch.float32, "x"), ptr(u, torch.float32, "u"),
-                            C.byref(rng) if rng is not None else None, ptr(probs, torch.float32, "probs"), ptr(cdf),
+                            C.byref(rng) if rng is not None else None,
+                            ptr(probs, torch.float32, "probs") if probs is not None else None, ptr(cdf),
                             ptr(u_out), ptr(sample, torch.int32, "sample"), ptr(prob), rows, cols, mask_size,
                             stream_ptr()))
     res = (probs, sample)
@@ -196,11 +209,13 @@ def get_action(x, u=None, rng=None, op="identity", size=0):
     return prob, action
 
 
-def binarize(x, modulo):
+def binarize(x, modulo, out=None):
     """row_reduce local_binarize (ml/primitives.spi:817-821; layer head ml/layers.spi:439-446)."""
     rows, cols = _rows_cols(x)
-    out = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device)   # holds the reference's u32
-    check(lib.sp_row_binarize(ptr(x, torch.float32, "x"), ptr(out), rows, cols, modulo, stream_ptr()))
+    if out is None:
+        out = torch.empty(x.shape[:-1], dtype=torch.int32, device=x.device)   # holds the reference's u32
+    check(lib.sp_row_binarize(ptr(x, torch.float32, "x"), ptr(out, torch.int32, "out"), rows, cols, modulo,
+                              stream_ptr()))
     return out
 
 

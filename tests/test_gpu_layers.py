@@ -1,0 +1,163 @@
+"""The layer graph on the GPU (every node through the C ABI) against the NumPy oracle composed by
+hand the way ml/layers.spi:194-240 interprets the nodes.  Bar: f32 tensors within a relative
+Frobenius error of 1e-5, 16-bit stacks 3e-3; sampled indices bit-exact given the kernel's own
+probabilities and the reference's per-thread Philox streams.
+
+PARITY UNPINNED against reference outputs: the reference's layer goldens hold inputs truncated to 100
+values, so no forward result can be recomputed from them; what they do pin (arena sizes, text
+format) is in test_layers_graph_cpu.py."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm, layers as olayers, philox as ophilox, row_ops as orow
+from gpu_util import announce, dev, host
+
+pytestmark = pytest.mark.gpu
+
+Q = 24   # blocks per grid of the reference's RTX 4060 runs
+
+
+@pytest.fixture()
+def L():
+    from ml import layers
+    layers.set_blocks_per_grid(Q)
+    layers.set_random_seed(5)
+    return layers
+
+
+def fill(t, rng, scale=1.0):
+    x = (rng.standard_normal(tuple(t.shape)) * scale).astype(np.float32)
+    t.copy_(torch.from_numpy(x).to(t.dtype))
+    return host(t.float()) if t.dtype != torch.float32 else x
+
+
+def dense_ln_relu(h, ws):
+    """matmul -> ln_l2 -> relu -> ... -> matmul on (rows, k) f32."""
+    for i, w in enumerate(ws):
+        h = ogemm.gemm_abt(h, w)
+        if i + 1 < len(ws):
+            h = orow.relu(orow.ln_l2(h))
+    return h
+
+
+def test_feedforward_sampling_graph(L):
+    """The graph of ml/layers.spi test3 (:564-593)."""
+    announce("layers test3 graph")
+    g = L.pipe(L.input("input", (Q, 64, 64)), L.matmul((64, 64)), L.ln_l2, L.relu, L.matmul((64, 64)), L.ln_l2, L.relu,
+               L.matmul((64, 64)), L.softmax_and_discrete_sample)
+    m = L.create_model(g)
+    L.pass_init(m)
+    rng = np.random.default_rng(0)
+    x = fill(L.key_extract(m, "input"), rng)
+    ws = [host(t) for _, t, _ in L.extract_layers_(m, L.weight_id())]
+    assert [w.shape for w in ws] == [(64, 64)] * 3 and 0.08 < ws[0].std() < 0.12
+    L.graph_run_host(m, {})
+    probs, idx = (host(t) for t in L.graph_extract(m, {}))
+    want = orow.softmax(dense_ln_relu(x.reshape(-1, 64), ws))
+    assert ogemm.rel_frobenius(probs.reshape(-1, 64), want) < 1e-5
+    u = ophilox.row_uniforms_layer(Q, 64, 64)
+    assert (idx.reshape(-1) == orow.discrete_sampling(probs.reshape(-1, 64), u, order="wave")).all()
+    # a second run redraws from the start of every thread's stream, like a second kernel launch
+    L.graph_run_host(m, {})
+    assert (host(L.graph_extract(m, {})[1]) == idx).all()
+
+
+@pytest.mark.parametrize("ensemble,size,deep", [(3, None, True), (4, 11, False)])
+def test_ensemble_graphs(L, ensemble, size, deep):
+    """The graphs of ml/layers.spi test4 (:596-630) and test5 (:633-665), smaller ensembles."""
+    announce("layers ensemble graph e=%d size=%s" % (ensemble, size))
+    out = L.pair(L.apply("ensemble", L.input("output_probs", (ensemble, Q, 64, 64))),
+                 L.apply("ensemble", L.input("output_indices", (ensemble, Q, 64), "int")))
+    x = L.pipe(L.input("input", (Q, 64, 64)), L.matmul_ensemble((ensemble, 64, 64)))
+    if deep:
+        x = L.pipe(x, L.ln_l2, L.relu, L.matmul_ensemble((ensemble, 64, 64)), L.ln_l2, L.relu,
+                   L.matmul_ensemble((ensemble, 64, 64)))
+    g = L.softmax_and_discrete_sample_(out, x) if size is None else L.masked_softmax_and_discrete_sample_(size, out, x)
+    m = L.create_model(g)
+    L.pass_init(m)
+    rng = np.random.default_rng(1)
+    xin = fill(L.key_extract(m, "input"), rng)
+    ws = [host(t) for t in L.key_extract_list(m, "weights")]
+    assert all(w.shape == (ensemble, 64, 64) for w in ws) and len(ws) == (3 if deep else 1)
+    L.graph_run_host(m, {"ensemble": ensemble})
+    probs, idx = host(L.key_extract(m, "output_probs")), host(L.key_extract(m, "output_indices"))
+    per_node = ophilox.draws_per_sampling_node(64, 64)
+    for e in range(ensemble):
+        logits = dense_ln_relu(xin.reshape(-1, 64), [w[e] for w in ws])
+        want = orow.softmax(logits) if size is None else orow.masked_softmax(logits, size)
+        assert ogemm.rel_frobenius(probs[e].reshape(-1, 64), want) < 1e-5
+        # one generator state per thread for the whole run: ensemble member e starts e nodes in
+        u = ophilox.row_uniforms_layer(Q, 64, 64, offset=e * per_node)
+        assert (idx[e].reshape(-1) == orow.discrete_sampling(probs[e].reshape(-1, 64), u, order="wave")).all()
+        if size is not None:
+            assert (idx[e] < size).all() and (probs[e][..., size:] == 0).all()
+
+
+def test_other_heads_and_maps(L):
+    announce("layers heads and maps")
+    x = L.input("input", (Q, 8, 32))
+    h = L.pipe(x, L.matmul((32, 32)))
+    g = L.pair(L.pair(L.argmax(L.tanh(h)), L.max(L.sigmoid(h))),
+               L.pair(L.binarize(1000003, h), L.pair(L.discrete_sample(L.regret_matching(h)),
+                                                    L.masked_regret_matching(5, L.copy(h)))))
+    m = L.create_model(g)
+    L.pass_init(m)
+    rng = np.random.default_rng(2)
+    xin = fill(L.key_extract(m, "input"), rng)
+    (w,) = [host(t) for _, t, _ in L.extract_layers_(m, L.weight_id())]
+    L.graph_run_host(m)
+    (am, mx), (bits, (smp, mrm)) = L.graph_extract(m)
+    hh = ogemm.gemm_abt(xin.reshape(-1, 32), w)
+    assert (host(am).reshape(-1) == orow.argmax(np.tanh(hh))).all()
+    assert np.abs(host(mx).reshape(-1) - (1 / (1 + np.exp(-hh))).max(axis=1)).max() < 1e-6
+    assert (host(bits).reshape(-1).view(np.uint32) == orow.binarize(hh, 1000003)).sum() >= hh.shape[0] - 2  # x ~ 0 ties
+    rm = orow.regret_matching(hh)
+    u = ophilox.row_uniforms_layer(Q, 8, 32)
+    picked = host(smp).reshape(-1)
+    agree = picked == orow.discrete_sampling(rm, u)
+    assert agree.mean() > 0.99 and (np.take_along_axis(rm, picked[:, None].astype(np.int64), 1) > 0).all()
+    assert ogemm.rel_frobenius(host(mrm).reshape(-1, 32), orow.masked_regret_matching(hh, 5)) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_relu_mlp_graph_runs_fused(L, dtype):
+    """A 16-bit matmul/relu chain with a masked sampling head is one sp_mlp_forward launch that
+    writes only the head's outputs."""
+    announce("layers fused graph " + dtype)
+    g = L.pipe(L.input("input", (Q, 128, 32), dtype), L.matmul((32, 256)), L.relu, L.matmul((256, 256)), L.relu,
+               L.matmul((256, 64)), L.masked_softmax_and_discrete_sample(3))
+    m = L.create_model(g)
+    assert L._fused_plan(m) is not None
+    rng = np.random.default_rng(4)
+    xin = fill(L.key_extract(m, "input"), rng)
+    ws = [fill(t, rng, 1 / np.sqrt(t.shape[1])) for _, t, _ in L.extract_layers_(m, L.weight_id())]
+    workspace = L.model_to_model_ptrs(m)[L.workspace_id()]
+    first_hidden = L.graph_extract(L.Model(g.a.a.a.a.a, m.dims, m.data))
+    first_hidden.fill_(7)
+    L.graph_run_host(m)
+    probs, idx = (host(t) for t in L.graph_extract(m))
+    u = ophilox.row_uniforms_layer(Q, 128, 64)
+    want, _, _ = olayers.mlp_forward(xin.reshape(-1, 32), ws, None, olayers.HEAD_SOFTMAX, u, None, 3)
+    assert ogemm.rel_frobenius(probs.reshape(-1, 64), want) < 3e-3
+    assert (idx.reshape(-1) == orow.discrete_sampling(probs.reshape(-1, 64), u)).all() and (idx < 3).all()
+    assert (host(first_hidden.float()) == 7).all() and workspace.numel() > 0     # intermediates were never written
+    with pytest.raises(Exception):
+        L.graph_run_host(m, fuse=False)    # node by node the maps and row ops are f32-only
+
+
+def test_main_body_writes_the_reference_files(L, tmp_path):
+    announce("layers main_body")
+    root = str(tmp_path) + "/"
+    L.main_body(root)
+    for i in range(1, 6):
+        assert os.path.getsize(os.path.join(root, "test%d" % i, "layers.txt")) > 0
+    t1 = open(os.path.join(root, "test1", "layers.txt")).read().splitlines()
+    assert t1[0] == "---" and t1[4] == "Done initing." and len(t1) == 8 and t1[1].count("0.000000") == 16
+    t3 = open(os.path.join(root, "test3", "layers.txt")).read()
+    assert t3.startswith("Here are the weight matrices.\n[[") and t3.rstrip().endswith("====") and " ...]" in t3
+    t5 = open(os.path.join(root, "test5", "layers.txt")).read()
+    idx = np.array([int(v) for v in t5.replace("[", " ").replace("]", " ").replace(";", " ").split()])
+    assert idx.size == 4 * Q * 64 and idx.min() >= 0 and idx.max() <= 10
