@@ -85,7 +85,7 @@ __device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane
 // local_discrete_sampling (ml/primitives.spi:782-798) with sequential prefix sums.  `src` holds the
 // row's N last-layer outputs; MAXN bounds N at compile time so that narrow heads stay in registers.
 template <int MAXN>
-__device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, long row, int N, int limit) {
+__device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, long row, int N, int limit, float u) {
     float p[MAXN];
 #pragma unroll
     for (int n = 0; n < MAXN; ++n) p[n] = n < N ? src[n] : 0.f;
@@ -131,7 +131,7 @@ __device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, lon
             cdf[n] = run;
             if (n < N && p[n] > 0.f) m = fmaxf(m, run);
         }
-        const float thr = a.u[row] * m;
+        const float thr = u * m;
         int pick = INT_MAX_;
 #pragma unroll
         for (int n = MAXN - 1; n >= 0; --n)
@@ -341,8 +341,274 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
         const int N = a.dims[a.n_layers];
         const int limit = a.mask_size > 0 ? a.mask_size : N;
         float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs
-        if (N <= 8) head_row<8>(a, p, row, N, limit);      // narrow heads run in registers
-        else head_row<MLP_MAX_OUT>(a, p, row, N, limit);
+        const float u = a.action != nullptr ? a.u[row] : 1.f;
+        if (N <= 8) head_row<8>(a, p, row, N, limit, u);      // narrow heads run in registers
+        else head_row<MLP_MAX_OUT>(a, p, row, N, limit, u);
+    }
+}
+
+
+// ---- stacks whose hidden layers are all 256 wide ------------------------------------------------
+// Same data flow as mlp_forward_kernel (16 batch rows per wave, activations in registers, weights
+// streamed through the LDS ring three chunks ahead), with the hidden width a compile-time 256 and
+// NO data-dependent control flow around the register arrays: every 256-row chunk has the same
+// shape, all per-lane DMA offsets are computed once, a chunk costs a wave no vector instructions
+// besides its 32 MFMAs and 32 LDS reads, and the DMA instructions are issued one by one between
+// the MFMA groups.  The first layer always runs C0 whole chunks (1 for K0 <= 64, else 4; K-pieces
+// past K0 re-read the last valid piece and meet zero activations), the last layer (at most 64
+// outputs) travels as ONE chunk holding its four 64-column slabs at 64-row spacing and always
+// computes 4 tiles (rows past the outputs are stale but finite-or-not they only reach unused columns).
+template <int N>
+struct IC { static constexpr int value = N; };
+
+// relu + rounding of four f32 to the 16-bit storage type: round first (v_cvt_pk), then clamp the two
+// packed values at zero as signed 16-bit integers -- a negative float of either format has the sign
+// bit set, so it is a negative integer, and relu commutes with the sign-symmetric rounding.
+template <int DT>
+__device__ __forceinline__ unsigned pack_relu2(float a, float b) {
+    unsigned p;
+    if constexpr (DT == SP_F16) p = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, f16x2));
+    else p = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
+    unsigned r;
+    asm("v_pk_max_i16 %0, %1, 0" : "=v"(r) : "v"(p));
+    return r;
+}
+
+template <int DT, int NW, int C0>
+__global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
+    constexpr int H = 256;
+    constexpr int PW = 32 / NW;                      // DMA instructions per wave and chunk
+    constexpr int ROWS = NW * 16;
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, q = lane >> 4;
+    const long row = (long)blockIdx.x * ROWS + wave * 16 + j;
+    const bool row_ok = row < a.batch;
+    const unsigned lds_base = (unsigned)(size_t)lds;
+    const unsigned dummy_dst = lds_base + MLP_STAGES * MLP_STAGE_BYTES;
+    const int K0 = a.dims[0], NL = a.n_layers, NOUT = a.dims[a.n_layers];
+    const int n_chunks = C0 + 4 * (NL - 2) + 1;
+
+    // ---- the wave's input rows, requested before any weight so that they are the oldest loads;
+    //      the row's uniform for the sampling head travels with them ----
+    u32x4 act[H / 32];
+    float u_row = 1.f;
+    {
+        const unsigned char* xr = (const unsigned char*)a.x + (row_ok ? row : 0) * K0 * 2;
+#pragma unroll
+        for (int s = 0; s < H / 32; ++s) {
+            const int k = 32 * s + 8 * q;
+            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(act[s]) : "v"(xr + (k < K0 ? k : 0) * 2) : "memory");
+        }
+        if (a.u != nullptr)
+            asm volatile("global_load_dword %0, %1, off" : "=v"(u_row) : "v"(a.u + (row_ok ? row : 0)) : "memory");
+    }
+
+    // ---- per-lane source offsets, once ----
+    // 256-row chunks: instruction m of this wave fetches rows 8 * (wave + NW * m) .. + 7; NW is a
+    // multiple of 4, so the swizzle of its rows does not depend on m.
+    static_assert(NW % 4 == 0, "the K piece of a lane must not depend on the DMA instruction");
+    const int piece = (lane & 7) ^ ((2 * (wave & 3)) | ((lane >> 4) & 1));
+    unsigned off0[PW], offH[PW], offL[PW];
+    unsigned dstL[PW];                               // LDS offsets of the last layer's instructions inside a stage
+    const int rb = (NOUT + 7) / 8;                   // 8-row blocks of the last layer (at most 8)
+#pragma unroll
+    for (int m = 0; m < PW; ++m) {
+        const int ii = wave + NW * m;
+        const int n = ii * 8 + (lane >> 3);
+        offH[m] = (unsigned)((n * H + piece * 8) * 2);
+        // first layer: in slab c the pieces past K0 re-read the last valid one (C0 slabs, one offset per slab
+        // would cost registers: the clamp is applied per chunk below with one subtraction)
+        off0[m] = (unsigned)(n * K0 * 2);
+        // last layer: instruction ii = (slab, 8-row block); no division: ii < 32, rb <= 8
+        const int slab = (ii >= rb) + (ii >= 2 * rb) + (ii >= 3 * rb);
+        const int blk = ii - slab * rb;
+        int nl = blk * 8 + (lane >> 3);
+        const int pl = (lane & 7) ^ mlp_swz(nl);
+        nl = nl < NOUT ? nl : NOUT - 1;
+        offL[m] = (unsigned)((nl * H + slab * 64 + pl * 8) * 2);
+        dstL[m] = ii < 4 * rb ? (unsigned)((slab * 64 + blk * 8) * 128) : ~0u;
+    }
+
+    int pf = 0, pf_stage = 0;                        // next chunk to fetch and its ring stage
+    const unsigned char* pf_base = (const unsigned char*)a.w[0];
+    unsigned pf_dst0 = lds_base;
+    bool pf_last = false, pf_none = false;
+    unsigned cur[PW];
+    auto prepare = [&]() {
+        pf_dst0 = lds_base + pf_stage * MLP_STAGE_BYTES;
+        pf_last = pf == n_chunks - 1;
+        pf_none = pf >= n_chunks;
+        if (pf < C0) {
+            pf_base = (const unsigned char*)a.w[0];
+            int k = pf * 64 + piece * 8;
+            k = k <= K0 - 8 ? k : K0 - 8;
+#pragma unroll
+            for (int m = 0; m < PW; ++m) cur[m] = off0[m] + (unsigned)(k * 2);
+        } else if (pf < n_chunks - 1) {
+            const int hl = (pf - C0) >> 2;
+            pf_base = (const unsigned char*)a.w[1 + hl] + ((pf - C0) & 3) * 128;
+#pragma unroll
+            for (int m = 0; m < PW; ++m) cur[m] = offH[m];
+        } else {
+            pf_base = (const unsigned char*)a.w[NL - 1];
+#pragma unroll
+            for (int m = 0; m < PW; ++m) cur[m] = offL[m];
+        }
+        ++pf;
+        pf_stage = (pf_stage + 1) & (MLP_STAGES - 1);
+    };
+    auto issue = [&](int m) {
+        const int ii = wave + NW * m;
+        unsigned dst = pf_dst0 + ii * 1024;                                        // 256-row chunk: 8 rows per KiB
+        if (pf_last) dst = dstL[m] != ~0u ? pf_dst0 + dstL[m] : dummy_dst;
+        if (pf_none) dst = dummy_dst;
+        mlp_dma(pf_base, cur[m], __builtin_amdgcn_readfirstlane(dst));
+    };
+    auto fetch = [&]() {
+        prepare();
+#pragma unroll
+        for (int m = 0; m < PW; ++m) issue(m);
+    };
+    fetch();
+    fetch();
+    fetch();
+
+    int stage = 0;
+    const int n0 = 8 * (j >> 2) + (j & 3);
+    unsigned frag_off[2];
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) frag_off[sp] = (unsigned)(n0 * 128 + (((4 * sp + q) ^ mlp_swz(n0)) << 4));
+    auto tile_off = [](int t) { return ((t >> 1) * 32 + (t & 1) * 4) * 128; };
+    auto tile_col = [&](int t) { return 32 * (t >> 1) + 4 * (t & 1) + 8 * q; };
+    auto mfma = [&](const f32x4& c, const u32x4& w, const u32x4& x) {
+        if constexpr (DT == SP_F16)
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, x), c, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), c, 0, 0, 0);
+    };
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc[H / 16];
+    // wait for the oldest chunk in flight, barrier, prepare the next fetch
+    auto chunk_sync = [&]() -> const unsigned char* {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PW) : "memory");
+        __syncthreads();
+        prepare();
+        const unsigned char* st = lds + stage * MLP_STAGE_BYTES;
+        stage = (stage + 1) & (MLP_STAGES - 1);
+        return st;
+    };
+    // all 16 output tiles x both 32-wide steps of chunk C (the layer's first chunk starts the
+    // accumulators from zero), software pipelined by hand: the weight pieces of group g + 2 are
+    // requested before the MFMAs of group g; one DMA instruction of the next fetch after every
+    // 8 / PW-th group
+    auto full_chunk = [&](auto C_) {
+        constexpr int c = decltype(C_)::value;
+        const unsigned char* st = chunk_sync();
+        auto read = [&](int t, int sp) { return *reinterpret_cast<const u32x4*>(st + frag_off[sp] + tile_off(t)); };
+        u32x4 w[3][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) w[0][t] = read(t, 0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) w[1][t] = read(t, 1);
+#pragma unroll
+        for (int g = 0; g < 8; ++g) {
+            if (g + 2 < 8) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t) w[(g + 2) % 3][t] = read(((g + 2) >> 1) * 4 + t, (g + 2) & 1);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                f32x4& d = acc[(g >> 1) * 4 + t];
+                d = mfma((c == 0 && (g & 1) == 0) ? zero4 : d, w[g % 3][t], act[2 * c + (g & 1)]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int m = g * PW / 8; m < (g + 1) * PW / 8; ++m) issue(m);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto next_activations = [&](const float* bias) {
+#pragma unroll
+        for (int s = 0; s < H / 32; ++s) {
+            f32x4 lo = acc[2 * s], hi = acc[2 * s + 1];
+            if (bias != nullptr) {   // uniform; only the two temporaries depend on it
+                lo += *reinterpret_cast<const f32x4*>(bias + tile_col(2 * s));
+                hi += *reinterpret_cast<const f32x4*>(bias + tile_col(2 * s + 1));
+            }
+            act[s] = u32x4{pack_relu2<DT>(lo[0], lo[1]), pack_relu2<DT>(lo[2], lo[3]), pack_relu2<DT>(hi[0], hi[1]),
+                           pack_relu2<DT>(hi[2], hi[3])};
+        }
+    };
+
+    // ---- first layer: K0 -> 256.  The inputs are older than every weight DMA, so they have landed
+    //      with the first chunk; lanes past K0 (and rows past the batch) feed zeros ----
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PW) : "memory");
+#pragma unroll
+    for (int s = 0; s < H / 32; ++s) {
+        asm volatile("" : "+v"(act[s]));
+        const bool live = row_ok && 32 * s + 8 * q < K0;
+        act[s] = live ? act[s] : u32x4{0u, 0u, 0u, 0u};
+    }
+    asm volatile("" : "+v"(u_row));
+    full_chunk(IC<0>{});
+    if constexpr (C0 > 1) {
+        full_chunk(IC<1>{});
+        full_chunk(IC<2>{});
+        full_chunk(IC<3>{});
+    }
+    next_activations(a.b[0]);
+
+    // ---- hidden layers: 256 -> 256 ----
+    for (int layer = 1; layer + 1 < NL; ++layer) {
+        full_chunk(IC<0>{});
+        full_chunk(IC<1>{});
+        full_chunk(IC<2>{});
+        full_chunk(IC<3>{});
+        next_activations(a.b[layer]);
+    }
+
+    // ---- last layer: 256 -> NOUT <= 64, one chunk, 4 tiles ----
+    {
+        const unsigned char* st = chunk_sync();
+#pragma unroll
+        for (int m = 0; m < PW; ++m) issue(m);
+#pragma unroll
+        for (int c = 0; c < H / 64; ++c)
+#pragma unroll
+            for (int sp = 0; sp < 2; ++sp) {
+                u32x4 w[MLP_MAX_OUT / 16];
+#pragma unroll
+                for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
+                    w[t] = *reinterpret_cast<const u32x4*>(st + c * 64 * 128 + frag_off[sp] + tile_off(t));
+#pragma unroll
+                for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
+                    acc[t] = mfma((c == 0 && sp == 0) ? zero4 : acc[t], w[t], act[2 * c + sp]);
+            }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the dummy DMAs before the LDS is released
+    __syncthreads();                                    // every wave has read its last weights: reuse stage 0
+    float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
+    const float* bias = a.b[NL - 1];
+#pragma unroll
+    for (int t = 0; t < MLP_MAX_OUT / 16; ++t) {
+        f32x4 v = acc[t];
+        if (bias != nullptr) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (tile_col(t) + r < NOUT) v[r] += bias[tile_col(t) + r];
+        }
+        *reinterpret_cast<f32x4*>(head_rows + j * MLP_MAX_OUT + tile_col(t)) = v;
+    }
+    // ---- head: lanes 0..15 of every wave own one batch row each (the staging is wave private) ----
+    if (lane < 16 && row_ok) {
+        const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
+        float* p = head_rows + lane * MLP_MAX_OUT;
+        if (NOUT <= 8) head_row<8>(a, p, row, NOUT, limit, u_row);
+        else head_row<MLP_MAX_OUT>(a, p, row, NOUT, limit, u_row);
     }
 }
 
@@ -405,9 +671,22 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     const int cus = device_cu_count();
     const bool wide = (batch + 127) / 128 * 2 >= cus;
     const int nw = wide ? 8 : 4;
+    bool h256 = n_layers >= 2;   // all hidden layers 256 wide: the lean kernel
+    for (int i = 1; i < n_layers; ++i) h256 = h256 && dims[i] == 256;
     const void* kernel;
-    if (dtype == SP_F16) kernel = wide ? (const void*)mlp_forward_kernel<SP_F16, 8> : (const void*)mlp_forward_kernel<SP_F16, 4>;
-    else kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
+    if (h256) {
+        const bool small_k = dims[0] <= 64;
+        if (dtype == SP_F16)
+            kernel = wide ? (small_k ? (const void*)mlp_h256_kernel<SP_F16, 8, 1> : (const void*)mlp_h256_kernel<SP_F16, 8, 4>)
+                          : (small_k ? (const void*)mlp_h256_kernel<SP_F16, 4, 1> : (const void*)mlp_h256_kernel<SP_F16, 4, 4>);
+        else
+            kernel = wide ? (small_k ? (const void*)mlp_h256_kernel<SP_BF16, 8, 1> : (const void*)mlp_h256_kernel<SP_BF16, 8, 4>)
+                          : (small_k ? (const void*)mlp_h256_kernel<SP_BF16, 4, 1> : (const void*)mlp_h256_kernel<SP_BF16, 4, 4>);
+    } else if (dtype == SP_F16) {
+        kernel = wide ? (const void*)mlp_forward_kernel<SP_F16, 8> : (const void*)mlp_forward_kernel<SP_F16, 4>;
+    } else {
+        kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
+    }
     const int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
     hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
