@@ -94,6 +94,8 @@ __device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, lon
         for (int n = 0; n < MAXN; ++n)
             if (n < N) a.logits[row * N + n] = p[n];
     }
+    // exp on the hardware exp2 unit and one reciprocal per normalisation: a 16-lane serial head is
+    // otherwise a visible part of a forward pass that takes a few microseconds
     if (a.head == SP_HEAD_SOFTMAX || a.head == SP_HEAD_SOFTMAX_RM) {
         float m = -__builtin_inff();
 #pragma unroll
@@ -102,11 +104,12 @@ __device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, lon
         float s = 0.f;
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) {
-            p[n] = n < limit ? expf(p[n] - m) : 0.f;
+            p[n] = n < limit ? __builtin_amdgcn_exp2f((p[n] - m) * 1.44269504088896340736f) : 0.f;
             if (n < N) s = s + p[n];
         }
+        const float inv = 1.f / s;
 #pragma unroll
-        for (int n = 0; n < MAXN; ++n) p[n] = p[n] / s;
+        for (int n = 0; n < MAXN; ++n) p[n] = p[n] * inv;
     }
     if (a.head == SP_HEAD_REGRET_MATCHING || a.head == SP_HEAD_SOFTMAX_RM) {
         float s = 0.f;
@@ -116,8 +119,9 @@ __device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, lon
             if (n < N) s = s + p[n];
         }
         const float inv_len = 1.f / (float)limit;
+        const float inv = s != 0.f ? 1.f / s : 0.f;
 #pragma unroll
-        for (int n = 0; n < MAXN; ++n) p[n] = n < limit ? (s != 0.f ? p[n] / s : inv_len) : 0.f;
+        for (int n = 0; n < MAXN; ++n) p[n] = n < limit ? (s != 0.f ? p[n] * inv : inv_len) : 0.f;
     }
 #pragma unroll
     for (int n = 0; n < MAXN; ++n)
@@ -413,23 +417,11 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     const int piece = (lane & 7) ^ ((2 * (wave & 3)) | ((lane >> 4) & 1));
     unsigned off0[PW], offH[PW], offL[PW];
     unsigned dstL[PW];                               // LDS offsets of the last layer's instructions inside a stage
-    const int rb = (NOUT + 7) / 8;                   // 8-row blocks of the last layer (at most 8)
 #pragma unroll
     for (int m = 0; m < PW; ++m) {
-        const int ii = wave + NW * m;
-        const int n = ii * 8 + (lane >> 3);
+        const int n = (wave + NW * m) * 8 + (lane >> 3);
         offH[m] = (unsigned)((n * H + piece * 8) * 2);
-        // first layer: in slab c the pieces past K0 re-read the last valid one (C0 slabs, one offset per slab
-        // would cost registers: the clamp is applied per chunk below with one subtraction)
-        off0[m] = (unsigned)(n * K0 * 2);
-        // last layer: instruction ii = (slab, 8-row block); no division: ii < 32, rb <= 8
-        const int slab = (ii >= rb) + (ii >= 2 * rb) + (ii >= 3 * rb);
-        const int blk = ii - slab * rb;
-        int nl = blk * 8 + (lane >> 3);
-        const int pl = (lane & 7) ^ mlp_swz(nl);
-        nl = nl < NOUT ? nl : NOUT - 1;
-        offL[m] = (unsigned)((nl * H + slab * 64 + pl * 8) * 2);
-        dstL[m] = ii < 4 * rb ? (unsigned)((slab * 64 + blk * 8) * 128) : ~0u;
+        off0[m] = (unsigned)(n * K0 * 2);            // + the K piece, clamped per slab when the chunk is prepared
     }
 
     int pf = 0, pf_stage = 0;                        // next chunk to fetch and its ring stage
@@ -472,7 +464,22 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
 #pragma unroll
         for (int m = 0; m < PW; ++m) issue(m);
     };
-    fetch();
+    fetch();   // the first chunk (always of the first layer) is on its way before the remaining setup
+    {
+        const int rb = (NOUT + 7) / 8;               // 8-row blocks of the last layer (at most 8)
+#pragma unroll
+        for (int m = 0; m < PW; ++m) {
+            // last layer: instruction ii = (slab, 8-row block); no division: ii < 32, rb <= 8
+            const int ii = wave + NW * m;
+            const int slab = (ii >= rb) + (ii >= 2 * rb) + (ii >= 3 * rb);
+            const int blk = ii - slab * rb;
+            int nl = blk * 8 + (lane >> 3);
+            const int pl = (lane & 7) ^ mlp_swz(nl);
+            nl = nl < NOUT ? nl : NOUT - 1;
+            offL[m] = (unsigned)((nl * H + slab * 64 + pl * 8) * 2);
+            dstL[m] = ii < 4 * rb ? (unsigned)((slab * 64 + blk * 8) * 128) : ~0u;
+        }
+    }
     fetch();
     fetch();
 
@@ -666,10 +673,11 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     if (rc != SP_OK) return rc;
     a.x = x; a.n_layers = n_layers; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size;
-    // 8 waves (128 rows) per workgroup halve the L2 -> LDS weight traffic and put two waves on every
-    // SIMD; taken once such workgroups still cover half the compute units
+    // 4 waves (64 rows) per workgroup while such workgroups fit the compute units in one round: every
+    // wave reads all weights from LDS, so 8 waves on a unit are LDS-bandwidth bound (2048 cycles per
+    // 32 KiB chunk) where 4 are not; beyond one round, 8 waves (128 rows) halve the rounds
     const int cus = device_cu_count();
-    const bool wide = (batch + 127) / 128 * 2 >= cus;
+    const bool wide = (batch + 63) / 64 > cus;
     const int nw = wide ? 8 : 4;
     bool h256 = n_layers >= 2;   // all hidden layers 256 wide: the lean kernel
     for (int i = 1; i < n_layers; ++i) h256 = h256 && dims[i] == 256;
