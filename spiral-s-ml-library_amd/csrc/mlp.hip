@@ -583,20 +583,27 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
         const unsigned char* st = chunk_sync();
 #pragma unroll
         for (int m = 0; m < PW; ++m) issue(m);
+        // two slabs (16 reads) are requested at a time: with so few MFMAs per read the LDS round
+        // trips, not the arithmetic, set the pace
 #pragma unroll
-        for (int c = 0; c < H / 64; ++c)
+        for (int c2 = 0; c2 < H / 128; ++c2) {
+            u32x4 w[2][2][MLP_MAX_OUT / 16];
 #pragma unroll
-            for (int sp = 0; sp < 2; ++sp) {
-                u32x4 w[MLP_MAX_OUT / 16];
+            for (int cc = 0; cc < 2; ++cc)
 #pragma unroll
-                for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
-                    w[t] = *reinterpret_cast<const u32x4*>(st + c * 64 * 128 + frag_off[sp] + tile_off(t));
+                for (int sp = 0; sp < 2; ++sp)
 #pragma unroll
-                for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
-                    acc[t] = mfma((c == 0 && sp == 0) ? zero4 : acc[t], w[t], act[2 * c + sp]);
-            }
+                    for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
+                        w[cc][sp][t] = *reinterpret_cast<const u32x4*>(st + (2 * c2 + cc) * 64 * 128 + frag_off[sp] + tile_off(t));
+#pragma unroll
+            for (int cc = 0; cc < 2; ++cc)
+#pragma unroll
+                for (int sp = 0; sp < 2; ++sp)
+#pragma unroll
+                    for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
+                        acc[t] = mfma((c2 == 0 && cc == 0 && sp == 0) ? zero4 : acc[t], w[cc][sp][t], act[2 * (2 * c2 + cc) + sp]);
+        }
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // drain the dummy DMAs before the LDS is released
     __syncthreads();                                    // every wave has read its last weights: reuse stage 0
     float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
     const float* bias = a.b[NL - 1];
@@ -617,6 +624,7 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
         if (NOUT <= 8) head_row<8>(a, p, row, NOUT, limit, u_row);
         else head_row<MLP_MAX_OUT>(a, p, row, NOUT, limit, u_row);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the dummy DMAs (they land in their own KiB) before the LDS is released
 }
 
 namespace {
