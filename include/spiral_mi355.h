@@ -202,6 +202,24 @@ int sp_row_get_prob(int op, const float* x, const int32_t* action, float* prob_o
  */
 int sp_row_binarize(const float* x, uint32_t* out, int64_t rows, int64_t cols, uint32_t modulo, void* stream);
 
+/*
+ * Cross-entropy-method update of one layer's weights (ml/cem.spi:99-117, `cem`): weights_t is the
+ * TRANSPOSED weight tensor (rows = weight positions, ensemble columns, what `grid_transpose`
+ * produces, :131-132); winners (mask[e] != 0) keep their value, every other member is redrawn as
+ * (normals[r, e] * max(std, noise) + mean) * decay with mean / std taken over the winners of the
+ * row (std = biased std * n / (n - 1), 0 for a single winner).  The reference draws `normals`
+ * from curand_normal on the fly; here the caller supplies standard normals (rows, ensemble).
+ * `out` may be weights_t.  The reference uses noise 0.1, decay 1 (:76-78).
+ */
+int sp_cem_resample(const float* weights_t, const int32_t* mask, const float* normals, float* out, int64_t rows,
+                    int64_t ensemble, float noise, float decay, void* stream);
+
+/*
+ * `grid_update_rewards_mask` (ml/cem.spi:92-96): rewards is (ensemble, 2) f32 pairs (reward sum,
+ * count); mask[e] = (count ? reward / count : 0) >= average over the ensemble; the pairs are zeroed.
+ */
+int sp_cem_update_mask(float* rewards, int32_t* mask, int64_t ensemble, void* stream);
+
 typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID = 3 } sp_map_op;
 
 /* out[i] = f(x[i]) over n f32 elements (n multiple of 4).  Replaces `primitives.map f from to`

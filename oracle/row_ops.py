@@ -261,3 +261,31 @@ def binarize(x, modulo):
 def transpose_inner(x):
     """`grid_transpose_snd` (ml/primitives.spi:36-112): swap the two innermost dimensions."""
     return np.ascontiguousarray(np.swapaxes(np.asarray(x), -1, -2))
+
+
+def cem_resample(x, mask, z, noise=0.1, decay=1.0):
+    """`cem` (ml/cem.spi:99-117): x (rows, ensemble) transposed weights, mask (ensemble,) winners,
+    z standard normals.  winner_std = biased std * n / (n - 1) (0 for one winner); losers become
+    (z * max(std, noise) + mean) * decay.  PARITY UNPINNED against the reference (it holds no
+    output of this function and draws its normals on the device); pinned by closed forms."""
+    x, z = _f32(x), _f32(z)
+    m = np.asarray(mask).astype(bool)
+    n = np.float32(m.sum())
+    mean = (np.where(m, x, np.float32(0)).sum(axis=-1, dtype=np.float32) / n).astype(np.float32)
+    r = (x - mean[..., None]).astype(np.float32)
+    var = (np.where(m, r * r, np.float32(0)).sum(axis=-1, dtype=np.float32) / n).astype(np.float32)
+    std = np.sqrt(var).astype(np.float32) * n / (n - np.float32(1)) if m.sum() > 1 else np.zeros_like(var)
+    scale = np.maximum(std.astype(np.float32), np.float32(noise))
+    redrawn = ((z * scale[..., None] + mean[..., None]) * np.float32(decay)).astype(np.float32)
+    return np.where(m, x, redrawn).astype(np.float32)
+
+
+def cem_update_rewards_mask(rewards):
+    """`grid_update_rewards_mask` (ml/cem.spi:92-96): (ensemble, 2) (reward, count) pairs ->
+    mask of the members whose average reward is at least the ensemble's mean (sequential f32 sum)."""
+    rewards = _f32(rewards)
+    r = np.where(rewards[:, 1] != 0, rewards[:, 0] / np.where(rewards[:, 1] != 0, rewards[:, 1], 1), 0).astype(np.float32)
+    s = np.float32(0)
+    for v in r:
+        s = np.float32(s + v)
+    return (r >= np.float32(s / np.float32(len(r)))).astype(np.int32)

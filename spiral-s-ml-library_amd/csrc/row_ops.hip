@@ -498,6 +498,99 @@ __global__ __launch_bounds__(ROW_THREADS) void philox_uniforms_kernel(const RowA
     if (r < a.rows) a.u_out[r] = reference_row_uniform(a, r);
 }
 
+// Cross-entropy-method resampling of one weight position across the ensemble (ml/cem.spi:99-117):
+// the row holds that weight for every ensemble member; winners (mask != 0) keep their value, the
+// others are redrawn from N(mean, max(std, noise)) of the winners' values, times `decay`.
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) void cem_kernel(const float* __restrict__ x, const int* __restrict__ mask,
+                                                          const float* __restrict__ z, float* __restrict__ out, long rows,
+                                                          int cols, float noise, float decay) {
+    constexpr int ROWS_PER_WAVE = WAVE / T;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int l = lane % T;
+    const int sub = lane / T;
+    const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
+    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < rows; row0 += n_waves * ROWS_PER_WAVE) {
+        const long row = row0 + sub;
+        const bool row_ok = row < rows;
+        float v[C][4], g[C][4];
+        bool win[C][4], ok[C];
+        int cnt = 0;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            const int col = c * 4 * T + 4 * l;
+            ok[c] = row_ok && col < cols;
+            f32x4 xv = {0.f, 0.f, 0.f, 0.f}, zv = {0.f, 0.f, 0.f, 0.f};
+            int4 mv = make_int4(0, 0, 0, 0);
+            if (ok[c]) {
+                xv = *reinterpret_cast<const f32x4*>(x + row * (long)cols + col);
+                zv = *reinterpret_cast<const f32x4*>(z + row * (long)cols + col);
+                mv = *reinterpret_cast<const int4*>(mask + col);
+            }
+            const int m4[4] = {mv.x, mv.y, mv.z, mv.w};
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                v[c][k] = xv[k];
+                g[c][k] = zv[k];
+                win[c][k] = m4[k] != 0;
+                cnt += win[c][k] ? 1 : 0;
+            }
+        }
+        cnt = group_reduce<T>(cnt, [](int a, int b) { return a + b; });
+        const float winner_count = (float)cnt;
+        float s = 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) s = s + (win[c][k] ? v[c][k] : 0.f);
+        s = group_reduce<T>(s, [](float a, float b) { return a + b; });
+        const float winner_mean = s / winner_count;
+        float q = 0.f;
+#pragma unroll
+        for (int c = 0; c < C; ++c)
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float r = v[c][k] - winner_mean;
+                q = q + (win[c][k] ? r * r : 0.f);
+            }
+        q = group_reduce<T>(q, [](float a, float b) { return a + b; });
+        const float biased_std = sqrtf(q / winner_count);
+        const float winner_std = cnt > 1 ? biased_std * winner_count / (winner_count - 1.f) : 0.f;
+        const float scale = fmaxf(winner_std, noise);
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            if (ok[c]) {
+                f32x4 o;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) o[k] = win[c][k] ? v[c][k] : (g[c][k] * scale + winner_mean) * decay;
+                *reinterpret_cast<f32x4*>(out + row * (long)cols + c * 4 * T + 4 * l) = o;
+            }
+        }
+    }
+}
+
+// grid_update_rewards_mask (ml/cem.spi:92-96) for up to a few thousand ensemble members: one
+// workgroup; the average is a sequential f32 sum like the reference's fold.
+__global__ __launch_bounds__(ROW_THREADS) void cem_mask_kernel(float* __restrict__ rewards, int* __restrict__ mask, int n) {
+    __shared__ float average;
+    if (threadIdx.x == 0) {
+        float s = 0.f;
+        for (int e = 0; e < n; ++e) {
+            const float r = rewards[2 * e], c = rewards[2 * e + 1];
+            s = s + (c != 0.f ? r / c : 0.f);
+        }
+        average = s / (float)n;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < n; e += ROW_THREADS) {
+        const float r = rewards[2 * e], c = rewards[2 * e + 1];
+        mask[e] = (c != 0.f ? r / c : 0.f) >= average ? 1 : 0;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < 2 * n; e += ROW_THREADS) rewards[e] = 0.f;
+}
+
 // Lanes that share a row.  Up to 64 columns: one lane per 4 columns (rounded up to a power of two).
 // Up to 256 columns: 16 lanes (one DPP row), each holding one 4-column piece of every 64-column
 // chunk, so a wave works on 4 rows at once and no reduction leaves its DPP row.  Wider rows: the
@@ -731,4 +824,36 @@ extern "C" int sp_row_binarize(const float* x, uint32_t* out, int64_t rows, int6
     a.x = x; a.bits_out = out; a.modulo = modulo; a.rows = rows; a.cols = (int)cols; a.op = SP_ROW_IDENTITY;
     a.mask_size = (int)cols; a.philox_mode = -1;
     return launch_row<false>(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_cem_resample(const float* weights_t, const int32_t* mask, const float* normals, float* out,
+                               int64_t rows, int64_t ensemble, float noise, float decay, void* stream) {
+    SP_REQUIRE_PTR(weights_t);
+    SP_REQUIRE_PTR(mask);
+    SP_REQUIRE_PTR(normals);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, ensemble);
+    if (rc != SP_OK) return rc;
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    const int t = lanes_per_row(ensemble);
+    const int c = (int)((ensemble + 4 * t - 1) / (4 * t));
+    const int grid = row_grid(rows, t);
+    rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
+        hipLaunchKernelGGL((cem_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
+                           (hipStream_t)stream, weights_t, mask, normals, out, (long)rows, (int)ensemble, noise, decay);
+    });
+    if (rc != SP_OK) return rc;
+    return check_launch(__func__);
+}
+
+extern "C" int sp_cem_update_mask(float* rewards, int32_t* mask, int64_t ensemble, void* stream) {
+    SP_REQUIRE_PTR(rewards);
+    SP_REQUIRE_PTR(mask);
+    if (ensemble <= 0 || ensemble > 65536)
+        return fail(SP_ERR_SHAPE, "sp_cem_update_mask: ensemble must be in [1, 65536], got %lld", (long long)ensemble);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    hipLaunchKernelGGL(cem_mask_kernel, dim3(1), dim3(ROW_THREADS), 0, (hipStream_t)stream, rewards, mask, (int)ensemble);
+    return check_launch(__func__);
 }

@@ -57,6 +57,8 @@ SIGNATURES = {
     "sp_row_sample": (C.c_int, [C.c_int, _P, _P, C.POINTER(PhiloxConfig), _P, _P, _P, _P, _P, _I64, _I64, _I32, _P]),
     "sp_philox_uniforms": (C.c_int, [C.POINTER(PhiloxConfig), _P, _I64, _I64, _P]),
     "sp_row_get_prob": (C.c_int, [C.c_int, _P, _P, _P, _I64, _I64, _I32, _P]),
+    "sp_cem_resample": (C.c_int, [_P, _P, _P, _P, _I64, _I64, C.c_float, C.c_float, _P]),
+    "sp_cem_update_mask": (C.c_int, [_P, _P, _I64, _P]),
     "sp_row_binarize": (C.c_int, [_P, _P, _I64, _I64, C.c_uint32, _P]),
     "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
     "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),

@@ -219,6 +219,42 @@ def binarize(x, modulo, out=None):
     return out
 
 
+def cem_update_rewards_mask(rewards, mask=None):
+    """`grid_update_rewards_mask` (ml/cem.spi:92-96): rewards (ensemble, 2) f32 (reward sum, count) pairs are
+    turned into the winners' mask (average reward at or above the ensemble's mean) and zeroed."""
+    if rewards.dim() != 2 or rewards.shape[1] != 2:
+        raise ValueError("rewards must be (ensemble, 2)")
+    n = rewards.shape[0]
+    if mask is None:
+        mask = torch.empty((n,), dtype=torch.int32, device=rewards.device)
+    check(lib.sp_cem_update_mask(ptr(rewards, torch.float32, "rewards"), ptr(mask, torch.int32, "mask"), n, stream_ptr()))
+    return mask
+
+
+def cem(transposed_weights, mask, normals=None, noise=0.1, decay=1.0, out=None, generator=None):
+    """`cem rng transposed_weights model` (ml/cem.spi:99-117), in place by default like the reference:
+    every row holds one weight position across the ensemble; the members outside `mask` are redrawn from the
+    winners' mean and spread.  `normals` (same shape) defaults to fresh standard normals."""
+    rows, cols = _rows_cols(transposed_weights)
+    if mask.shape != (cols,):
+        raise ValueError("one mask entry per ensemble member expected")
+    if normals is None:
+        normals = torch.randn(transposed_weights.shape, generator=generator, device=transposed_weights.device,
+                              dtype=torch.float32)
+    if out is None:
+        out = transposed_weights
+    check(lib.sp_cem_resample(ptr(transposed_weights, torch.float32, "transposed_weights"), ptr(mask, torch.int32, "mask"),
+                              ptr(normals, torch.float32, "normals"), ptr(out, torch.float32, "out"), rows, cols, noise,
+                              decay, stream_ptr()))
+    return out
+
+
+def grid_transpose(x, out=None):
+    """`grid_transpose from to` (ml/primitives.spi:100-112): 2-D transpose, e.g. (ensemble, dim) <-> (dim, ensemble)
+    of the CEM weight duals (ml/cem.spi:131-146)."""
+    return transpose_snd(x, out)
+
+
 def map(op, x, out=None):  # noqa: A001  (the reference's name, ml/primitives.spi:128)
     """primitives.map f from to for f in {"copy", "relu", "tanh", "sigmoid"} (ml/layers.spi:353-355)."""
     code = {"copy": _lib.MAP_COPY, "relu": _lib.MAP_RELU, "tanh": _lib.MAP_TANH, "sigmoid": _lib.MAP_SIGMOID}[op]

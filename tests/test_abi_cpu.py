@@ -82,6 +82,10 @@ def test_row_argument_errors(L):
     assert lib.sp_row_get_prob(L.ROW_MASKED_REGRET_MATCHING, p, p, p, 8, 8, 0, None) == -5
     assert lib.sp_row_binarize(p, p, 8, 8, 0, None) == -5 and "modulo" in _err(L)
     assert lib.sp_row_binarize(p, None, 8, 8, 7, None) == -1
+    assert lib.sp_cem_resample(p, p, None, p, 8, 8, 0.1, 1.0, None) == -1
+    assert lib.sp_cem_resample(p, p, p, p, 8, 6, 0.1, 1.0, None) == -2
+    assert lib.sp_cem_update_mask(p, p, 0, None) == -2
+    assert lib.sp_cem_update_mask(None, p, 4, None) == -1
 
 
 def test_misc_argument_errors(L):

@@ -223,6 +223,39 @@ def test_layer_stream_uniforms(P):
     assert (host(u) == ophilox.row_uniforms_block(blocks * m, n)).all()
 
 
+@pytest.mark.parametrize("dim,ensemble", [(77, 16), (1000, 64), (33, 256), (5, 1024), (19, 12)])
+def test_cem_update(P, dim, ensemble):
+    """Cross-entropy-method weight update (ml/cem.spi:92-146): rewards -> mask, transpose, resample, transpose."""
+    announce("cem dim=%d ensemble=%d" % (dim, ensemble))
+    rng = np.random.default_rng(dim * 7 + ensemble)
+    rewards = np.stack([rng.standard_normal(ensemble) * 3, rng.integers(0, 4, ensemble)], axis=1).astype(np.float32)
+    rd = dev(rewards)
+    mask = P.cem_update_rewards_mask(rd)
+    want_mask = orow.cem_update_rewards_mask(rewards)
+    assert (host(mask) == want_mask).all() and (host(rd) == 0).all()
+    if want_mask.sum() == 0:
+        want_mask[0] = 1
+        mask = dev(want_mask)
+    weights = rng.standard_normal((ensemble, dim)).astype(np.float32)        # (ensemble, dim) as the layers hold them
+    z = rng.standard_normal((dim, ensemble)).astype(np.float32)
+    wt = P.grid_transpose(dev(weights))
+    assert (host(wt) == weights.T).all()
+    out = P.cem(wt, mask, normals=dev(z))
+    assert out.data_ptr() == wt.data_ptr()                                    # in place, like the reference
+    want = orow.cem_resample(weights.T, want_mask, z)
+    assert ogemm.rel_frobenius(host(out), want) < FLOAT_TOL
+    winners = want_mask.astype(bool)
+    assert (host(out)[:, winners] == weights.T[:, winners]).all()           # winners bit for bit
+    back = host(P.grid_transpose(out))
+    assert back.shape == (ensemble, dim) and (back[winners] == weights[winners]).all()
+    # one winner: every other member becomes z * noise + winner
+    single = np.zeros(ensemble, dtype=np.int32); single[ensemble // 2] = 1
+    got = host(P.cem(dev(weights.T.copy()), dev(single), normals=dev(z), noise=0.25, decay=1.0))
+    want1 = z * np.float32(0.25) + weights.T[:, ensemble // 2: ensemble // 2 + 1]
+    want1[:, ensemble // 2] = weights.T[:, ensemble // 2]
+    assert np.abs(got - want1).max() < 1e-6
+
+
 def test_sampling_edge_cases(P):
     announce("sampling edge cases")
     p = np.zeros((4, 8), dtype=np.float32)

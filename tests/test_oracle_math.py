@@ -185,3 +185,27 @@ def test_layer_stream_reduces_to_block_stream_and_shifts_by_offset():
     fresh = philox.row_uniforms_layer(2, 64, 64)
     later = philox.row_uniforms_layer(2, 32, 64, offset=philox.draws_per_sampling_node(32, 64))
     assert (later.reshape(2, 32) == fresh.reshape(2, 64)[:, 32:]).all()
+
+
+def test_cem_resample_closed_forms():
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((5, 8)).astype(np.float32)
+    z = rng.standard_normal((5, 8)).astype(np.float32)
+    everyone = np.ones(8, dtype=np.int32)
+    assert (row_ops.cem_resample(x, everyone, z) == x).all()                 # winners are never touched
+    one = np.zeros(8, dtype=np.int32); one[3] = 1                            # one winner: std 0 -> the noise floor
+    got = row_ops.cem_resample(x, one, z, noise=0.1)
+    assert (got[:, 3] == x[:, 3]).all()
+    others = np.delete(got, 3, axis=1)
+    assert np.allclose(others, np.delete(z, 3, axis=1) * np.float32(0.1) + x[:, 3:4], rtol=1e-6, atol=1e-7)
+    two = np.zeros(8, dtype=np.int32); two[[1, 6]] = 1                       # two winners a, b: mean (a+b)/2,
+    got = row_ops.cem_resample(x, two, z, noise=0.0, decay=0.5)              # std = |a-b|/2 * 2/(2-1) = |a-b|
+    a, b = x[:, 1], x[:, 6]
+    want = (z[:, 0] * np.abs(a - b) + (a + b) / 2) * 0.5
+    assert np.allclose(got[:, 0], want, rtol=1e-5, atol=1e-6)
+    assert (got[:, [1, 6]] == x[:, [1, 6]]).all()
+
+
+def test_cem_rewards_mask_by_hand():
+    rewards = np.array([[2.0, 1.0], [0.0, 0.0], [9.0, 3.0], [1.0, 2.0]], dtype=np.float32)   # averages 2, 0, 3, 0.5
+    assert row_ops.cem_update_rewards_mask(rewards).tolist() == [1, 0, 1, 0]                 # mean 1.375
