@@ -91,6 +91,25 @@ def test_other_stacks(LY, dims, head, mask):
         check(LY, x, ws, u, "f16", head, mask)
 
 
+@pytest.mark.parametrize("dims,head,mask,batch,dtype,with_bias", [
+    ([48, 256, 256, 17], "softmax", 0, 300, "f16", True),                 # K0 not a multiple of 64, ragged head
+    ([128, 256, 256, 256, 64], "softmax_regret_matching", 40, 200, "bf16", True),   # four first-layer chunks, widest head
+    ([256, 256, 8], "regret_matching", 5, 130, "f16", False),             # no hidden 256 -> 256 layer at all
+    ([64, 256, 256, 3], "softmax_regret_matching", 0, 20000, "f16", False),  # more rows than 4-wave workgroups cover: 8 waves
+    ([16, 256, 256, 256, 256, 256, 256, 256, 4], "softmax", 0, 64, "f16", True),  # the deepest stack
+])
+def test_stacks_with_256_wide_hidden_layers(LY, dims, head, mask, batch, dtype, with_bias):
+    """The shapes served by the lean kernel (all hidden layers 256 wide)."""
+    announce("mlp h256 %s head=%s mask=%d batch=%d %s bias=%s" % (dims, head, mask, batch, dtype, with_bias))
+    rng = np.random.default_rng(sum(dims) + batch)
+    x, ws, u = make_problem(rng, batch, dims, dtype)
+    biases = None
+    if with_bias:
+        biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
+        biases[0] = None
+    check(LY, x, ws, u, dtype, head, mask, biases)
+
+
 def test_bias_extension(LY):
     announce("mlp biases")
     rng = np.random.default_rng(9)
