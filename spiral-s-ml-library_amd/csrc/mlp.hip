@@ -704,8 +704,26 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
         kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
     }
     const int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
-    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+    // the LDS opt-in is per kernel and device; remember which (kernel, device) pairs have it (a lost
+    // race only repeats an idempotent call)
+    static const void* opted_kernel[64];
+    static int opted_device[64];
+    static int n_opted = 0;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    bool opted = false;
+    const int n_seen = n_opted < 64 ? n_opted : 64;
+    for (int i = 0; i < n_seen; ++i) opted = opted || (opted_kernel[i] == kernel && opted_device[i] == dev);
+    hipError_t e = hipSuccess;
+    if (!opted) {
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
+        if (n_seen < 64) {
+            opted_kernel[n_seen] = kernel;
+            opted_device[n_seen] = dev;
+            n_opted = n_seen + 1;
+        }
+    }
     const long blocks = (batch + nw * 16 - 1) / (nw * 16);
     void* args[] = {(void*)&a};
     e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(nw * 64), args, lds_bytes, (hipStream_t)stream);
