@@ -101,6 +101,19 @@ int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
 int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
                 int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream);
 
+/*
+ * `batch` independent products C_e = alpha * A_e . B_e^T + beta * C_e [+ bias] [ReLU] in one launch:
+ * member e starts stride_a / stride_b / stride_c ELEMENTS after member e - 1 (0 = every member
+ * uses the same A or B).  Replaces the loop over `.ensemble` that `graph_run_host model {ensemble}`
+ * makes around `BlockMatmul(x, apply .ensemble weights)` for `matmul_ensemble` layers
+ * (ml/layers.spi:227-240,336-344,468-471): A = the shared input, stride_a = 0, B = the (E, out, in)
+ * weight tensor, stride_b = out * in.  The tile is chosen for the whole batch, so many small members
+ * fill the chip.  bias (N,) is shared by all members.
+ */
+int sp_gemm_abt_batched(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
+                        int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a, int64_t stride_b,
+                        int64_t stride_c, float alpha, float beta, uint32_t flags, void* stream);
+
 /* Which tile configuration sp_gemm_abt picks for a shape (the counterpart of
  * `matmul_config_tf32`, ml/matmul/run.spi:8-19).  Writes block tile sizes and the workgroup size;
  * tile_m == 0 means the general kernel. */

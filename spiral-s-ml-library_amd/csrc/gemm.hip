@@ -33,6 +33,8 @@ struct GemmArgs {
     int relu;
     int out_dtype;
     int tiles_m, tiles_n;
+    long stride_a, stride_b, stride_c;   // bytes between the matrices of a batch (0: shared)
+    int batch;
     int group_m;   // tile rows per group of the block -> tile walk (4: an XCD's 32 concurrent tiles form a 4 x 8 patch)
 };
 
@@ -125,6 +127,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm, tn);
     const long m0 = (long)tm * BM, n0 = (long)tn * BN;
     const long K = g.K;
+    // batch member blockIdx.y (strided-batched launches; a plain GEMM has one member and zero strides)
+    const unsigned char* const Ab = (const unsigned char*)g.A + (long)blockIdx.y * g.stride_a;
+    const unsigned char* const Bb = (const unsigned char*)g.B + (long)blockIdx.y * g.stride_b;
+    unsigned char* const Cb = (unsigned char*)g.C + (long)blockIdx.y * g.stride_c;
 
     // ---- loader: DMA instruction q of wave w fills the 8 rows of row block q * NW + w of the
     //      stacked (A rows, then B rows) tile ----
@@ -142,8 +148,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         const int blk = (is_a ? q : q - NIA) * NW + wave;           // row block inside the A (or B) tile
         const int r = lane >> 3;                                    // row inside the block
         const int kc = (lane & 7) ^ ((r ^ blk) & 7);                // global chunk that belongs in slot lane & 7
-        const unsigned char* origin = is_a ? (const unsigned char*)g.A + (m0 + blk * 8) * K * ES
-                                           : (const unsigned char*)g.B + (n0 + blk * 8) * K * ES;
+        const unsigned char* origin = is_a ? Ab + (m0 + blk * 8) * K * ES : Bb + (n0 + blk * 8) * K * ES;
         src[q] = uniform_ptr(origin);
         lane_off[q] = (unsigned)(r * K * ES + kc * 16);
         dst[q] = __builtin_amdgcn_readfirstlane(lds_base + (is_a ? 0 : BM * ROW_BYTES) + blk * 8 * ROW_BYTES);
@@ -300,13 +305,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
                 const long idx = (m0 + wm * WTM + i * 32 + rl) * g.N + col;
                 v = v * alpha;
                 if constexpr (OT == SP_F32) {
-                    f32x4* c = reinterpret_cast<f32x4*>((float*)g.C + idx);
+                    f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
                     if (beta != 0.f) v += beta * *c;
                     v += bias4;
                     if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
                     *c = v;
                 } else {
-                    u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)g.C + idx);
+                    u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
                     if (beta != 0.f) {
                         const u32x2 o = *c;
                         v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
@@ -333,8 +338,9 @@ __global__ __launch_bounds__(256) void gemm_abt_generic_kernel(const GemmArgs g)
     const long n = (long)blockIdx.x * 16 + (threadIdx.x & 15);
     const long m = (long)blockIdx.y * 16 + (threadIdx.x >> 4);
     if (m >= g.M || n >= g.N) return;
-    const unsigned char* a = (const unsigned char*)g.A + m * g.K * ES;
-    const unsigned char* b = (const unsigned char*)g.B + n * g.K * ES;
+    const unsigned char* a = (const unsigned char*)g.A + (long)blockIdx.z * g.stride_a + m * g.K * ES;
+    const unsigned char* b = (const unsigned char*)g.B + (long)blockIdx.z * g.stride_b + n * g.K * ES;
+    unsigned char* const Cb = (unsigned char*)g.C + (long)blockIdx.z * g.stride_c;
     float s = 0.f;
     for (long k = 0; k < g.K; k += PER) {
         const u32x4 va = *reinterpret_cast<const u32x4*>(a + k * ES);
@@ -361,19 +367,19 @@ __global__ __launch_bounds__(256) void gemm_abt_generic_kernel(const GemmArgs g)
     float v = g.alpha * s;
     const float bias = g.bias ? g.bias[n] : 0.f;
     if (g.out_dtype == SP_F32) {
-        float* c = (float*)g.C;
+        float* c = (float*)Cb;
         if (g.beta != 0.f) v += g.beta * c[idx];
         v += bias;
         if (g.relu) v = fmaxf(v, 0.f);
         c[idx] = v;
     } else if (g.out_dtype == SP_BF16) {
-        unsigned short* c = (unsigned short*)g.C;
+        unsigned short* c = (unsigned short*)Cb;
         if (g.beta != 0.f) v += g.beta * __uint_as_float((unsigned)c[idx] << 16);
         v += bias;
         if (g.relu) v = fmaxf(v, 0.f);
         c[idx] = f32_to_bf16_rne(v);
     } else {
-        _Float16* c = (_Float16*)g.C;
+        _Float16* c = (_Float16*)Cb;
         if (g.beta != 0.f) v += g.beta * (float)c[idx];
         v += bias;
         if (g.relu) v = fmaxf(v, 0.f);
@@ -390,7 +396,7 @@ static const TileCfg kTileCfgs[] = {{256, 256, 2, 4}, {128, 128, 2, 2}, {64, 64,
 constexpr int kNumCfgs = 3;
 
 // Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.
-static int choose_cfg(int dtype_in, long M, long N, long K) {
+static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
     const int bk = dtype_in == SP_F32 ? 32 : 64;
     if (K % bk != 0) return -1;
     const int cus = device_cu_count();
@@ -399,7 +405,7 @@ static int choose_cfg(int dtype_in, long M, long N, long K) {
         const TileCfg& c = kTileCfgs[i];
         if (M % c.bm != 0 || N % c.bn != 0) continue;
         smallest = i;
-        const long tiles = (M / c.bm) * (N / c.bn);
+        const long tiles = (M / c.bm) * (N / c.bn) * batch;
         if (tiles * 5 >= (long)cus * 4) return i;
     }
     return smallest;
@@ -419,7 +425,7 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
         attr_set[dev & 63] = true;
     }
     const long tiles = (long)g.tiles_m * g.tiles_n;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles), dim3(WM * WN * 64), lds_bytes, stream, g);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(WM * WN * 64), lds_bytes, stream, g);
     return check_launch("sp_gemm_abt");
 }
 
@@ -430,7 +436,7 @@ static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
         case 1: return launch_tiled<DT, OT, 128, 128, 2, 2>(g, stream);
         case 2: return launch_tiled<DT, OT, 64, 64, 2, 2>(g, stream);
     }
-    dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16));
+    dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16), (unsigned)g.batch);
     hipLaunchKernelGGL(gemm_abt_generic_kernel<DT>, grid, dim3(256), 0, stream, g);
     return check_launch("sp_gemm_abt(generic)");
 }
@@ -481,23 +487,28 @@ extern "C" int sp_gemm_config(int dtype_in, int64_t M, int64_t N, int64_t K, int
     return SP_OK;
 }
 
-extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
-                           int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream) {
-    SP_REQUIRE_PTR(A);
-    SP_REQUIRE_PTR(B);
-    SP_REQUIRE_PTR(C);
-    SP_OPTIONAL_PTR(bias);
+static int gemm_entry(const char* fn, int dtype_in, int dtype_out, const void* A, const void* B, void* C,
+                      const float* bias, int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a,
+                      int64_t stride_b, int64_t stride_c, float alpha, float beta, uint32_t flags, void* stream) {
     int rc = validate_gemm(dtype_in, dtype_out, M, N, K);
     if (rc != SP_OK) return rc;
-    if (alpha == 0.f) return fail(SP_ERR_ARG, "sp_gemm_abt: The alpha must not be zero.");
-    rc = require_gfx950(__func__);
+    if (alpha == 0.f) return fail(SP_ERR_ARG, "%s: The alpha must not be zero.", fn);
+    if (batch < 1 || batch > 65535) return fail(SP_ERR_SHAPE, "%s: batch must be in [1, 65535], got %lld", fn, (long long)batch);
+    const int es_in = dtype_in == SP_F32 ? 4 : 2, es_out = dtype_out == SP_F32 ? 4 : 2;
+    if (stride_a < 0 || stride_b < 0 || stride_c < 0 || (stride_a * es_in) % 16 != 0 || (stride_b * es_in) % 16 != 0 ||
+        (stride_c * es_out) % 16 != 0)
+        return fail(SP_ERR_ALIGN, "%s: batch strides must be non-negative and keep every matrix 16-byte aligned", fn);
+    if (batch > 1 && stride_c < M * N) return fail(SP_ERR_ARG, "%s: the outputs of a batch must not overlap", fn);
+    rc = require_gfx950(fn);
     if (rc != SP_OK) return rc;
-    int cfg = (flags & SP_GEMM_FORCE_GENERIC) ? -1 : choose_cfg(dtype_in, M, N, K);
+    int cfg = (flags & SP_GEMM_FORCE_GENERIC) ? -1 : choose_cfg(dtype_in, M, N, K, batch);
     GemmArgs g{};
     g.A = A; g.B = B; g.C = C; g.bias = bias; g.M = M; g.N = N; g.K = K; g.alpha = alpha; g.beta = beta;
     g.relu = (flags & SP_GEMM_RELU) ? 1 : 0;
     g.out_dtype = dtype_out;
     g.group_m = 4;
+    g.batch = (int)batch;
+    g.stride_a = stride_a * es_in; g.stride_b = stride_b * es_in; g.stride_c = stride_c * es_out;
     if (cfg >= 0) {
         g.tiles_m = (int)(M / kTileCfgs[cfg].bm);
         g.tiles_n = (int)(N / kTileCfgs[cfg].bn);
@@ -510,4 +521,24 @@ extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const voi
         default:
             return dtype_out == SP_F32 ? launch_dtype<SP_BF16, SP_F32>(cfg, g, s) : launch_dtype<SP_BF16, SP_BF16>(cfg, g, s);
     }
+}
+
+extern "C" int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
+                           int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream) {
+    SP_REQUIRE_PTR(A);
+    SP_REQUIRE_PTR(B);
+    SP_REQUIRE_PTR(C);
+    SP_OPTIONAL_PTR(bias);
+    return gemm_entry(__func__, dtype_in, dtype_out, A, B, C, bias, M, N, K, 1, 0, 0, 0, alpha, beta, flags, stream);
+}
+
+extern "C" int sp_gemm_abt_batched(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
+                                   int64_t M, int64_t N, int64_t K, int64_t batch, int64_t stride_a, int64_t stride_b,
+                                   int64_t stride_c, float alpha, float beta, uint32_t flags, void* stream) {
+    SP_REQUIRE_PTR(A);
+    SP_REQUIRE_PTR(B);
+    SP_REQUIRE_PTR(C);
+    SP_OPTIONAL_PTR(bias);
+    return gemm_entry(__func__, dtype_in, dtype_out, A, B, C, bias, M, N, K, batch, stride_a, stride_b, stride_c, alpha,
+                      beta, flags, stream);
 }

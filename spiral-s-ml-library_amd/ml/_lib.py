@@ -50,6 +50,8 @@ SIGNATURES = {
     "sp_device_info": (C.c_int, [C.POINTER(DeviceInfo)]),
     "sp_kernel_info": (C.c_int, [C.c_char_p, C.POINTER(KernelInfo)]),
     "sp_gemm_abt": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, _P, _I64, _I64, _I64, _F, _F, _U32, _P]),
+    "sp_gemm_abt_batched": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _F, _F,
+                                      _U32, _P]),
     "sp_gemm_config": (C.c_int, [C.c_int, _I64, _I64, _I64] + [C.POINTER(C.c_int32)] * 4),
     "sp_row_ops": (C.c_int, [_P] * 8 + [_I64, _I64, _U32, _P]),
     "sp_row_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _I64, _I32, _P]),

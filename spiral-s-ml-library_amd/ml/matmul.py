@@ -46,6 +46,33 @@ def matmul_abt(a, b, c=None, alpha=1.0, beta=0.0, bias=None, relu=False, out_dty
     return c
 
 
+def matmul_abt_batched(a, b, c=None, alpha=1.0, beta=0.0, bias=None, relu=False, out_dtype=None, force_generic=False):
+    """C[e] = alpha * A[e] . B[e]^T + beta * C[e] for every batch member in ONE launch.  a: (E, M, K) or (M, K)
+    (shared by all members), b: (E, N, K) or (N, K), at least one of them batched; c: (E, M, N).  This is the
+    loop `graph_run_host model {ensemble}` makes around a `matmul_ensemble` layer (ml/layers.spi:336-344,468-471)."""
+    if a.dtype != b.dtype or a.dtype not in _lib.DTYPES:
+        raise TypeError("a and b must share one of the dtypes f32/f16/bf16")
+    if a.dim() not in (2, 3) or b.dim() not in (2, 3) or (a.dim() == 2 and b.dim() == 2):
+        raise ValueError("a is (E, M, K) or (M, K), b is (E, N, K) or (N, K), and one of them must carry the batch")
+    e = a.shape[0] if a.dim() == 3 else b.shape[0]
+    if a.dim() == 3 and b.dim() == 3:
+        assert a.shape[0] == b.shape[0], "The batch dimensions of the A and B tensors must match."
+    m, k = a.shape[-2:]
+    n, kb = b.shape[-2:]
+    assert k == kb, "The K dimension of the A and B tensors must match."
+    if c is None:
+        assert beta == 0.0, "beta != 0 needs an existing C"
+        c = torch.empty((e, m, n), dtype=out_dtype or torch.float32, device=a.device)
+    assert tuple(c.shape) == (e, m, n), "The dimensions of the C tensor must be (batch, M, N)."
+    assert alpha != 0, "The alpha must not be zero."
+    flags = (_lib.GEMM_RELU if relu else 0) | (_lib.GEMM_FORCE_GENERIC if force_generic else 0)
+    check(lib.sp_gemm_abt_batched(_lib.DTYPES[a.dtype], _lib.DTYPES[c.dtype], ptr(a, name="a"), ptr(b, name="b"),
+                                  ptr(c, name="c"), ptr(bias, torch.float32, "bias"), m, n, k, e,
+                                  m * k if a.dim() == 3 else 0, n * k if b.dim() == 3 else 0, m * n, float(alpha),
+                                  float(beta), flags, stream_ptr()))
+    return c
+
+
 def _transposed(x):
     """Materialise x^T with the library's transpose kernel (4-byte elements only)."""
     if x.dtype != torch.float32:

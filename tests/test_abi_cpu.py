@@ -56,6 +56,18 @@ def test_gemm_argument_errors(L):
     assert lib.sp_gemm_abt(*args(alpha=0.0)) == -5 and "alpha must not be zero" in _err(L)
 
 
+def test_batched_gemm_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x1000)
+    call = lambda **kw: lib.sp_gemm_abt_batched(0, 0, p, p, p, None, 64, 64, 64, kw.get("batch", 4), kw.get("sa", 0),
+                                                kw.get("sb", 4096), kw.get("sc", 4096), 1.0, 0.0, 0, None)
+    assert call(batch=0) == -2 and call(batch=70000) == -2
+    assert call(sc=100) == -5 and "overlap" in _err(L)
+    assert call(sb=4097) == -3
+    assert call(sa=-4) == -3
+    assert lib.sp_gemm_abt_batched(0, 0, None, p, p, None, 64, 64, 64, 2, 0, 4096, 4096, 1.0, 0.0, 0, None) == -1
+
+
 def test_row_argument_errors(L):
     lib = L.lib
     p = C.c_void_p(0x2000)

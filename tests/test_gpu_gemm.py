@@ -194,3 +194,31 @@ def test_device_and_kernel_info():
     assert k["threads_per_block"] == 512 and k["vgprs"] > 64
     with pytest.raises(_lib.SpiralError):
         _lib.kernel_info("no_such_kernel")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("e,m,n,k,shared", [(16, 1536, 64, 64, "a"), (5, 256, 256, 128, None), (3, 100, 24, 40, "a"),
+                                            (4, 128, 512, 64, "b"), (40, 64, 64, 64, "a")])
+def test_batched(MM, dtype, e, m, n, k, shared):
+    """One launch for a whole ensemble (`matmul_ensemble`: E weight matrices, one shared input)."""
+    announce("gemm batched %s e=%d %dx%dx%d shared=%s" % (dtype, e, m, n, k, shared))
+    rng = np.random.default_rng(e * 1000 + m + n + k)
+    a = ogemm.round_to(rng.standard_normal(((1 if shared == "a" else e), m, k), dtype=np.float32) / np.float32(np.sqrt(k)), dtype)
+    b = ogemm.round_to(rng.standard_normal(((1 if shared == "b" else e), n, k), dtype=np.float32) / np.float32(np.sqrt(k)), dtype)
+    t = TORCH[dtype]
+    ad = dev(a[0] if shared == "a" else a, t)
+    bd = dev(b[0] if shared == "b" else b, t)
+    bias = rng.standard_normal(n, dtype=np.float32)
+    c0 = rng.standard_normal((e, m, n), dtype=np.float32)
+    cd = dev(c0)
+    got = host(MM.matmul_abt_batched(ad, bd, c=cd, alpha=0.5, beta=2.0, bias=dev(bias), relu=True))
+    for i in range(e):
+        want = ogemm.gemm_abt(a[0 if shared == "a" else i], b[0 if shared == "b" else i], c=c0[i], alpha=0.5, beta=2.0,
+                              bias=bias, relu=True)
+        assert ogemm.rel_frobenius(got[i], want) < TOL[dtype]
+    # every member equals the plain launch on its own operands, bit for bit
+    one = host(MM.matmul_abt(dev(a[0], t), dev(b[0], t)))
+    many = host(MM.matmul_abt_batched(ad, bd))
+    assert (many[0] == one).all()
+    with pytest.raises(AssertionError, match="K dimension"):
+        MM.matmul_abt_batched(ad, dev(np.zeros((e, n, k + 8), dtype=np.float32), t))
