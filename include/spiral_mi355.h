@@ -177,6 +177,11 @@ typedef struct {
     int32_t threads_per_block;   /* reference: 256 */
     int32_t blocks_per_grid;     /* reference: 24 (RTX 4060) or 112 (H100), corecuda/base.spi:14-42 */
     int32_t rows_per_block;      /* SP_PHILOX_LAYER only: rows of one block's slice */
+    int64_t member_rows;         /* 0, or: the rows are `rows / member_rows` stacked runs of the same op (the
+                                    members of an ensemble evaluated in one launch); row r then draws what row
+                                    r % member_rows of a run starting at offset + (r / member_rows) * member_draws
+                                    would draw */
+    uint64_t member_draws;       /* draws every thread consumes per run: all sampling nodes of the graph */
 } sp_philox_t;
 
 /*

@@ -43,6 +43,8 @@ struct RowArgs {
     int blocks;
     int rows_per_block;
     unsigned long long draw_offset;
+    long member_rows;                  // 0: one run; else the rows are stacked runs of member_rows rows each
+    unsigned long long member_draws;   // extra draw offset per run
 };
 
 // Philox4x32-10 (Salmon et al., SC'11) with cuRAND's counter layout: key = seed, counter =
@@ -72,6 +74,11 @@ __device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigne
 // the row draws once per element it holds and the draw attached to column 0 wins
 // (ml/primitives.spi:786-791), i.e. the first draw of the row's lane 0 in that row-iteration.
 __device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r) {
+    unsigned long long draw_offset = a.draw_offset;
+    if (a.member_rows > 0) {              // stacked runs (ensemble members): each restarts the row walk, later in the stream
+        draw_offset += (unsigned long long)(r / a.member_rows) * a.member_draws;
+        r = r % a.member_rows;
+    }
     const long t = a.cols / 4;            // threads per row in the reference
     const long per_iter = a.tpb / t;      // rows per block-iteration
     unsigned long long sub, group;
@@ -92,7 +99,7 @@ __device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r)
         group = rb / per_iter;
     }
     // the generator is `draw_offset` draws in; this row uses the first draw of its 4-draw group
-    return philox_uniform(a.seed, sub, group + a.draw_offset / 4, (int)(a.draw_offset % 4));
+    return philox_uniform(a.seed, sub, group + draw_offset / 4, (int)(draw_offset % 4));
 }
 
 // exp(x) = 2^(x * log2 e) on the hardware exp2 unit; relative error about 1e-6 for |x| < 20.
@@ -688,12 +695,18 @@ static int set_philox(RowArgs& a, const sp_philox_t* philox, int64_t rows, int64
                     philox->threads_per_block, (long long)t);
     if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
         return fail(SP_ERR_ARG, "%s: blocks_per_grid must be positive", fn);
-    if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || rows % philox->rows_per_block != 0))
-        return fail(SP_ERR_ARG, "%s: rows_per_block (%d) must be positive and divide rows (%lld)", fn,
-                    philox->rows_per_block, (long long)rows);
+    if (philox->member_rows < 0 || (philox->member_rows > 0 && rows % philox->member_rows != 0))
+        return fail(SP_ERR_ARG, "%s: member_rows (%lld) must divide rows (%lld)", fn, (long long)philox->member_rows,
+                    (long long)rows);
+    const int64_t run_rows = philox->member_rows > 0 ? philox->member_rows : rows;
+    if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || run_rows % philox->rows_per_block != 0))
+        return fail(SP_ERR_ARG, "%s: rows_per_block (%d) must be positive and divide the rows of a run (%lld)", fn,
+                    philox->rows_per_block, (long long)run_rows);
     a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
     a.blocks = philox->blocks_per_grid; a.rows_per_block = philox->rows_per_block;
     a.draw_offset = philox->offset;
+    a.member_rows = philox->member_rows;
+    a.member_draws = philox->member_draws;
     return SP_OK;
 }
 

@@ -29,7 +29,8 @@ class SpiralError(RuntimeError):
 
 class PhiloxConfig(C.Structure):
     _fields_ = [("seed", C.c_uint64), ("offset", C.c_uint64), ("mode", C.c_int32), ("threads_per_block", C.c_int32),
-                ("blocks_per_grid", C.c_int32), ("rows_per_block", C.c_int32)]
+                ("blocks_per_grid", C.c_int32), ("rows_per_block", C.c_int32), ("member_rows", C.c_int64),
+                ("member_draws", C.c_uint64)]
 
 
 class DeviceInfo(C.Structure):

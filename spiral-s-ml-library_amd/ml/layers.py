@@ -628,9 +628,164 @@ def _fused_plan(model):
     return (node, weights, top, head_ops[top.f]) if ok else None
 
 
-def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True):
+def _sampling_draws(w, cols):
+    """32-bit draws one sampling node takes from every thread's generator: 4 per row-iteration."""
+    rows_per_iteration = THREADS_PER_BLOCK // (cols // 4)
+    return 4 * ((w + rows_per_iteration - 1) // rows_per_iteration)
+
+
+def _batchable_key(model, sizes):
+    """The key of `sizes` if the whole loop over it can run as one batched pass: a single key that the
+    graph only uses to index leading dimensions (`apply key tensor`)."""
+    if len(sizes) != 1:
+        return None
+    (key,) = sizes
+    ok = [True]
+
+    def f(k, under_apply=False):
+        if isinstance(k, KeyScalar):
+            ok[0] = ok[0] and under_apply and k.key == key
+        elif isinstance(k, (BlockMap, BlockRowMap, BlockRowReduce, BlockRowMapReduce)):
+            f(k.a)
+            if k.out is not None:
+                f(k.out)
+        elif isinstance(k, Apply):
+            f(k.a)
+            f(k.b, True)
+        elif isinstance(k, (BlockMatmul, Pair, Zip)):
+            f(k.a)
+            f(k.b)
+        elif isinstance(k, (Fst, Snd, KeyGraph)):
+            f(k.x)
+
+    f(model.graph)
+    return key if ok[0] else None
+
+
+def _graph_run_batched(model, key, count, ls):
+    """`loop.linear {key=count} fun indices => graph_run_device m ls indices` (ml/layers.spi:343-344) as ONE
+    pass: `apply key t` yields the whole tensor, every node downstream works on `count` stacked members
+    (temporaries outside the workspace arena, which is sized for one member), matmuls become one
+    strided-batched launch, and sampling nodes draw for member e what the e-th sequential run would."""
+    data, dims = model.data, model.dims
+    tmp = model.__dict__.setdefault("_batched_tmp", {})
+
+    def count_draws(k):
+        if isinstance(k, (BlockRowReduce, BlockRowMapReduce)):
+            sampling = isinstance(k, BlockRowMapReduce) or k.f == "discrete_sample"
+            _, w, cols = get_dim(dims, k.a).dim
+            return count_draws(k.a) + (_sampling_draws(w, cols) if sampling else 0)
+        if isinstance(k, (BlockMap, BlockRowMap)):
+            return count_draws(k.a)
+        if isinstance(k, (BlockMatmul, Pair, Zip)):
+            return count_draws(k.a) + count_draws(k.b)
+        if isinstance(k, (Fst, Snd, KeyGraph)):
+            return count_draws(k.x)
+        if isinstance(k, Apply):
+            return count_draws(k.a)
+        return 0
+
+    draws_per_run = count_draws(model.graph)
+
+    def extract_current(node):
+        for x in data:
+            if node in x["partition"]:
+                return _from_offsets(x["array"], x["partition"][node])
+        raise KeyError("Cannot find the offset in the dictionaries for node %r." % (node,))
+
+    def stacked(t, spec):
+        return t.dim() == len(spec.dim) + 1
+
+    def out_for(node, batched):
+        if getattr(node, "out", None) is not None:
+            return loop(node.out)
+        if not batched:
+            return extract_current(node)
+        if node not in tmp:
+            spec = get_dim_pair(dims, node)
+            device = data[workspace_id()]["array"].device
+            make = lambda sp: torch.empty((count,) + sp.dim, dtype=sp.dtype, device=device)
+            tmp[node] = make(spec) if isinstance(spec, TensorSpec) else tuple(make(sp) for sp in spec)
+        return tmp[node]
+
+    def rng(a, batched):
+        q, w, cols = a.shape[-3:]
+        cfg = _prim.philox(_lib.PHILOX_LAYER, seed=ls.seed, threads_per_block=THREADS_PER_BLOCK, blocks_per_grid=q,
+                           rows_per_block=w, offset=ls.draws, member_rows=q * w if batched else 0,
+                           member_draws=draws_per_run)
+        ls.draws += _sampling_draws(w, cols)
+        return cfg
+
+    def loop(graph):
+        if isinstance(graph, BlockMap):
+            a = loop(graph.a)
+            out = out_for(graph, stacked(a, get_dim(dims, graph.a)))
+            assert out.shape == a.shape, "a batched input needs a batched output tensor"
+            _prim.map(graph.f, a, out)
+            return out
+        if isinstance(graph, BlockRowMap):
+            a = loop(graph.a)
+            out = out_for(graph, stacked(a, get_dim(dims, graph.a)))
+            assert out.shape == a.shape, "a batched input needs a batched output tensor"
+            _prim._row_map(_prim._ROW_OPS[graph.f], _flat(a), _flat(out), graph.size)
+            return out
+        if isinstance(graph, BlockRowReduce):
+            a = loop(graph.a)
+            batched = stacked(a, get_dim(dims, graph.a))
+            out = out_for(graph, batched)
+            assert out.shape == a.shape[:-1], "a batched input needs a batched output tensor"
+            if graph.f == "argmax":
+                _prim.row_ops(_flat(a), want=("argmax",), into={"argmax": out.reshape(-1)})
+            elif graph.f == "max":
+                _prim.row_ops(_flat(a), want=("rowmax",), into={"rowmax": out.reshape(-1)})
+            elif graph.f == "binarize":
+                _prim.binarize(_flat(a), graph.arg, out=out.reshape(-1))
+            else:
+                _prim._sample(_lib.ROW_IDENTITY, _flat(a), rng=rng(a, batched), want_probs=False,
+                              sample_out=out.reshape(-1))
+            return out
+        if isinstance(graph, BlockRowMapReduce):
+            a = loop(graph.a)
+            batched = stacked(a, get_dim(dims, graph.a))
+            out_map, out_reduce = out_for(graph, batched)
+            assert out_map.shape == a.shape, "a batched input needs batched output tensors"
+            _prim._sample(_ROW_MAP_REDUCES[graph.f], _flat(a), rng=rng(a, batched), mask_size=graph.size,
+                          probs_out=_flat(out_map), sample_out=out_reduce.reshape(-1))
+            return out_map, out_reduce
+        if isinstance(graph, BlockMatmul):
+            a, b = loop(graph.a), loop(graph.b)
+            ab, bb = stacked(a, get_dim(dims, graph.a)), stacked(b, get_dim(dims, graph.b))
+            out = out_for(graph, ab or bb)
+            if not (ab or bb):
+                _matmul.matmul_abt(_flat(a), b, c=_flat(out), alpha=1.0, beta=0.0)
+            else:
+                a3 = a.reshape(count, -1, a.shape[-1]) if ab else _flat(a)
+                _matmul.matmul_abt_batched(a3, b, c=out.reshape(count, -1, out.shape[-1]), alpha=1.0, beta=0.0)
+            return out
+        if isinstance(graph, (Zip, Pair)):
+            return loop(graph.a), loop(graph.b)
+        if isinstance(graph, Fst):
+            return loop(graph.x)[0]
+        if isinstance(graph, Snd):
+            return loop(graph.x)[1]
+        if isinstance(graph, Layer):
+            return extract_current(graph)
+        if isinstance(graph, Apply):
+            t = loop(graph.a)
+            assert t.shape[0] == count, "the key's size must be the tensor's leading dimension"
+            return t          # the key is the batch: all members at once
+        if isinstance(graph, KeyGraph):
+            return loop(graph.x)
+        raise TypeError("unknown graph node %r" % (graph,))
+
+    return loop(model.graph)
+
+
+def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batched=True):
     """Runs the graph for every combination of the key indices in `sizes`, e.g. {"ensemble": 16}
-    (ml/layers.spi:336-344).  Uniforms come from the reference's per-thread Philox streams."""
+    (ml/layers.spi:336-344).  Uniforms come from the reference's per-thread Philox streams.  A loop over
+    one key that only indexes leading dimensions runs as a single batched pass with the same results
+    (`batched=False` keeps the member-by-member loop)."""
     ls = create_layer_state(seed)
     sizes = sizes or {}
     plan = _fused_plan(model) if fuse and not sizes else None
@@ -643,6 +798,10 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True):
         u = _prim.philox_uniforms(ls.rng(q, w, cols), q * w, cols)
         mlp_forward(_flat(x), ws, head=head, u=u, mask_size=top.size, policy_out=_flat(probs),
                     action_out=action.reshape(-1))
+        return
+    key = _batchable_key(model, sizes) if batched and sizes else None
+    if key is not None and sizes[key] > 1:
+        _graph_run_batched(model, key, sizes[key], ls)
         return
     keys = list(sizes)
     for combo in itertools.product(*[range(sizes[k]) for k in keys]):

@@ -112,11 +112,12 @@ def argmax(x):
 
 
 def philox(mode=_lib.PHILOX_BLOCK, seed=CONSTANT_SEED, threads_per_block=THREADS_PER_BLOCK,
-           blocks_per_grid=BLOCKS_PER_GRID, rows_per_block=0, offset=0):
+           blocks_per_grid=BLOCKS_PER_GRID, rows_per_block=0, offset=0, member_rows=0, member_draws=0):
     """The reference's device RNG: Philox4_32_10 seeded like `random.init {seed subsequence offset=0}`
     (ml/primitives.spi:927,1014; corecuda/random.spi:22-32).  `offset` = draws every thread's generator
-    has already handed out (a graph run keeps one state per thread across its sampling nodes)."""
-    return PhiloxConfig(seed, offset, mode, threads_per_block, blocks_per_grid, rows_per_block)
+    has already handed out (a graph run keeps one state per thread across its sampling nodes); member_rows /
+    member_draws describe stacked runs (ensemble members evaluated in one launch), see sp_philox_t."""
+    return PhiloxConfig(seed, offset, mode, threads_per_block, blocks_per_grid, rows_per_block, member_rows, member_draws)
 
 
 def philox_uniforms(rng, rows, cols, out=None):

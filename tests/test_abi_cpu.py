@@ -81,14 +81,16 @@ def test_row_argument_errors(L):
     assert lib.sp_row_map_f32(L.ROW_MASKED_SOFTMAX, p, p, 8, 8, 0, None) == -5
     assert lib.sp_row_map_f32(L.ROW_MASKED_SOFTMAX, p, p, 8, 8, 9, None) == -5
     assert lib.sp_row_map_i32(L.ROW_SOFTMAX, p, p, 8, 8, None) == -5
-    ph = L.PhiloxConfig(1, 0, L.PHILOX_BLOCK, 256, 24, 0)
+    ph = L.PhiloxConfig(1, 0, L.PHILOX_BLOCK, 256, 24, 0, 0, 0)
     assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, None, None, None, None, p, None, 8, 8, 0, None) == -5
     assert lib.sp_row_sample(L.ROW_SOFTMAX, p, p, C.byref(ph), None, None, None, p, None, 8, 8, 0, None) == -5
     assert lib.sp_row_sample(L.ROW_LN_L2, p, p, None, None, None, None, p, None, 8, 8, 0, None) == -5
-    bad = L.PhiloxConfig(1, 0, L.PHILOX_BLOCK, 100, 24, 0)  # 100 threads is not a multiple of cols/4 = 16
+    bad = L.PhiloxConfig(1, 0, L.PHILOX_BLOCK, 100, 24, 0, 0, 0)  # 100 threads is not a multiple of cols/4 = 16
     assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, C.byref(bad), None, None, None, p, None, 8, 64, 0, None) == -5
-    layer = L.PhiloxConfig(1, 0, L.PHILOX_LAYER, 256, 24, 3)  # 3 rows per block do not divide 8 rows
+    layer = L.PhiloxConfig(1, 0, L.PHILOX_LAYER, 256, 24, 3, 0, 0)  # 3 rows per block do not divide 8 rows
     assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, C.byref(layer), None, None, None, p, None, 8, 64, 0, None) == -5
+    members = L.PhiloxConfig(1, 0, L.PHILOX_LAYER, 256, 24, 2, 3, 16)   # runs of 3 rows do not divide 8 rows
+    assert lib.sp_row_sample(L.ROW_SOFTMAX, p, None, C.byref(members), None, None, None, p, None, 8, 64, 0, None) == -5
     assert lib.sp_row_get_prob(L.ROW_IDENTITY, p, None, p, 8, 8, 0, None) == -1
     assert lib.sp_row_get_prob(L.ROW_INCLUSIVE_SCAN, p, p, p, 8, 8, 0, None) == -5
     assert lib.sp_row_get_prob(L.ROW_MASKED_REGRET_MATCHING, p, p, p, 8, 8, 0, None) == -5

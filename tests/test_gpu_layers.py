@@ -96,6 +96,30 @@ def test_ensemble_graphs(L, ensemble, size, deep):
             assert (idx[e] < size).all() and (probs[e][..., size:] == 0).all()
 
 
+def test_batched_ensemble_pass_equals_member_by_member_loop(L):
+    """`graph_run_host model {ensemble}` as one batched pass (strided-batched GEMMs, stacked row ops, per-member
+    Philox offsets) gives bit for bit what the loop over the members gives."""
+    announce("layers batched ensemble pass")
+    ensemble = 6
+    out = L.pair(L.apply("ensemble", L.input("output_probs", (ensemble, Q, 64, 64))),
+                 L.apply("ensemble", L.input("output_indices", (ensemble, Q, 64), "int")))
+    x = L.pipe(L.input("input", (Q, 64, 64)), L.matmul_ensemble((ensemble, 64, 64)), L.ln_l2, L.relu,
+               L.matmul_ensemble((ensemble, 64, 32)), L.tanh, L.matmul((32, 64)))
+    g = L.masked_softmax_and_discrete_sample_(17, out, x)
+    m = L.create_model(g)
+    L.pass_init(m)
+    fill(L.key_extract(m, "input"), np.random.default_rng(8))
+    assert L._batchable_key(m, {"ensemble": ensemble}) == "ensemble"
+    L.graph_run_host(m, {"ensemble": ensemble}, batched=False)
+    want_p, want_i = host(L.key_extract(m, "output_probs")).copy(), host(L.key_extract(m, "output_indices")).copy()
+    L.key_extract(m, "output_probs").zero_()
+    L.key_extract(m, "output_indices").zero_()
+    L.graph_run_host(m, {"ensemble": ensemble})
+    assert (host(L.key_extract(m, "output_probs")) == want_p).all()
+    assert (host(L.key_extract(m, "output_indices")) == want_i).all()
+    assert (want_i < 17).all() and len(np.unique(want_i)) > 5
+
+
 def test_other_heads_and_maps(L):
     announce("layers heads and maps")
     x = L.input("input", (Q, 8, 32))
