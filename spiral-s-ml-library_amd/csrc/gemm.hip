@@ -249,23 +249,35 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // waves w and w + NW / 2 share a SIMD when there are 8 of them; with 4 this splits the SIMDs into two groups
+    const bool dma_first = __builtin_amdgcn_readfirstlane(wave) < NW / 2;
     for (int kt = 0; kt + 1 < nk; ++kt) {
         first_three_steps();
         asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         __syncthreads();
         toggle_stage();
+        // The two waves of a SIMD take turns: a wave issuing its DMA instructions waits at the texture
+        // path's queue (one 1 KiB instruction per ~16 cycles, 8 waves x NI of them per tile: measured
+        // ~600 cycles per wave and tile) and issues no MFMA meanwhile, so one wave of each pair fetches
+        // before the last k-step's MFMAs and the other one after them.  Only the DMA issue sits in the
+        // (wave-uniform) branches: MFMAs in both arms would make the compiler copy the accumulators.
+        auto issue_dma = [&]() {
+            if (kt + 2 < nk) {
+                const unsigned stage_off = (kt & 1) * STAGE_BYTES;
+#pragma unroll
+                for (int q = 0; q < NI; ++q) {
+                    src[q] += ROW_BYTES;
+                    dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
+                }
+            }
+        };
+        if (dma_first) issue_dma();
+        __builtin_amdgcn_sched_barrier(0);
         load_frags(0, fa[0], fb[0]);
         __builtin_amdgcn_sched_barrier(0);
         mma(fa[1], fb[1]);
         __builtin_amdgcn_sched_barrier(0);
-        if (kt + 2 < nk) {
-            const unsigned stage_off = (kt & 1) * STAGE_BYTES;
-#pragma unroll
-            for (int q = 0; q < NI; ++q) {
-                src[q] += ROW_BYTES;
-                dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
-            }
-        }
+        if (!dma_first) issue_dma();
     }
     first_three_steps();
     mma(fa[1], fb[1]);
