@@ -248,8 +248,12 @@ def main():
     # cannot be read from inside this process); profiles/traffic.json holds the scaled figure
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
-            if head["roofline"] is not None:
-                head["roofline"]["traffic"] = json.load(f)["headline"]["traffic_bytes"]
+            measured = json.load(f)
+        if head["roofline"] is not None:
+            head["roofline"]["traffic"] = measured["headline"]["traffic_bytes"]
+        for name, res in extra.items():
+            if name in measured and res.get("roofline") is not None:
+                res["roofline"]["traffic"] = measured[name]["traffic_bytes"]
     except (OSError, KeyError, ValueError):
         pass
 
