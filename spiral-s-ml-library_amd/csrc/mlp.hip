@@ -604,25 +604,33 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
                         acc[t] = mfma((c2 == 0 && cc == 0 && sp == 0) ? zero4 : acc[t], w[cc][sp][t], act[2 * (2 * c2 + cc) + sp]);
         }
     }
-    __syncthreads();                                    // every wave has read its last weights: reuse stage 0
-    float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
     const float* bias = a.b[NL - 1];
+    const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
+    if (NOUT <= 8) {
+        // narrow heads never leave the registers: in tiles 0 and 1 lane (j, q = 0) holds columns 0..3 and
+        // 4..7 of batch row j, and those lanes are lanes 0..15 of the wave
+        float p[8];
 #pragma unroll
-    for (int t = 0; t < MLP_MAX_OUT / 16; ++t) {
-        f32x4 v = acc[t];
-        if (bias != nullptr) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r)
-                if (tile_col(t) + r < NOUT) v[r] += bias[tile_col(t) + r];
+        for (int n = 0; n < 8; ++n) {
+            p[n] = acc[n >> 2][n & 3];
+            if (bias != nullptr && n < NOUT) p[n] += bias[n];
         }
-        *reinterpret_cast<f32x4*>(head_rows + j * MLP_MAX_OUT + tile_col(t)) = v;
-    }
-    // ---- head: lanes 0..15 of every wave own one batch row each (the staging is wave private) ----
-    if (lane < 16 && row_ok) {
-        const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
-        float* p = head_rows + lane * MLP_MAX_OUT;
-        if (NOUT <= 8) head_row<8>(a, p, row, NOUT, limit, u_row);
-        else head_row<MLP_MAX_OUT>(a, p, row, NOUT, limit, u_row);
+        if (lane < 16 && row_ok) head_row<8>(a, p, row, NOUT, limit, u_row);
+    } else {
+        __syncthreads();                                    // every wave has read its last weights: reuse stage 0
+        float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
+#pragma unroll
+        for (int t = 0; t < MLP_MAX_OUT / 16; ++t) {
+            f32x4 v = acc[t];
+            if (bias != nullptr) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    if (tile_col(t) + r < NOUT) v[r] += bias[tile_col(t) + r];
+            }
+            *reinterpret_cast<f32x4*>(head_rows + j * MLP_MAX_OUT + tile_col(t)) = v;
+        }
+        // lanes 0..15 of every wave own one batch row each (the staging is wave private)
+        if (lane < 16 && row_ok) head_row<MLP_MAX_OUT>(a, head_rows + lane * MLP_MAX_OUT, row, NOUT, limit, u_row);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the dummy DMAs (they land in their own KiB) before the LDS is released
 }
