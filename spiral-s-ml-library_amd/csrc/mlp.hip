@@ -54,6 +54,7 @@ struct MlpArgs {
     long batch;
     int head;
     int mask_size;
+    int k0, nout;        // dims[0] and dims[n_layers] once more, so that a kernel needs no dependent load for them
 };
 
 // max(x, 0) and rounding of two f32 values to the 16-bit storage type, packed into one register
@@ -84,63 +85,76 @@ __device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane
 // Head of one batch row: optional softmax and/or regret matching over the columns j < limit, then
 // local_discrete_sampling (ml/primitives.spi:782-798) with sequential prefix sums.  `src` holds the
 // row's N last-layer outputs; MAXN bounds N at compile time so that narrow heads stay in registers.
+// Columns past `limit` enter the softmax as -inf and leave it as exact zeros, columns past N are zeros
+// from the start: sums over all MAXN columns then equal the sums over the valid ones bit for bit, and
+// the loops need no per-column conditions.
+struct HeadOut {
+    float* policy;
+    int* action;
+    float* logits;
+    int head;
+};
+__device__ __forceinline__ HeadOut head_out(const MlpArgs& a) { return HeadOut{a.policy, a.action, a.logits, a.head}; }
+
 template <int MAXN>
-__device__ __forceinline__ void head_row(const MlpArgs& a, const float* src, long row, int N, int limit, float u) {
+__device__ __forceinline__ void head_row(const HeadOut& o, const float* src, long row, int N, int limit, float u) {
     float p[MAXN];
 #pragma unroll
     for (int n = 0; n < MAXN; ++n) p[n] = n < N ? src[n] : 0.f;
-    if (a.logits != nullptr) {
+    if (o.logits != nullptr) {
 #pragma unroll
         for (int n = 0; n < MAXN; ++n)
-            if (n < N) a.logits[row * N + n] = p[n];
+            if (n < N) o.logits[row * N + n] = p[n];
     }
     // exp on the hardware exp2 unit and one reciprocal per normalisation: a 16-lane serial head is
     // otherwise a visible part of a forward pass that takes a few microseconds
-    if (a.head == SP_HEAD_SOFTMAX || a.head == SP_HEAD_SOFTMAX_RM) {
+    if (o.head == SP_HEAD_SOFTMAX || o.head == SP_HEAD_SOFTMAX_RM) {
         float m = -__builtin_inff();
 #pragma unroll
-        for (int n = 0; n < MAXN; ++n)
-            if (n < limit) m = fmaxf(m, p[n]);
+        for (int n = 0; n < MAXN; ++n) {
+            p[n] = n < limit ? p[n] : -__builtin_inff();
+            m = fmaxf(m, p[n]);
+        }
         float s = 0.f;
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) {
-            p[n] = n < limit ? __builtin_amdgcn_exp2f((p[n] - m) * 1.44269504088896340736f) : 0.f;
-            if (n < N) s = s + p[n];
+            p[n] = __builtin_amdgcn_exp2f((p[n] - m) * 1.44269504088896340736f);
+            s = s + p[n];
         }
         const float inv = 1.f / s;
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) p[n] = p[n] * inv;
     }
-    if (a.head == SP_HEAD_REGRET_MATCHING || a.head == SP_HEAD_SOFTMAX_RM) {
+    if (o.head == SP_HEAD_REGRET_MATCHING || o.head == SP_HEAD_SOFTMAX_RM) {
         float s = 0.f;
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) {
             p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
-            if (n < N) s = s + p[n];
+            s = s + p[n];
         }
         const float inv_len = 1.f / (float)limit;
         const float inv = s != 0.f ? 1.f / s : 0.f;
 #pragma unroll
-        for (int n = 0; n < MAXN; ++n) p[n] = n < limit ? (s != 0.f ? p[n] * inv : inv_len) : 0.f;
+        for (int n = 0; n < MAXN; ++n) p[n] = s != 0.f ? p[n] * inv : (n < limit ? inv_len : 0.f);
     }
 #pragma unroll
     for (int n = 0; n < MAXN; ++n)
-        if (n < N) a.policy[row * N + n] = p[n];
-    if (a.action != nullptr) {
+        if (n < N) o.policy[row * N + n] = p[n];
+    if (o.action != nullptr) {
         float run = 0.f, m = -__builtin_inff();
         float cdf[MAXN];
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) {
-            if (n < N) run = run + p[n];
+            run = run + p[n];
             cdf[n] = run;
-            if (n < N && p[n] > 0.f) m = fmaxf(m, run);
+            if (p[n] > 0.f) m = fmaxf(m, run);
         }
         const float thr = u * m;
         int pick = INT_MAX_;
 #pragma unroll
         for (int n = MAXN - 1; n >= 0; --n)
-            if (n < N && p[n] > 0.f && cdf[n] >= thr) pick = n;
-        a.action[row] = pick;
+            if (p[n] > 0.f && cdf[n] >= thr) pick = n;
+        o.action[row] = pick;
     }
 }
 
@@ -346,8 +360,8 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
         const int limit = a.mask_size > 0 ? a.mask_size : N;
         float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs
         const float u = a.action != nullptr ? a.u[row] : 1.f;
-        if (N <= 8) head_row<8>(a, p, row, N, limit, u);      // narrow heads run in registers
-        else head_row<MLP_MAX_OUT>(a, p, row, N, limit, u);
+        if (N <= 8) head_row<8>(head_out(a), p, row, N, limit, u);      // narrow heads run in registers
+        else head_row<MLP_MAX_OUT>(head_out(a), p, row, N, limit, u);
     }
 }
 
@@ -389,25 +403,50 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int j = lane & 15, q = lane >> 4;
     const long row = (long)blockIdx.x * ROWS + wave * 16 + j;
-    const bool row_ok = row < a.batch;
     const unsigned lds_base = (unsigned)(size_t)lds;
     const unsigned dummy_dst = lds_base + MLP_STAGES * MLP_STAGE_BYTES;
-    const int K0 = a.dims[0], NL = a.n_layers, NOUT = a.dims[a.n_layers];
+    // Every scalar the kernel needs is read from the argument block HERE, in one round trip: a read
+    // at the point of use costs a few hundred cycles each time, and the wait for it also drains the
+    // LDS reads in flight.  The per-layer pointers, which the layer loop indexes at run time, travel
+    // in two registers instead (lane l holds weights[l] and biases[l]) and are picked by v_readlane.
+    const int K0 = a.k0, NL = a.n_layers, NOUT = a.nout;
+    const unsigned char* const x_ptr = (const unsigned char*)a.x;
+    const unsigned char* const w0_ptr = (const unsigned char*)a.w[0];
+    const unsigned char* const w1_ptr = (const unsigned char*)a.w[1];
+    const float* const b0_ptr = a.b[0];
+    const float* const u_ptr = a.u;
+    const long batch = a.batch;
+    const HeadOut out = head_out(a);
+    const int mask_size = a.mask_size;
+    asm volatile("" ::"s"(K0), "s"(NL), "s"(NOUT), "s"(x_ptr), "s"(w0_ptr), "s"(w1_ptr), "s"(b0_ptr), "s"(u_ptr), "s"(batch),
+                 "s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(mask_size));
     const int n_chunks = C0 + 4 * (NL - 2) + 1;
+    u32x2 tab_w, tab_b;
+    {
+        const unsigned char* args = (const unsigned char*)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_w) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, w)) : "memory");
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_b) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, b)) : "memory");
+    }
+    auto table_ptr = [&](const u32x2& tab, int l) {
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)tab[0], l);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)tab[1], l);
+        return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
+    };
 
     // ---- the wave's input rows, requested before any weight so that they are the oldest loads;
     //      the row's uniform for the sampling head travels with them ----
+    const bool row_ok = row < batch;
     u32x4 act[H / 32];
     float u_row = 1.f;
     {
-        const unsigned char* xr = (const unsigned char*)a.x + (row_ok ? row : 0) * K0 * 2;
+        const unsigned char* xr = x_ptr + (row_ok ? row : 0) * K0 * 2;
 #pragma unroll
         for (int s = 0; s < H / 32; ++s) {
             const int k = 32 * s + 8 * q;
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(act[s]) : "v"(xr + (k < K0 ? k : 0) * 2) : "memory");
         }
-        if (a.u != nullptr)
-            asm volatile("global_load_dword %0, %1, off" : "=v"(u_row) : "v"(a.u + (row_ok ? row : 0)) : "memory");
+        if (u_ptr != nullptr)
+            asm volatile("global_load_dword %0, %1, off" : "=v"(u_row) : "v"(u_ptr + (row_ok ? row : 0)) : "memory");
     }
 
     // ---- per-lane source offsets, once ----
@@ -425,27 +464,31 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     }
 
     int pf = 0, pf_stage = 0;                        // next chunk to fetch and its ring stage
-    const unsigned char* pf_base = (const unsigned char*)a.w[0];
+    const unsigned char* pf_base = w0_ptr;
     unsigned pf_dst0 = lds_base;
     bool pf_last = false, pf_none = false;
     unsigned cur[PW];
-    auto prepare = [&]() {
+    // EARLY: one of the three fetches issued before the pointer table has landed; they read the first
+    // or the second layer, whose pointers are in scalar registers
+    auto prepare = [&](auto EARLY_) {
+        constexpr bool early = decltype(EARLY_)::value != 0;
+        auto layer_ptr = [&](int l) { return early ? (l == 0 ? w0_ptr : w1_ptr) : table_ptr(tab_w, l); };
         pf_dst0 = lds_base + pf_stage * MLP_STAGE_BYTES;
         pf_last = pf == n_chunks - 1;
         pf_none = pf >= n_chunks;
         if (pf < C0) {
-            pf_base = (const unsigned char*)a.w[0];
+            pf_base = w0_ptr;
             int k = pf * 64 + piece * 8;
             k = k <= K0 - 8 ? k : K0 - 8;
 #pragma unroll
             for (int m = 0; m < PW; ++m) cur[m] = off0[m] + (unsigned)(k * 2);
         } else if (pf < n_chunks - 1) {
             const int hl = (pf - C0) >> 2;
-            pf_base = (const unsigned char*)a.w[1 + hl] + ((pf - C0) & 3) * 128;
+            pf_base = layer_ptr(1 + hl) + ((pf - C0) & 3) * 128;
 #pragma unroll
             for (int m = 0; m < PW; ++m) cur[m] = offH[m];
         } else {
-            pf_base = (const unsigned char*)a.w[NL - 1];
+            pf_base = layer_ptr(NL - 1);
 #pragma unroll
             for (int m = 0; m < PW; ++m) cur[m] = offL[m];
         }
@@ -460,7 +503,7 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
         mlp_dma(pf_base, cur[m], __builtin_amdgcn_readfirstlane(dst));
     };
     auto fetch = [&]() {
-        prepare();
+        prepare(IC<1>{});
 #pragma unroll
         for (int m = 0; m < PW; ++m) issue(m);
     };
@@ -498,57 +541,101 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     };
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     f32x4 acc[H / 16];
-    // wait for the oldest chunk in flight, barrier, prepare the next fetch
-    auto chunk_sync = [&]() -> const unsigned char* {
+    // ---- the MFMA pipeline ----
+    // A chunk is 8 groups (output-tile quad g / 2, 32-wide k-step g % 2) of 4 operand reads + 4 MFMAs.
+    // The reads run D = RING - 1 groups ahead of the MFMAs, across chunk boundaries: with four waves on
+    // a compute unit an LDS read comes back after 250 cycles or more and a group's MFMAs take 64, so a
+    // short look-ahead leaves the matrix pipe waiting for every group.  (Seven groups ahead need 128
+    // registers, which 8-wave workgroups do not have; they look three ahead.)  Group g of a chunk lives
+    // in slot g % RING; when it starts, slot (g + D) % RING is free and receives group g + D of this
+    // chunk or, from g = 8 - D on, group g + D - 8 of the next one.  The next chunk must therefore have
+    // landed when group 8 - D starts: that is where the wave waits for its DMA, meets the others at the
+    // barrier (which also frees the stage of the previous chunk for the fetch three chunks ahead) and
+    // prepares that fetch.
+    constexpr int RING = NW == 4 ? 8 : 4;
+    constexpr int D = RING - 1;
+    constexpr int GSYNC = 8 - D;
+    u32x4 w[RING][4];
+    const unsigned char* st_cur = lds;
+    auto read_group = [&](const unsigned char* st, int g) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            w[g % RING][t] = *reinterpret_cast<const u32x4*>(st + frag_off[g & 1] + tile_off((g >> 1) * 4 + t));
+    };
+    // the first chunk: it has landed when only the two younger fetches are outstanding
+    auto first_sync = [&]() {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PW) : "memory");
         __syncthreads();
-        prepare();
-        const unsigned char* st = lds + stage * MLP_STAGE_BYTES;
-        stage = (stage + 1) & (MLP_STAGES - 1);
-        return st;
+        st_cur = lds;
+        stage = 1;
+#pragma unroll
+        for (int g = 0; g < D; ++g) read_group(st_cur, g);
     };
-    // all 16 output tiles x both 32-wide steps of chunk C (the layer's first chunk starts the
-    // accumulators from zero), software pipelined by hand: the weight pieces of group g + 2 are
-    // requested before the MFMAs of group g; one DMA instruction of the next fetch after every
-    // 8 / PW-th group
-    auto full_chunk = [&](auto C_) {
-        constexpr int c = decltype(C_)::value;
-        const unsigned char* st = chunk_sync();
-        auto read = [&](int t, int sp) { return *reinterpret_cast<const u32x4*>(st + frag_off[sp] + tile_off(t)); };
-        u32x4 w[3][4];
-#pragma unroll
-        for (int t = 0; t < 4; ++t) w[0][t] = read(t, 0);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) w[1][t] = read(t, 1);
+    // KIND 0..3: chunk KIND of a layer, i.e. K-columns 64 KIND .. + 63 for all 16 output tiles (chunk 0
+    // starts the accumulators from zero); KIND 4: the last layer, whose chunk holds the K-columns
+    // 64 s .. + 63 of all its (at most 64) outputs in slab s = g / 2 and accumulates into tiles 0..3.
+    // FIRST: the chunk behind first_sync (no earlier fetch is waiting for its last DMA instructions).
+    auto run_chunk = [&](auto KIND_, auto FIRST_) {
+        constexpr int kind = decltype(KIND_)::value;
+        constexpr bool first = decltype(FIRST_)::value != 0;
+        constexpr bool last = kind == 4;
+        const unsigned char* st_next = st_cur;
 #pragma unroll
         for (int g = 0; g < 8; ++g) {
-            if (g + 2 < 8) {
-#pragma unroll
-                for (int t = 0; t < 4; ++t) w[(g + 2) % 3][t] = read(((g + 2) >> 1) * 4 + t, (g + 2) & 1);
+            if (g + D < 8) {
+                read_group(st_cur, g + D);
+            } else if (!last) {
+                if (g == GSYNC) {
+                    // a bare s_barrier: __syncthreads() would first wait for the LDS reads in flight, which
+                    // is the pipeline this loop exists to keep full.  Nothing needs that wait: the DMA data is
+                    // covered by vmcnt, and a stage is only overwritten after its reads have fed MFMAs
+                    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(PW) : "memory");
+                    prepare(IC<0>{});
+                    st_next = lds + stage * MLP_STAGE_BYTES;
+                    stage = (stage + 1) & (MLP_STAGES - 1);
+                }
+                read_group(st_next, g + D - 8);
             }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                f32x4& d = acc[(g >> 1) * 4 + t];
-                d = mfma((c == 0 && (g & 1) == 0) ? zero4 : d, w[g % 3][t], act[2 * c + (g & 1)]);
+                if constexpr (last) {
+                    acc[t] = mfma(g == 0 ? zero4 : acc[t], w[g % RING][t], act[g]);
+                } else {
+                    f32x4& d = acc[(g >> 1) * 4 + t];
+                    d = mfma((kind == 0 && (g & 1) == 0) ? zero4 : d, w[g % RING][t], act[2 * kind + (g & 1)]);
+                }
             }
             __builtin_amdgcn_sched_barrier(0);
+            if (!last && !(first && g < GSYNC)) {
+                // the DMA instructions of the fetch prepared at group GSYNC go out one by one behind the
+                // groups from there to group GSYNC - 1 of the next chunk
+                const int gi = (g + 8 - GSYNC) & 7;
 #pragma unroll
-            for (int m = g * PW / 8; m < (g + 1) * PW / 8; ++m) issue(m);
+                for (int m = gi * PW / 8; m < (gi + 1) * PW / 8; ++m) issue(m);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        st_cur = st_next;
     };
+    // (the bias test is uniform and made once per layer, not once per register pair)
     auto next_activations = [&](const float* bias) {
+        auto convert = [&](auto HAS_BIAS_) {
 #pragma unroll
-        for (int s = 0; s < H / 32; ++s) {
-            f32x4 lo = acc[2 * s], hi = acc[2 * s + 1];
-            if (bias != nullptr) {   // uniform; only the two temporaries depend on it
-                lo += *reinterpret_cast<const f32x4*>(bias + tile_col(2 * s));
-                hi += *reinterpret_cast<const f32x4*>(bias + tile_col(2 * s + 1));
+            for (int s = 0; s < H / 32; ++s) {
+                f32x4 lo = acc[2 * s], hi = acc[2 * s + 1];
+                if constexpr (decltype(HAS_BIAS_)::value != 0) {
+                    // (a pointer that came out of a register table must be told that it points to global memory)
+                    typedef const __attribute__((address_space(1))) f32x4* gptr;
+                    lo += *(gptr)(unsigned long long)(bias + tile_col(2 * s));
+                    hi += *(gptr)(unsigned long long)(bias + tile_col(2 * s + 1));
+                }
+                act[s] = u32x4{pack_relu2<DT>(lo[0], lo[1]), pack_relu2<DT>(lo[2], lo[3]), pack_relu2<DT>(hi[0], hi[1]),
+                               pack_relu2<DT>(hi[2], hi[3])};
             }
-            act[s] = u32x4{pack_relu2<DT>(lo[0], lo[1]), pack_relu2<DT>(lo[2], lo[3]), pack_relu2<DT>(hi[0], hi[1]),
-                           pack_relu2<DT>(hi[2], hi[3])};
-        }
+        };
+        if (bias != nullptr) convert(IC<1>{});
+        else convert(IC<0>{});
     };
 
     // ---- first layer: K0 -> 256.  The inputs are older than every weight DMA, so they have landed
@@ -560,52 +647,33 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
         const bool live = row_ok && 32 * s + 8 * q < K0;
         act[s] = live ? act[s] : u32x4{0u, 0u, 0u, 0u};
     }
-    asm volatile("" : "+v"(u_row));
-    full_chunk(IC<0>{});
+    asm volatile("" : "+v"(u_row), "+v"(tab_w), "+v"(tab_b));
+    first_sync();
+    run_chunk(IC<0>{}, IC<1>{});
     if constexpr (C0 > 1) {
-        full_chunk(IC<1>{});
-        full_chunk(IC<2>{});
-        full_chunk(IC<3>{});
+        run_chunk(IC<1>{}, IC<0>{});
+        run_chunk(IC<2>{}, IC<0>{});
+        run_chunk(IC<3>{}, IC<0>{});
     }
-    next_activations(a.b[0]);
+    next_activations(b0_ptr);
 
     // ---- hidden layers: 256 -> 256 ----
     for (int layer = 1; layer + 1 < NL; ++layer) {
-        full_chunk(IC<0>{});
-        full_chunk(IC<1>{});
-        full_chunk(IC<2>{});
-        full_chunk(IC<3>{});
-        next_activations(a.b[layer]);
+        run_chunk(IC<0>{}, IC<0>{});
+        run_chunk(IC<1>{}, IC<0>{});
+        run_chunk(IC<2>{}, IC<0>{});
+        run_chunk(IC<3>{}, IC<0>{});
+        next_activations((const float*)table_ptr(tab_b, layer));
     }
 
     // ---- last layer: 256 -> NOUT <= 64, one chunk, 4 tiles ----
-    {
-        const unsigned char* st = chunk_sync();
-#pragma unroll
-        for (int m = 0; m < PW; ++m) issue(m);
-        // two slabs (16 reads) are requested at a time: with so few MFMAs per read the LDS round
-        // trips, not the arithmetic, set the pace
-#pragma unroll
-        for (int c2 = 0; c2 < H / 128; ++c2) {
-            u32x4 w[2][2][MLP_MAX_OUT / 16];
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                for (int sp = 0; sp < 2; ++sp)
-#pragma unroll
-                    for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
-                        w[cc][sp][t] = *reinterpret_cast<const u32x4*>(st + (2 * c2 + cc) * 64 * 128 + frag_off[sp] + tile_off(t));
-#pragma unroll
-            for (int cc = 0; cc < 2; ++cc)
-#pragma unroll
-                for (int sp = 0; sp < 2; ++sp)
-#pragma unroll
-                    for (int t = 0; t < MLP_MAX_OUT / 16; ++t)
-                        acc[t] = mfma((c2 == 0 && cc == 0 && sp == 0) ? zero4 : acc[t], w[cc][sp][t], act[2 * (2 * c2 + cc) + sp]);
-        }
-    }
-    const float* bias = a.b[NL - 1];
-    const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
+    run_chunk(IC<4>{}, IC<0>{});
+    // the dummy DMAs (they land in their own KiB) must be done before the LDS is released; they are
+    // long done, and waiting here rather than at the end keeps the outputs' stores out of the wait
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // (a pointer that came out of a register table must be told that it points to global memory)
+    const __attribute__((address_space(1))) float* bias = (const __attribute__((address_space(1))) float*)(unsigned long long)table_ptr(tab_b, NL - 1);
+    const int limit = mask_size > 0 ? mask_size : NOUT;
     if (NOUT <= 8) {
         // narrow heads never leave the registers: in tiles 0 and 1 lane (j, q = 0) holds columns 0..3 and
         // 4..7 of batch row j, and those lanes are lanes 0..15 of the wave
@@ -615,7 +683,10 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
             p[n] = acc[n >> 2][n & 3];
             if (bias != nullptr && n < NOUT) p[n] += bias[n];
         }
-        if (lane < 16 && row_ok) head_row<8>(a, p, row, NOUT, limit, u_row);
+        if (lane < 16 && row_ok) {
+            if (NOUT <= 4) head_row<4>(out, p, row, NOUT, limit, u_row);
+            else head_row<8>(out, p, row, NOUT, limit, u_row);
+        }
     } else {
         __syncthreads();                                    // every wave has read its last weights: reuse stage 0
         float* head_rows = reinterpret_cast<float*>(lds) + wave * 16 * MLP_MAX_OUT;
@@ -630,9 +701,8 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
             *reinterpret_cast<f32x4*>(head_rows + j * MLP_MAX_OUT + tile_col(t)) = v;
         }
         // lanes 0..15 of every wave own one batch row each (the staging is wave private)
-        if (lane < 16 && row_ok) head_row<MLP_MAX_OUT>(a, head_rows + lane * MLP_MAX_OUT, row, NOUT, limit, u_row);
+        if (lane < 16 && row_ok) head_row<MLP_MAX_OUT>(out, head_rows + lane * MLP_MAX_OUT, row, NOUT, limit, u_row);
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the dummy DMAs (they land in their own KiB) before the LDS is released
 }
 
 namespace {
@@ -688,7 +758,7 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     int rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
     a.x = x; a.n_layers = n_layers; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
-    a.batch = batch; a.head = head; a.mask_size = mask_size;
+    a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.nout = dims[n_layers];
     // 4 waves (64 rows) per workgroup while such workgroups fit the compute units in one round: every
     // wave reads all weights from LDS, so 8 waves on a unit are LDS-bandwidth bound (2048 cycles per
     // 32 KiB chunk) where 4 are not; beyond one round, 8 waves (128 rows) halve the rounds
