@@ -435,13 +435,16 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
 
     // ---- the wave's input rows, requested before any weight so that they are the oldest loads;
     //      the row's uniform for the sampling head travels with them ----
+    constexpr int XS = C0 == 1 ? 2 : H / 32;         // 32-wide k-steps of the input (K0 <= 64 when C0 is 1)
     const bool row_ok = row < batch;
     u32x4 act[H / 32];
     float u_row = 1.f;
     {
         const unsigned char* xr = x_ptr + (row_ok ? row : 0) * K0 * 2;
+        // (in operand order a lane touches a cache line of its own, which the texture path serves at a
+        //  quarter of its rate: no loads for k-steps the first layer cannot have)
 #pragma unroll
-        for (int s = 0; s < H / 32; ++s) {
+        for (int s = 0; s < XS; ++s) {
             const int k = 32 * s + 8 * q;
             asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(act[s]) : "v"(xr + (k < K0 ? k : 0) * 2) : "memory");
         }
@@ -643,9 +646,13 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PW) : "memory");
 #pragma unroll
     for (int s = 0; s < H / 32; ++s) {
-        asm volatile("" : "+v"(act[s]));
-        const bool live = row_ok && 32 * s + 8 * q < K0;
-        act[s] = live ? act[s] : u32x4{0u, 0u, 0u, 0u};
+        if (s < XS) {
+            asm volatile("" : "+v"(act[s]));
+            const bool live = row_ok && 32 * s + 8 * q < K0;
+            act[s] = live ? act[s] : u32x4{0u, 0u, 0u, 0u};
+        } else {
+            act[s] = u32x4{0u, 0u, 0u, 0u};
+        }
     }
     asm volatile("" : "+v"(u_row), "+v"(tab_w), "+v"(tab_b));
     first_sync();
