@@ -712,6 +712,341 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     }
 }
 
+// ---- stacks of three or more layers, all hidden layers 256 wide, at most 16 outputs, one 64-row
+//      workgroup per compute unit ----
+// With 16 batch rows per wave every wave reads ALL weights from LDS: 32 KiB per 64-column chunk, and a
+// SIMD's registers take operands from LDS at little more than 47 bytes per cycle -- 700 cycles for a
+// chunk whose MFMAs need 512.  This kernel splits a hidden layer by OUTPUT FEATURES instead: wave w
+// computes features 64 w .. 64 w + 63 for all 64 batch rows of the workgroup.  It streams only its own
+// quarter of the weights (8 KiB per chunk: 64 rows x 64 K-columns) through a ring of four LDS stages
+// that no other wave touches -- weights need no barrier, only the wave's own vmcnt -- and reads the
+// activations of all 64 rows from a shared 32 KiB buffer ([row][feature], the 16-byte pieces of a row
+// XOR-swizzled with the row number, so that the 16 rows of an operand fetch fall into different banks).
+// Per layer a SIMD takes 64 KiB from LDS instead of 128.  A layer ends with: barrier, the outputs (bias,
+// relu, rounded to 16 bits) written over the activations, barrier.
+// Tile (p, h) of a wave's 64 features feeds MFMA row i with feature 32 p + 8 (i / 4) + 4 h + i % 4: the
+// two quads a lane holds in tiles (p, 0) and (p, 1) are then 8 consecutive features, one 16-byte write.
+// The last layer (at most 16 outputs, one MFMA tile) is split by batch rows: wave w multiplies rows
+// 16 w .. 16 w + 15 with all outputs (every wave streams the whole last matrix, one chunk of four
+// 64-column slabs), and lanes 0..15 run the head.
+// Every global load is issued from assembly and counted by hand: the counter of outstanding loads is in
+// order and the schedule is static, so each wait names the exact number of younger loads.  Chunk c + 3
+// is requested behind the first k-step of chunk c; chunk c + 1 is awaited before the second.
+constexpr int SPLIT_ROWS = 64;
+constexpr int SPLIT_ACT_BYTES = SPLIT_ROWS * 2 * MLP_MAX_DIM;      // 32 KiB
+constexpr int SPLIT_STAGE_BYTES = 64 * 128;                        // 64 weight rows x 64 K-columns
+constexpr int SPLIT_STAGES = 4;
+constexpr int SPLIT_RING_BYTES = SPLIT_STAGES * SPLIT_STAGE_BYTES;
+constexpr int SPLIT_LDS_BYTES = SPLIT_ACT_BYTES + 4 * SPLIT_RING_BYTES;
+
+template <int DT, int KS0>
+__global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
+    constexpr int C0 = (KS0 + 1) / 2;                // chunks of the first layer
+    constexpr bool HALF0 = KS0 == 1;                 // ... which is half a chunk when K0 <= 32
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = lane & 15, q = lane >> 4;
+    const long row0 = (long)blockIdx.x * SPLIT_ROWS;
+    const u32x4 zero_u4 = {0u, 0u, 0u, 0u};
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+    // every scalar argument in one round trip; the per-layer pointers in a register table (lane l holds
+    // weights[l] and biases[l], picked by v_readlane)
+    const int K0 = a.k0, NL = a.n_layers, NOUT = a.nout;
+    const unsigned char* const x_ptr = (const unsigned char*)a.x;
+    const unsigned char* const w0_ptr = (const unsigned char*)a.w[0];
+    const unsigned char* const w1_ptr = (const unsigned char*)a.w[1];
+    const unsigned char* const b0_ptr = (const unsigned char*)a.b[0];
+    const float* const u_ptr = a.u;
+    const long batch = a.batch;
+    const HeadOut out = head_out(a);
+    const int mask_size = a.mask_size;
+    asm volatile("" ::"s"(K0), "s"(NL), "s"(NOUT), "s"(x_ptr), "s"(w0_ptr), "s"(w1_ptr), "s"(b0_ptr), "s"(u_ptr), "s"(batch),
+                 "s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(mask_size));
+    u32x2 tab_w, tab_b;
+    {
+        const unsigned char* args = (const unsigned char*)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_w) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, w)) : "memory");
+        asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_b) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, b)) : "memory");
+    }
+    auto table_ptr = [&](const u32x2& tab, int l) {
+        const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)tab[0], l);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readlane((int)tab[1], l);
+        return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
+    };
+
+    // ---- the workgroup's input rows (16-byte pieces, 4 KS0 per row) and the uniform of the row this
+    //      lane will finish ----
+    u32x4 xin[KS0];
+    bool x_ok[KS0];
+#pragma unroll
+    for (int i = 0; i < KS0; ++i) {
+        const int idx = tid + 256 * i;
+        const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
+        x_ok[i] = row0 + r < batch && pc * 8 < K0;
+        const long off = x_ok[i] ? ((row0 + r) * K0 + pc * 8) * 2 : 0;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(xin[i]) : "v"(x_ptr + off) : "memory");
+    }
+    const long head_row_idx = row0 + wave * 16 + j;          // the row lanes 0..15 finish
+    const bool head_ok = lane < 16 && head_row_idx < batch;
+    float u_row = 1.f;
+    {
+        const unsigned char* up = u_ptr != nullptr ? (const unsigned char*)(u_ptr + (head_ok ? head_row_idx : 0)) : x_ptr;
+        asm volatile("global_load_dword %0, %1, off" : "=v"(u_row) : "v"(up) : "memory");
+    }
+    // ---- a layer's 64 bias values of this wave, always four loads: a missing bias reads the layer's
+    //      weights instead (and is not added), so that the number of loads never depends on the arguments ----
+    f32x4 bias_r[4];                                         // [2 p + h]: features 64 wave + 32 p + 8 q + 4 h ..+ 3
+    bool has_bias = false;
+    auto load_bias = [&](const unsigned char* bias, const unsigned char* valid) {
+        has_bias = bias != nullptr;
+        const unsigned char* src = (has_bias ? bias : valid) + (64 * wave + 8 * q) * 4;
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(bias_r[0]) : "v"(src) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:16" : "=v"(bias_r[1]) : "v"(src) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:128" : "=v"(bias_r[2]) : "v"(src) : "memory");
+        asm volatile("global_load_dwordx4 %0, %1, off offset:144" : "=v"(bias_r[3]) : "v"(src) : "memory");
+    };
+    load_bias(b0_ptr, w0_ptr);
+
+    // ---- the weight stream of this wave: chunk after chunk, 8 DMA instructions each ----
+    // Instruction m fills stage rows 8 m .. 8 m + 7: lane l fetches, for row R = 8 m + l / 8, the 16-byte
+    // piece (l % 8) ^ swz(R), swz(R) = 2 ((R >> 3) & 3) + ((R >> 1) & 1) = 2 (m & 3) + ((l >> 4) & 1).
+    const unsigned ring_base = (unsigned)(size_t)lds + SPLIT_ACT_BYTES + wave * SPLIT_RING_BYTES;
+    const int dr = lane >> 3, dc = lane & 7, db = (lane >> 4) & 1;
+    int f_layer = 0, f_kc = 0, f_stage = 0;
+    auto issue_chunk = [&](auto EARLY_) {
+        constexpr bool early = decltype(EARLY_)::value != 0;   // before the table has landed: layers 0 and 1 only
+        const unsigned dst0 = ring_base + f_stage * SPLIT_STAGE_BYTES;
+        if (f_layer == 0) {
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                int k = f_kc * 64 + (dc ^ (2 * (m & 3) + db)) * 8;
+                k = k <= K0 - 8 ? k : K0 - 8;                  // pieces past K0 meet zero activations
+                mlp_dma(w0_ptr, (unsigned)(((64 * wave + 8 * m + dr) * K0 + k) * 2), dst0 + m * 1024);
+            }
+        } else if (f_layer < NL - 1) {
+            const unsigned char* base = (early ? w1_ptr : table_ptr(tab_w, f_layer)) + f_kc * 128;
+#pragma unroll
+            for (int m = 0; m < 8; ++m)
+                mlp_dma(base, (unsigned)(((64 * wave + 8 * m + dr) * 256 + (dc ^ (2 * (m & 3) + db)) * 8) * 2), dst0 + m * 1024);
+        } else {
+            const unsigned char* base = table_ptr(tab_w, NL - 1);
+#pragma unroll
+            for (int m = 0; m < 8; ++m) {
+                // one chunk: slab s = R / 16 holds K-columns 64 s .. of outputs R % 16 (outputs past NOUT repeat
+                // the last one and only reach accumulator rows nobody reads)
+                const int R = 8 * m + dr;
+                int o = R & 15;
+                o = o < NOUT ? o : NOUT - 1;
+                const int kcol = (R >> 4) * 64 + (dc ^ (2 * (m & 3) + db)) * 8;
+                mlp_dma(base, (unsigned)((o * 256 + kcol) * 2), dst0 + m * 1024);
+            }
+        }
+        const int count = f_layer == 0 ? C0 : (f_layer < NL - 1 ? 4 : 1);
+        ++f_kc;
+        if (f_kc == count) { f_kc = 0; ++f_layer; }
+        f_stage = (f_stage + 1) & (SPLIT_STAGES - 1);
+    };
+    issue_chunk(IC<1>{});
+    issue_chunk(IC<1>{});
+    issue_chunk(IC<1>{});
+
+    // ---- operand addresses ----
+    // weights: tile (p, h), MFMA row j -> stage row R = 32 p + 4 h + R0, R0 = 8 (j / 4) + j % 4; swz(R) does not
+    // depend on p and h
+    const int R0 = 8 * (j >> 2) + (j & 3);
+    const int swzR = 2 * ((j >> 2) & 3) + ((j >> 1) & 1);
+    unsigned fragW[2];
+#pragma unroll
+    for (int sp = 0; sp < 2; ++sp) fragW[sp] = (unsigned)(SPLIT_ACT_BYTES + wave * SPLIT_RING_BYTES + R0 * 128 + (((4 * sp + q) ^ swzR) << 4));
+    auto read_w = [&](int stage, int sp, int t) {
+        return *reinterpret_cast<const u32x4*>(lds + fragW[sp] + stage * SPLIT_STAGE_BYTES + (32 * (t >> 1) + 4 * (t & 1)) * 128);
+    };
+    // activations: row r, piece P (of 32) lives in slot (P & 16) | ((P ^ r) & 15)
+    unsigned aoff[4];
+#pragma unroll
+    for (int k4 = 0; k4 < 4; ++k4) aoff[k4] = (unsigned)(j * 512 + (((4 * k4 + q) ^ j) << 4));
+    auto read_a = [&](int bt_bytes, int ks) {               // bt_bytes = 8192 * batch tile
+        return *reinterpret_cast<const u32x4*>(lds + aoff[ks & 3] + bt_bytes + (ks >> 2) * 256);
+    };
+    unsigned pw[2];
+#pragma unroll
+    for (int p = 0; p < 2; ++p) pw[p] = (unsigned)(j * 512 + (wave >> 1) * 256 + (((8 * (wave & 1) + 4 * p + q) ^ j) << 4));
+
+    // ---- everything older than the second chunk has landed: inputs into the activation buffer ----
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < KS0; ++i) asm volatile("" : "+v"(xin[i]));
+    asm volatile("" : "+v"(u_row), "+v"(tab_w), "+v"(tab_b), "+v"(bias_r[0]), "+v"(bias_r[1]), "+v"(bias_r[2]), "+v"(bias_r[3]));
+#pragma unroll
+    for (int i = 0; i < KS0; ++i) {
+        const int idx = tid + 256 * i;
+        const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
+        *reinterpret_cast<u32x4*>(lds + r * 512 + (pc & 16) * 16 + (((pc ^ r) & 15) << 4)) = x_ok[i] ? xin[i] : zero_u4;
+    }
+    __syncthreads();
+
+    auto mfma = [&](const f32x4& c, const u32x4& w, const u32x4& x) {
+        if constexpr (DT == SP_F16)
+            return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, x), c, 0, 0, 0);
+        else
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), c, 0, 0, 0);
+    };
+    f32x4 acc[4][4];                                         // [batch tile][feature tile]
+    u32x4 wf[2][4], bf[2][4];                                // operands of k-step parity 0 / 1
+    int r_stage = 0;                                         // ring stage of the chunk being multiplied
+#pragma unroll
+    for (int t = 0; t < 4; ++t) wf[0][t] = read_w(0, 0, t);
+
+    // One chunk of a feature-split layer.  KC: its place in the layer (activation k-steps 2 KC, 2 KC + 1);
+    // FIRSTK / LASTK: first / last chunk of the layer; HALF: only the first k-step exists; ISSUE: request chunk
+    // c + 3 behind the first k-step; BIAS: then request this layer's bias; WAITN: loads younger than chunk c + 1
+    // at that point; NEXTW: chunk c + 1 is of the same kind, fetch its first operands.
+    auto chunk = [&](auto KC_, auto FIRSTK_, auto LASTK_, auto HALF_, auto ISSUE_, auto BIAS_, auto WAITN_, auto NEXTW_,
+                     const unsigned char* bias, const unsigned char* valid) {
+        constexpr int KC = decltype(KC_)::value;
+        constexpr bool firstk = decltype(FIRSTK_)::value != 0, lastk = decltype(LASTK_)::value != 0;
+        constexpr bool half = decltype(HALF_)::value != 0, issue = decltype(ISSUE_)::value != 0;
+        constexpr bool want_bias = decltype(BIAS_)::value != 0, nextw = decltype(NEXTW_)::value != 0;
+        constexpr int WAITN = decltype(WAITN_)::value;
+        if constexpr (firstk) {
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_a(bt * 8192, 2 * KC);
+        }
+        if constexpr (!half) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) wf[1][t] = read_w(r_stage, 1, t);
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) bf[1][bt] = read_a(bt * 8192, 2 * KC + 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) acc[bt][t] = mfma(KC == 0 ? zero4 : acc[bt][t], wf[0][t], bf[0][bt]);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (issue) issue_chunk(IC<0>{});
+        if constexpr (want_bias) load_bias(bias, valid);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WAITN) : "memory");
+        const int next_stage = (r_stage + 1) & (SPLIT_STAGES - 1);
+        if constexpr (nextw) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) wf[0][t] = read_w(next_stage, 0, t);
+        }
+        if constexpr (!lastk) {
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_a(bt * 8192, 2 * KC + 2);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (!half) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int bt = 0; bt < 4; ++bt) acc[bt][t] = mfma(acc[bt][t], wf[1][t], bf[1][bt]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        r_stage = next_stage;
+    };
+    // the layer's outputs replace its inputs: barrier (every wave is done reading), bias, relu, rounding,
+    // 16 bytes per (batch tile, tile pair), barrier
+    auto publish = [&]() {
+        asm volatile("s_barrier" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(bias_r[i]));
+        auto convert = [&](auto HAS_BIAS_) {
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt)
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    f32x4 lo = acc[bt][2 * p], hi = acc[bt][2 * p + 1];
+                    if constexpr (decltype(HAS_BIAS_)::value != 0) {
+                        lo += bias_r[2 * p];
+                        hi += bias_r[2 * p + 1];
+                    }
+                    const u32x4 v = {pack_relu2<DT>(lo[0], lo[1]), pack_relu2<DT>(lo[2], lo[3]), pack_relu2<DT>(hi[0], hi[1]),
+                                     pack_relu2<DT>(hi[2], hi[3])};
+                    *reinterpret_cast<u32x4*>(lds + pw[p] + bt * 8192) = v;
+                }
+        };
+        if (has_bias) convert(IC<1>{});                      // uniform, once per layer
+        else convert(IC<0>{});
+        __syncthreads();
+    };
+
+    // ---- first layer: K0 -> 256 (its bias was requested with the inputs) ----
+    if constexpr (C0 == 1) {
+        chunk(IC<0>{}, IC<1>{}, IC<1>{}, IC<HALF0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+    } else {
+        chunk(IC<0>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<2>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<3>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+    }
+    publish();
+    // ---- hidden layers but the last one ----
+    for (int layer = 1; layer + 2 < NL; ++layer) {
+        const unsigned char* bias = table_ptr(tab_b, layer);
+        const unsigned char* valid = table_ptr(tab_w, layer);
+        chunk(IC<0>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, IC<20>{}, IC<1>{}, bias, valid);
+        chunk(IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<20>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<2>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<20>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<3>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<16>{}, IC<1>{}, nullptr, nullptr);
+        publish();
+    }
+    // ---- the last hidden layer: the stream ends with the output layer's chunk ----
+    {
+        const unsigned char* bias = table_ptr(tab_b, NL - 2);
+        const unsigned char* valid = table_ptr(tab_w, NL - 2);
+        chunk(IC<0>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, IC<20>{}, IC<1>{}, bias, valid);
+        chunk(IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<20>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<2>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<12>{}, IC<1>{}, nullptr, nullptr);
+        chunk(IC<3>{}, IC<0>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nullptr, nullptr);
+        publish();
+    }
+    // ---- output layer: rows 16 wave .. + 15 of the workgroup; MFMA row i is output i, stage row 16 s + i
+    //      in slab s ----
+    f32x4 d;
+    {
+        u32x4 al[8], wl[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+            al[ks] = read_a(wave * 8192, ks);
+            const int R = 16 * (ks >> 1) + j;
+            const int sw = 2 * ((R >> 3) & 3) + ((R >> 1) & 1);
+            wl[ks] = *reinterpret_cast<const u32x4*>(lds + SPLIT_ACT_BYTES + wave * SPLIT_RING_BYTES + r_stage * SPLIT_STAGE_BYTES + R * 128 +
+                                                     (((4 * (ks & 1) + q) ^ sw) << 4));
+        }
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) d = mfma(ks == 0 ? zero4 : d, wl[ks], al[ks]);
+    }
+    // (a pointer that came out of a register table must be told that it points to global memory)
+    const __attribute__((address_space(1))) float* bias =
+        (const __attribute__((address_space(1))) float*)(unsigned long long)table_ptr(tab_b, NL - 1);
+    const int limit = mask_size > 0 ? mask_size : NOUT;
+    if (NOUT <= 4) {
+        // lane (j, q = 0) holds outputs 0..3 of batch row j; those are lanes 0..15 of the wave
+        float p[4];
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+            p[n] = d[n];
+            if (bias != nullptr && n < NOUT) p[n] += bias[n];
+        }
+        if (head_ok) head_row<4>(out, p, head_row_idx, NOUT, limit, u_row);
+    } else {
+        // every chunk of this wave's ring has been consumed: its first stage stages the 16 x NOUT outputs
+        float* head_rows = reinterpret_cast<float*>(lds + SPLIT_ACT_BYTES + wave * SPLIT_RING_BYTES);
+        f32x4 v = d;
+        if (bias != nullptr) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (4 * q + r < NOUT) v[r] += bias[4 * q + r];
+        }
+        *reinterpret_cast<f32x4*>(head_rows + j * 16 + 4 * q) = v;
+        if (head_ok) head_row<16>(out, head_rows + lane * 16, head_row_idx, NOUT, limit, u_row);
+    }
+}
+
 namespace {
 struct MlpKernelNames {
     MlpKernelNames() {
@@ -724,6 +1059,17 @@ struct MlpKernelNames {
 }  // namespace sp
 
 using namespace sp;
+
+static const void* pick_split_kernel(int dtype, int ks0) {
+    if (dtype == SP_F16) {
+        if (ks0 == 1) return (const void*)mlp_split_kernel<SP_F16, 1>;
+        if (ks0 == 2) return (const void*)mlp_split_kernel<SP_F16, 2>;
+        return (const void*)mlp_split_kernel<SP_F16, 8>;
+    }
+    if (ks0 == 1) return (const void*)mlp_split_kernel<SP_BF16, 1>;
+    if (ks0 == 2) return (const void*)mlp_split_kernel<SP_BF16, 2>;
+    return (const void*)mlp_split_kernel<SP_BF16, 8>;
+}
 
 extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights,
                               const float* const* biases, const int32_t* dims, const float* u, float* policy_out,
@@ -775,7 +1121,18 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     bool h256 = n_layers >= 2;   // all hidden layers 256 wide: the lean kernel
     for (int i = 1; i < n_layers; ++i) h256 = h256 && dims[i] == 256;
     const void* kernel;
-    if (h256) {
+    int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
+    int rows_per_block = nw * 16;
+    int threads = nw * 64;
+    // at most one 64-row workgroup per compute unit and a narrow head: hidden layers split by output features
+    const bool split = h256 && n_layers >= 3 && !wide && dims[n_layers] <= 16;
+    if (split) {
+        const int ks0 = dims[0] <= 32 ? 1 : dims[0] <= 64 ? 2 : 8;
+        kernel = pick_split_kernel(dtype, ks0);
+        lds_bytes = SPLIT_LDS_BYTES;
+        rows_per_block = SPLIT_ROWS;
+        threads = 256;
+    } else if (h256) {
         const bool small_k = dims[0] <= 64;
         if (dtype == SP_F16)
             kernel = wide ? (small_k ? (const void*)mlp_h256_kernel<SP_F16, 8, 1> : (const void*)mlp_h256_kernel<SP_F16, 8, 4>)
@@ -788,7 +1145,6 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     } else {
         kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
     }
-    const int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
     // the LDS opt-in is per kernel and device; remember which (kernel, device) pairs have it (a lost
     // race only repeats an idempotent call)
     static const void* opted_kernel[64];
@@ -809,9 +1165,9 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
             n_opted = n_seen + 1;
         }
     }
-    const long blocks = (batch + nw * 16 - 1) / (nw * 16);
+    const long blocks = (batch + rows_per_block - 1) / rows_per_block;
     void* args[] = {(void*)&a};
-    e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(nw * 64), args, lds_bytes, (hipStream_t)stream);
+    e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward: launch failed: %s", hipGetErrorString(e));
     return check_launch(__func__);
 }

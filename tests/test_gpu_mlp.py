@@ -97,9 +97,13 @@ def test_other_stacks(LY, dims, head, mask):
     ([256, 256, 8], "regret_matching", 5, 130, "f16", False),             # no hidden 256 -> 256 layer at all
     ([64, 256, 256, 3], "softmax_regret_matching", 0, 20000, "f16", False),  # more rows than 4-wave workgroups cover: 8 waves
     ([16, 256, 256, 256, 256, 256, 256, 256, 4], "softmax", 0, 64, "f16", True),  # the deepest stack
+    # up to one 64-row workgroup per compute unit and at most 16 outputs: hidden layers split by output features
+    ([128, 256, 256, 256, 10], "softmax", 7, 300, "f16", True),           # four first-layer chunks, head staged in LDS
+    ([48, 256, 256, 16], "regret_matching", 0, 130, "bf16", False),       # K0 in (32, 64], not a multiple of 32; 16 outputs
+    ([32, 256, 256, 256, 256, 5], "softmax_regret_matching", 0, 16384, "bf16", True),   # every compute unit busy
 ])
 def test_stacks_with_256_wide_hidden_layers(LY, dims, head, mask, batch, dtype, with_bias):
-    """The shapes served by the lean kernel (all hidden layers 256 wide)."""
+    """The shapes served by the two kernels for stacks whose hidden layers are all 256 wide."""
     announce("mlp h256 %s head=%s mask=%d batch=%d %s bias=%s" % (dims, head, mask, batch, dtype, with_bias))
     rng = np.random.default_rng(sum(dims) + batch)
     x, ws, u = make_problem(rng, batch, dims, dtype)
