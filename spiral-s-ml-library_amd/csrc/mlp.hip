@@ -106,8 +106,8 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
         for (int n = 0; n < MAXN; ++n)
             if (n < N) o.logits[row * N + n] = p[n];
     }
-    // exp on the hardware exp2 unit and one reciprocal per normalisation: a 16-lane serial head is
-    // otherwise a visible part of a forward pass that takes a few microseconds
+    // exp on the hardware exp2 unit and one hardware reciprocal (1 ulp) per normalisation: a 16-lane
+    // serial head is otherwise a visible part of a forward pass that takes a few microseconds
     if (o.head == SP_HEAD_SOFTMAX || o.head == SP_HEAD_SOFTMAX_RM) {
         float m = -__builtin_inff();
 #pragma unroll
@@ -121,7 +121,7 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
             p[n] = __builtin_amdgcn_exp2f((p[n] - m) * 1.44269504088896340736f);
             s = s + p[n];
         }
-        const float inv = 1.f / s;
+        const float inv = __builtin_amdgcn_rcpf(s);
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) p[n] = p[n] * inv;
     }
@@ -132,8 +132,8 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
             p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
             s = s + p[n];
         }
-        const float inv_len = 1.f / (float)limit;
-        const float inv = s != 0.f ? 1.f / s : 0.f;
+        const float inv_len = __builtin_amdgcn_rcpf((float)limit);
+        const float inv = s != 0.f ? __builtin_amdgcn_rcpf(s) : 0.f;
 #pragma unroll
         for (int n = 0; n < MAXN; ++n) p[n] = s != 0.f ? p[n] * inv : (n < limit ? inv_len : 0.f);
     }
