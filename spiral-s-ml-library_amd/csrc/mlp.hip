@@ -19,6 +19,10 @@
 //
 // The head (softmax / regret matching / sampling) runs on the last layer's f32 outputs.
 //
+// Stacks of 256-wide hidden layers with a narrow head and at most 64 rows per compute unit take another
+// route (mlp_split_kernel, described where it is defined): there a wave owns 64 OUTPUT FEATURES of all
+// 64 rows of the workgroup and the activations are exchanged through LDS.
+//
 // Semantics follow the graph interpreter of ml/layers.spi:194-240 (BlockMatmul = x . w^T with w
 // stored (out, in), relu = max 0) and the heads of ml/primitives.spi:711-722,748-798.
 #include "common.h"
