@@ -13,6 +13,7 @@
 // Semantics follow matmul_tf32_template (ml/matmul/kernel.spi:25-240) with a_trans=false,
 // b_trans=true; the f32 path multiplies in full f32 (v_mfma_f32_32x32x2_f32), not TF32.
 #include "common.h"
+#include <type_traits>
 
 namespace sp {
 
@@ -341,6 +342,251 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     }
 }
 
+// ---- 256 x 256 x 64 tiles on FOUR waves (one per SIMD), 16x16x32 MFMAs: the kernel for large 16-bit GEMMs ----
+// Same data movement as gemm_abt_kernel (DMA into two swizzled LDS stages, one barrier per K-tile), but a wave owns a
+// 128 x 128 quarter of the tile: 64 accumulator tiles of 16 x 16 = 256 registers in the accumulation file (the wave
+// has all 512 registers of its SIMD).  Operands of a 32-wide k-step are 8 + 8 fragments of "16 rows x one 16-byte
+// chunk per lane": 32 KiB of LDS reads per wave and K-tile against 24 KiB for each of eight waves, a third less
+// per compute unit, and v_mfma_f32_16x16x32 draws less power per flop than the 32x32x16 form, which is what the
+// clock of a power-limited GEMM is made of.
+// What makes a lone wave per SIMD work: every instruction it issues costs the matrix pipe ~4-5 cycles (there is no
+// second wave to issue in the shadow of its MFMAs), and two memory instructions back to back cost more than that.
+// So the loop body is straight-line code for two K-tiles (stage addresses are immediates), carries no address
+// arithmetic (one scalar base per matrix, per-lane offsets in registers, fragment addresses in registers), and puts
+// every LDS read and every DMA alone between two MFMAs: 128 MFMAs + ~76 other instructions per K-tile.
+// The fragment of the B matrix is the MFMA's first operand: register r of lane l of accumulator tile
+// (tm, tn) holds C[m = 16 tm + l % 16][n = 16 tn + 4 (l / 16) + r].
+template <int DT, int OT>
+__global__ __launch_bounds__(256) void gemm_abt_w4_kernel(const GemmArgs g) {
+    static_assert(DT != SP_F32, "16-bit inputs only");
+    constexpr int BM = 256, BN = 256, NW = 4, ES = 2;
+    constexpr int BK = ROW_BYTES / ES;
+    constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
+    constexpr int NI = (BM + BN) / 8 / NW;      // 16 DMA instructions per wave and K-tile
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
+    int tm_, tn_;
+    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm_, tn_);
+    const long m0 = (long)tm_ * BM, n0 = (long)tn_ * BN;
+    const long K = g.K;
+    const unsigned char* const Ab = (const unsigned char*)g.A + (long)blockIdx.y * g.stride_a;
+    const unsigned char* const Bb = (const unsigned char*)g.B + (long)blockIdx.y * g.stride_b;
+    unsigned char* const Cb = (unsigned char*)g.C + (long)blockIdx.y * g.stride_c;
+
+    // loader: DMA instruction q of wave w fills the 8 rows of row block (q % 8) * NW + w of the A (q < 8) or B tile.
+    // One scalar base per matrix (row block `wave` of the tile, advanced by one K-tile at a time) and one per-lane
+    // offset per q % 8, shared by A and B (same row pitch): a lone wave per SIMD pays ~4 cycles of matrix-pipe time
+    // for EVERY instruction it issues, so the loop carries no per-instruction address arithmetic.
+    const unsigned lds_base = (unsigned)(size_t)lds;
+    const unsigned char* sA = uniform_ptr(Ab + (m0 + wave * 8) * K * ES);
+    const unsigned char* sB = uniform_ptr(Bb + (n0 + wave * 8) * K * ES);
+    unsigned dstw = __builtin_amdgcn_readfirstlane(lds_base + wave * 8 * ROW_BYTES);
+    unsigned voff[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+        const int r = lane >> 3;
+        // chunk fetched by a lane: (lane & 7) ^ swz(row), row = 8 blk + r, blk & 7 = (4 q + wave) & 7
+        const unsigned chunk = (unsigned)((((lane & 7) ^ r ^ ((4 * q + wave) & 7)) & 7) << 4);
+        voff[q] = (unsigned)((q * 8 * NW + r) * K * ES) + chunk;
+    }
+    auto dma_plain = [&](int q, int stage) {
+        const unsigned d = dstw + (q < 8 ? 0 : BM * ROW_BYTES) + (q & 7) * NW * 8 * ROW_BYTES + stage * STAGE_BYTES;
+        dma_to_lds(q < 8 ? sA : sB, voff[q & 7], d);
+    };
+
+    f32x4 acc[8][8];
+    const int fi = lane & 15, fq = lane >> 4;
+    // fragment addresses: row = R0 + 16 t + fi, chunk 4 ks + fq; its slot is (4 ks + fq) ^ fi ^ (fi >> 3) ^ 2 (t & 3)
+    // (R0 is a multiple of 128): per stage 2 k-steps x 4 values of t & 3 = 8 registers per operand, the rest immediates
+    int va[2][2][4], vb[2][2][4];
+#pragma unroll
+    for (int st = 0; st < 2; ++st)
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                va[st][ks][t] = st * STAGE_BYTES + lds_offset(wm * 128 + 16 * t + fi, 4 * ks + fq);
+                vb[st][ks][t] = st * STAGE_BYTES + BM * ROW_BYTES + lds_offset(wn * 128 + 16 * t + fi, 4 * ks + fq);
+                // opaque to the compiler, or it keeps one of them and re-derives the others inside the loop
+                asm volatile("" : "+v"(va[st][ks][t]), "+v"(vb[st][ks][t]));
+            }
+    auto load_a = [&](int st, int ks, int t, u32x4(&fa)[8]) {
+        fa[t] = *reinterpret_cast<const u32x4*>(lds + va[st][ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
+    };
+    auto load_b = [&](int st, int ks, int t, u32x4(&fb)[8]) {
+        fb[t] = *reinterpret_cast<const u32x4*>(lds + vb[st][ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
+    };
+    // operand read h (0 or 1) of row i: rows 0..3 fetch the B-matrix fragments (the next step's first row needs all
+    // of them), rows 4..7 the A-matrix fragments
+    auto load_one = [&](int st, int ks, int i, int h, u32x4(&fa)[8], u32x4(&fb)[8]) {
+        if (i < 4) load_b(st, ks, 2 * i + h, fb);
+        else load_a(st, ks, 2 * (i - 4) + h, fa);
+    };
+    // The MFMAs are issued from assembly with the accumulator pinned to the accumulation registers: left to
+    // itself the register allocator moves parts of the 256-register accumulator between the two register
+    // files around the loop.  (Tiles are revisited 64 MFMAs later, so no wait states are needed in between.)
+    auto mfma_acc = [&](f32x4& c, const u32x4& b, const u32x4& a) {
+        if constexpr (DT == SP_BF16)
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+        else
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(b), "v"(a));
+    };
+    // MFMAs 4..7 of a row with two DMA instructions among them, as one block: each write of M0 has an MFMA between
+    // itself and the DMA that reads it (the wait state it needs), and nothing else can be scheduled in between
+    auto mfma4_dma2 = [&](f32x4& c4, f32x4& c5, f32x4& c6, f32x4& c7, const u32x4& b4, const u32x4& b5, const u32x4& b6,
+                          const u32x4& b7, const u32x4& a, unsigned vo0, unsigned vo1, const unsigned char* base, unsigned dw,
+                          auto D0_, auto D1_) {
+        constexpr unsigned D0 = decltype(D0_)::value, D1 = decltype(D1_)::value;
+#define SP_W4_BLOCK(T)                                                                                                   \
+        asm volatile("s_add_u32 m0, %12, %13\n\t"                                                                      \
+                     "v_mfma_f32_16x16x32_" T " %0, %4, %8, %0\n\t"                                                    \
+                     "global_load_lds_dwordx4 %9, %11\n\t"                                                             \
+                     "v_mfma_f32_16x16x32_" T " %1, %5, %8, %1\n\t"                                                    \
+                     "v_mfma_f32_16x16x32_" T " %2, %6, %8, %2\n\t"                                                    \
+                     "s_add_u32 m0, %12, %14\n\t"                                                                      \
+                     "v_mfma_f32_16x16x32_" T " %3, %7, %8, %3\n\t"                                                    \
+                     "global_load_lds_dwordx4 %10, %11"                                                                  \
+                     : "+a"(c4), "+a"(c5), "+a"(c6), "+a"(c7)                                                            \
+                     : "v"(b4), "v"(b5), "v"(b6), "v"(b7), "v"(a), "v"(vo0), "v"(vo1), "s"(base), "s"(dw), "n"(D0), "n"(D1) \
+                     : "memory", "scc")
+        if constexpr (DT == SP_BF16) SP_W4_BLOCK("bf16");
+        else SP_W4_BLOCK("f16");
+#undef SP_W4_BLOCK
+    };
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    const int nk = (int)(K / BK);     // even (the launcher checks K % 128 == 0)
+    u32x4 fa[2][8], fb[2][8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = zero4;
+    // prologue: tiles 0 and 1 into stages 0 and 1
+#pragma unroll
+    for (int q = 0; q < NI; ++q) dma_plain(q, 0);
+    sA += ROW_BYTES;
+    sB += ROW_BYTES;
+#pragma unroll
+    for (int q = 0; q < NI; ++q) dma_plain(q, 1);
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");   // tile 0 has landed
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+        load_a(0, 0, t, fa[0]);
+        load_b(0, 0, t, fb[0]);
+    }
+    // row I of k-step 1 of a tile in stage ST: fetches 2 I and 2 I + 1 of the tile after the next go into stage ST
+    auto row1 = [&](auto ST_, auto I_) {
+        constexpr int ST = decltype(ST_)::value, i = decltype(I_)::value;
+        constexpr int q0 = 2 * i, q1 = 2 * i + 1;     // 0..7: A, 8..15: B
+        constexpr unsigned D0 = (q0 < 8 ? 0 : BM * ROW_BYTES) + (q0 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
+        constexpr unsigned D1 = (q1 < 8 ? 0 : BM * ROW_BYTES) + (q1 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
+        const unsigned char* base = i < 4 ? sA : sB;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            mfma_acc(acc[i][j], fb[1][j], fa[1][i]);
+            if (j == 1) load_one(ST ^ 1, 0, i, 0, fa[0], fb[0]);
+            if (j == 3) load_one(ST ^ 1, 0, i, 1, fa[0], fb[0]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        mfma4_dma2(acc[i][4], acc[i][5], acc[i][6], acc[i][7], fb[1][4], fb[1][5], fb[1][6], fb[1][7], fa[1][i], voff[q0 & 7],
+                   voff[q1 & 7], base, dstw, std::integral_constant<unsigned, D0>{}, std::integral_constant<unsigned, D1>{});
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    // One K-tile in stage ST.  k-step 0 multiplies fragments taken before it and takes those of k-step 1; the
+    // boundary in the middle waits for tile kt + 1 (fetched during the previous tile) and releases stage ST, all
+    // of whose fragments are in registers by then; k-step 1 takes the first fragments of tile kt + 1 and sends
+    // all 16 fetches of tile kt + 2 into stage ST, two per row of 8 MFMAs, so the last one has a whole k-step plus
+    // what the first ones needed to land.  Every memory instruction stands alone between two MFMAs.  Fetches past
+    // the last tile repeat the last tile into a stage nobody reads any more: no branch in the loop.
+    auto tile = [&](int kt, auto ST_) {
+        constexpr int ST = decltype(ST_)::value;
+        __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): one wait for all fragments of this k-step instead of one per row
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                mfma_acc(acc[i][j], fb[0][j], fa[0][i]);
+                if (j == 1) load_one(ST, 1, i, 0, fa[1], fb[1]);
+                if (j == 3) load_one(ST, 1, i, 1, fa[1], fb[1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        {
+            const int adv = kt + 2 < nk ? ROW_BYTES : 0;
+            sA += adv;
+            sB += adv;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        row1(ST_, std::integral_constant<int, 0>{});
+        row1(ST_, std::integral_constant<int, 1>{});
+        row1(ST_, std::integral_constant<int, 2>{});
+        row1(ST_, std::integral_constant<int, 3>{});
+        row1(ST_, std::integral_constant<int, 4>{});
+        row1(ST_, std::integral_constant<int, 5>{});
+        row1(ST_, std::integral_constant<int, 6>{});
+        row1(ST_, std::integral_constant<int, 7>{});
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        tile(kt, std::integral_constant<int, 0>{});
+        tile(kt + 1, std::integral_constant<int, 1>{});
+    }
+    // the fetches past the end must be done before the stages are reused; the last MFMAs must have written
+    // their results before the accumulators are read (18 wait states, which the compiler cannot know about)
+    asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+
+    // ---- epilogue: per 16-row accumulator row, the wave transposes 16 x 128 values through a private LDS
+    //      strip and writes C (and, for beta != 0, reads it) as whole 512-byte (f32) row segments ----
+    constexpr int EPI_STRIDE = 128 * 4 + 16;
+    static_assert(NW * 16 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
+    __syncthreads();
+    unsigned char* strip = lds + wave * (16 * EPI_STRIDE);
+    const int er = lane >> 5, ec = (lane & 31) * 4;          // 32 lanes per row, 2 rows per pass
+    const float alpha = g.alpha, beta = g.beta;
+    const long col = n0 + wn * 128 + ec;
+    f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+    if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            *reinterpret_cast<f32x4*>(strip + fi * EPI_STRIDE + (16 * j + 4 * fq) * 4) = acc[i][j];
+#pragma unroll
+        for (int p = 0; p < 8; ++p) {
+            const int rl = 2 * p + er;
+            f32x4 v = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
+            const long idx = (m0 + wm * 128 + i * 16 + rl) * g.N + col;
+            v = v * alpha;
+            if constexpr (OT == SP_F32) {
+                f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
+                if (beta != 0.f) v += beta * *c;
+                v += bias4;
+                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                *c = v;
+            } else {
+                u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
+                if (beta != 0.f) {
+                    const u32x2 o = *c;
+                    v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
+                    v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
+                }
+                v += bias4;
+                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+                u32x2 o;
+                o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
+                o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
+                *c = o;
+            }
+        }
+    }
+}
+
+
 // Shape-agnostic kernel: one thread per output element, 16-byte loads along K.  Used for shapes
 // the tiled kernels do not divide (the MLP's K = 32 or N = 3 for instance).
 template <int DT>
@@ -441,10 +687,41 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     return check_launch("sp_gemm_abt");
 }
 
+// The four-wave kernel takes the 256 x 256 tiles of 16-bit GEMMs whose K is a whole number of K-tile pairs and whose
+// B matrix spans more than one tile column; with a single column every A panel is read once, straight from HBM, and
+// two waves per SIMD hide that latency better (65536 x 256 x 2048: 85 us against 89-93 us).
+static bool use_four_waves(int dtype_in, long N, long K) {
+    return dtype_in != SP_F32 && K % 128 == 0 && K <= (1l << 22) && N >= 512;
+}
+
+template <int DT, int OT>
+static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
+    if constexpr (DT == SP_F32) {
+        return fail(SP_ERR_DTYPE, "sp_gemm_abt: the four-wave kernel takes 16-bit inputs");
+    } else {
+        auto kernel = gemm_abt_w4_kernel<DT, OT>;
+        const int lds_bytes = 2 * (256 + 256) * ROW_BYTES;
+        static bool attr_set[64] = {false};
+        int dev = 0;
+        (void)hipGetDevice(&dev);
+        if (!attr_set[dev & 63]) {
+            hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+            if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes,
+                                             hipGetErrorString(e));
+            attr_set[dev & 63] = true;
+        }
+        const long tiles = (long)g.tiles_m * g.tiles_n;
+        hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(256), lds_bytes, stream, g);
+        return check_launch("sp_gemm_abt");
+    }
+}
+
 template <int DT, int OT>
 static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
     switch (cfg) {
-        case 0: return launch_tiled<DT, OT, 256, 256, 2, 4>(g, stream);
+        case 0:
+            if (use_four_waves(DT, g.N, g.K)) return launch_four_waves<DT, OT>(g, stream);
+            return launch_tiled<DT, OT, 256, 256, 2, 4>(g, stream);
         case 1: return launch_tiled<DT, OT, 128, 128, 2, 2>(g, stream);
         case 2: return launch_tiled<DT, OT, 64, 64, 2, 2>(g, stream);
     }
@@ -476,6 +753,8 @@ struct GemmKernelNames {
         register_kernel("gemm_f16_256x256", (const void*)gemm_abt_kernel<SP_F16, SP_F32, 256, 256, 2, 4>, 512);
         register_kernel("gemm_bf16_128x128", (const void*)gemm_abt_kernel<SP_BF16, SP_F32, 128, 128, 2, 2>, 256);
         register_kernel("gemm_f32_64x64", (const void*)gemm_abt_kernel<SP_F32, SP_F32, 64, 64, 2, 2>, 256);
+        register_kernel("gemm_bf16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32>, 256);
+        register_kernel("gemm_f16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_F16, SP_F32>, 256);
     }
 } gemm_kernel_names;
 }  // namespace
@@ -495,6 +774,7 @@ extern "C" int sp_gemm_config(int dtype_in, int64_t M, int64_t N, int64_t K, int
     } else {
         *tile_m = kTileCfgs[cfg].bm; *tile_n = kTileCfgs[cfg].bn; *tile_k = dtype_in == SP_F32 ? 32 : 64;
         *threads = kTileCfgs[cfg].wm * kTileCfgs[cfg].wn * 64;
+        if (cfg == 0 && use_four_waves(dtype_in, N, K)) *threads = 256;
     }
     return SP_OK;
 }

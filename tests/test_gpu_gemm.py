@@ -149,6 +149,38 @@ def test_config2_4096(MM, dtype):
     assert ogemm.rel_frobenius(got16, ogemm.round_to(want, dtype)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_four_wave_kernel_is_exact_on_integers(MM, dtype):
+    """Large 16-bit shapes run on the four-wave kernel (256 threads per tile).  Small integers make every option
+    exact, so an indexing slip in its fragments, fetch offsets or epilogue changes the result: a non-square
+    output, K of two, six and eleven K-tile pairs... alpha/beta, bias + ReLU, 16-bit output, a batch."""
+    announce("gemm four-wave kernel, integer problems " + dtype)
+    m, n = 4096, 3584
+    t = TORCH[dtype]
+    a = ((np.arange(m * 768, dtype=np.int64).reshape(m, 768) * 7 + 3) % 11 - 5).astype(np.float32)
+    b = ((np.arange(n * 768, dtype=np.int64).reshape(n, 768) * 5 + 1) % 13 - 6).astype(np.float32)
+    for k in (128, 384, 768):
+        assert MM.matmul_config_tf32(False, True, m, n, k, t) == dict(m_tile=256, n_tile=256, k_tile=64, threads=256)
+        ak, bk = np.ascontiguousarray(a[:, :k]), np.ascontiguousarray(b[:, :k])
+        want = ak.astype(np.float64) @ bk.astype(np.float64).T      # |sum| <= 30 * 768: exact in f32
+        assert (run(MM, ak, bk, dtype) == want).all(), k
+    k = 384
+    ak, bk = np.ascontiguousarray(a[:, :k]), np.ascontiguousarray(b[:, :k])
+    want = ak.astype(np.float64) @ bk.astype(np.float64).T
+    c0 = ((np.arange(m * n, dtype=np.int64).reshape(m, n) * 3) % 17 - 8).astype(np.float32)
+    bias = ((np.arange(n) * 5) % 201 - 100).astype(np.float32)
+    c = dev(c0.copy())
+    MM.matmul_abt(dev(ak, t), dev(bk, t), c, 2.0, -3.0)
+    assert (host(c) == 2.0 * want - 3.0 * c0).all()
+    got = run(MM, ak, bk, dtype, bias=dev(bias), relu=True)
+    assert (got == np.maximum(want + bias, 0.0)).all()
+    got16 = run(MM, ak, bk, dtype, out_dtype=t)
+    assert (got16 == ogemm.round_to(want.astype(np.float32), dtype)).all()
+    # batch of 4 members of 1024 rows (4 x 14 tiles each), B shared
+    many = host(MM.matmul_abt_batched(dev(ak.reshape(4, 1024, k), t), dev(bk, t)))
+    assert (many.reshape(m, n) == want).all()
+
+
 def test_config2_8192_sampled_rows(MM):
     """8192^3 in bf16: the oracle is evaluated on 192 sampled rows of C (a full CPU product is
     ~1.1 TFLOP); linearity is checked on the whole output: (2A).B^T == 2 (A.B^T) exactly."""
