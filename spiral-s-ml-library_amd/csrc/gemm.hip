@@ -54,19 +54,21 @@ __device__ __forceinline__ float half_bits_to_f32(unsigned bits) {
     else return (float)__builtin_bit_cast(_Float16, (unsigned short)bits);
 }
 
-__device__ __forceinline__ unsigned short f32_to_bf16_rne(float x);
-
-template <int T>
-__device__ __forceinline__ unsigned f32_to_half_bits(float x) {
-    if constexpr (T == SP_BF16) return f32_to_bf16_rne(x);
-    else return __builtin_bit_cast(unsigned short, (_Float16)x);
-}
-
 __device__ __forceinline__ unsigned short f32_to_bf16_rne(float x) {
     unsigned u = __float_as_uint(x);
     if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40u);
     u += 0x7fffu + ((u >> 16) & 1u);
     return (unsigned short)(u >> 16);
+}
+
+// Two f32 values rounded to nearest even and packed into one register (v_cvt_pk_{f16,bf16}_f32).
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+template <int T>
+__device__ __forceinline__ unsigned pack_halves(float a, float b) {
+    if constexpr (T == SP_BF16) return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
+    else return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, f16x2));
 }
 
 // Map the linear workgroup id to an output tile.  Workgroups are dealt round-robin to the 8 XCDs
@@ -296,49 +298,66 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     unsigned char* stg = lds + wave * (32 * EPI_STRIDE);
     const int er = lane / LPR, ec = (lane % LPR) * 4;
     const float alpha = g.alpha, beta = g.beta;
+    const long row_step = (long)RPP * g.N;
+    // The options are compile-time inside the loops: a branch per output row would split them into blocks of one
+    // LDS read -> one store each, with every latency exposed.
+    auto write_tile = [&](auto BETA_, auto RELU_) {
+        constexpr bool HAS_BETA = decltype(BETA_)::value, RELU = decltype(RELU_)::value;
+        auto finish = [&](f32x4 v, const f32x4& old, const f32x4& bias) {
+            v = v * alpha;
+            if constexpr (HAS_BETA) v += beta * old;
+            v += bias;
+            if constexpr (RELU) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+            return v;
+        };
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+        for (int i = 0; i < TM; ++i) {
 #pragma unroll
-        for (int js = 0; js < TN / SF; ++js) {
-            const long col = n0 + wn * WTN + js * SW + ec;
-            f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
-            if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
+            for (int js = 0; js < TN / SF; ++js) {
+                const long col = n0 + wn * WTN + js * SW + ec;
+                f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
+                if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
 #pragma unroll
-            for (int jj = 0; jj < SF; ++jj)
+                for (int jj = 0; jj < SF; ++jj)
 #pragma unroll
-                for (int gq = 0; gq < 4; ++gq) {
-                    const f32x16& c16 = acc[i][js * SF + jj];
-                    f32x4 v = {c16[4 * gq], c16[4 * gq + 1], c16[4 * gq + 2], c16[4 * gq + 3]};
-                    *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (jj * 32 + gq * 8 + frag_half * 4) * 4) = v;
-                }
-#pragma unroll
-            for (int p = 0; p < 32 / RPP; ++p) {
-                const int rl = p * RPP + er;
-                f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
-                const long idx = (m0 + wm * WTM + i * 32 + rl) * g.N + col;
-                v = v * alpha;
-                if constexpr (OT == SP_F32) {
-                    f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
-                    if (beta != 0.f) v += beta * *c;
-                    v += bias4;
-                    if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                    *c = v;
-                } else {
-                    u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
-                    if (beta != 0.f) {
-                        const u32x2 o = *c;
-                        v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
-                        v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
+                    for (int gq = 0; gq < 4; ++gq) {
+                        const f32x16& c16 = acc[i][js * SF + jj];
+                        f32x4 v = {c16[4 * gq], c16[4 * gq + 1], c16[4 * gq + 2], c16[4 * gq + 3]};
+                        *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (jj * 32 + gq * 8 + frag_half * 4) * 4) = v;
                     }
-                    v += bias4;
-                    if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                    u32x2 o;
-                    o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
-                    o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
-                    *c = o;
+                long idx = (m0 + wm * WTM + i * 32 + er) * g.N + col;     // advanced by RPP rows per pass
+#pragma unroll
+                for (int p = 0; p < 32 / RPP; ++p, idx += row_step) {
+                    const int rl = p * RPP + er;
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
+                    f32x4 old = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (OT == SP_F32) {
+                        f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
+                        if constexpr (HAS_BETA) old = *c;
+                        *c = finish(v, old, bias4);
+                    } else {
+                        u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
+                        if constexpr (HAS_BETA) {
+                            const u32x2 o = *c;
+                            old = f32x4{half_bits_to_f32<OT>(o.x & 0xffffu), half_bits_to_f32<OT>(o.x >> 16),
+                                        half_bits_to_f32<OT>(o.y & 0xffffu), half_bits_to_f32<OT>(o.y >> 16)};
+                        }
+                        const f32x4 r = finish(v, old, bias4);
+                        u32x2 o;
+                        o.x = pack_halves<OT>(r.x, r.y);
+                        o.y = pack_halves<OT>(r.z, r.w);
+                        *c = o;
+                    }
                 }
             }
         }
+    };
+    if (beta != 0.f) {
+        if (g.relu) write_tile(std::true_type{}, std::true_type{});
+        else write_tile(std::true_type{}, std::false_type{});
+    } else {
+        if (g.relu) write_tile(std::false_type{}, std::true_type{});
+        else write_tile(std::false_type{}, std::false_type{});
     }
 }
 
@@ -540,52 +559,82 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(const GemmArgs g) {
     // their results before the accumulators are read (18 wait states, which the compiler cannot know about)
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 
-    // ---- epilogue: per 16-row accumulator row, the wave transposes 16 x 128 values through a private LDS
-    //      strip and writes C (and, for beta != 0, reads it) as whole 512-byte (f32) row segments ----
+    // ---- epilogue: per 16-row accumulator row, the wave transposes 16 x 128 values through a private LDS strip
+    //      and writes C (and, for beta != 0, reads it) 16 bytes per lane: 512-byte row segments, two rows per
+    //      instruction for f32 output, 256-byte segments, four rows per instruction for 16-bit output ----
     constexpr int EPI_STRIDE = 128 * 4 + 16;
     static_assert(NW * 16 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
     __syncthreads();
     unsigned char* strip = lds + wave * (16 * EPI_STRIDE);
-    const int er = lane >> 5, ec = (lane & 31) * 4;          // 32 lanes per row, 2 rows per pass
+    constexpr int PER = OT == SP_F32 ? 4 : 8;                 // columns per lane
+    constexpr int LPR = 128 / PER;                            // lanes per row
+    constexpr int RPP = 64 / LPR;                             // rows per pass
+    const int er = lane / LPR, ec = (lane % LPR) * PER;
     const float alpha = g.alpha, beta = g.beta;
     const long col = n0 + wn * 128 + ec;
-    f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
-    if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
+    f32x4 bias4[PER / 4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            *reinterpret_cast<f32x4*>(strip + fi * EPI_STRIDE + (16 * j + 4 * fq) * 4) = acc[i][j];
-#pragma unroll
-        for (int p = 0; p < 8; ++p) {
-            const int rl = 2 * p + er;
-            f32x4 v = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
-            const long idx = (m0 + wm * 128 + i * 16 + rl) * g.N + col;
+    for (int h = 0; h < PER / 4; ++h) {
+        bias4[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+        if (g.bias) bias4[h] = *reinterpret_cast<const f32x4*>(g.bias + col + 4 * h);
+    }
+    // The options are compile-time inside the loops: a branch per output row would split them into blocks of one
+    // LDS read -> one store each, with every latency exposed.
+    auto write_tile = [&](auto BETA_, auto RELU_) {
+        constexpr bool HAS_BETA = decltype(BETA_)::value, RELU = decltype(RELU_)::value;
+        auto finish = [&](f32x4 v, const f32x4& old, const f32x4& bias) {
             v = v * alpha;
-            if constexpr (OT == SP_F32) {
-                f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
-                if (beta != 0.f) v += beta * *c;
-                v += bias4;
-                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                *c = v;
-            } else {
-                u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
-                if (beta != 0.f) {
-                    const u32x2 o = *c;
-                    v.x += beta * half_bits_to_f32<OT>(o.x & 0xffffu); v.y += beta * half_bits_to_f32<OT>(o.x >> 16);
-                    v.z += beta * half_bits_to_f32<OT>(o.y & 0xffffu); v.w += beta * half_bits_to_f32<OT>(o.y >> 16);
+            if constexpr (HAS_BETA) v += beta * old;
+            v += bias;
+            if constexpr (RELU) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
+            return v;
+        };
+        long idx = (m0 + wm * 128 + er) * g.N + col;      // advanced by RPP rows per pass
+        const long row_step = (long)RPP * g.N;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                *reinterpret_cast<f32x4*>(strip + fi * EPI_STRIDE + (16 * j + 4 * fq) * 4) = acc[i][j];
+#pragma unroll
+            for (int p = 0; p < 16 / RPP; ++p, idx += row_step) {
+                const int rl = RPP * p + er;
+                f32x4 old0 = {0.f, 0.f, 0.f, 0.f}, old1 = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (OT == SP_F32) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
+                    f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
+                    if constexpr (HAS_BETA) old0 = *c;
+                    *c = finish(v, old0, bias4[0]);
+                } else {
+                    const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
+                    const f32x4 v1 = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4 + 16);
+                    u32x4* c = reinterpret_cast<u32x4*>((unsigned short*)Cb + idx);
+                    if constexpr (HAS_BETA) {
+                        const u32x4 o = *c;
+                        old0 = f32x4{half_bits_to_f32<OT>(o.x & 0xffffu), half_bits_to_f32<OT>(o.x >> 16),
+                                     half_bits_to_f32<OT>(o.y & 0xffffu), half_bits_to_f32<OT>(o.y >> 16)};
+                        old1 = f32x4{half_bits_to_f32<OT>(o.z & 0xffffu), half_bits_to_f32<OT>(o.z >> 16),
+                                     half_bits_to_f32<OT>(o.w & 0xffffu), half_bits_to_f32<OT>(o.w >> 16)};
+                    }
+                    const f32x4 r0 = finish(v0, old0, bias4[0]), r1 = finish(v1, old1, bias4[PER / 4 - 1]);
+                    u32x4 o;
+                    o.x = pack_halves<OT>(r0.x, r0.y);
+                    o.y = pack_halves<OT>(r0.z, r0.w);
+                    o.z = pack_halves<OT>(r1.x, r1.y);
+                    o.w = pack_halves<OT>(r1.z, r1.w);
+                    *c = o;
                 }
-                v += bias4;
-                if (g.relu) { v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f); }
-                u32x2 o;
-                o.x = f32_to_half_bits<OT>(v.x) | (f32_to_half_bits<OT>(v.y) << 16);
-                o.y = f32_to_half_bits<OT>(v.z) | (f32_to_half_bits<OT>(v.w) << 16);
-                *c = o;
             }
         }
+    };
+    if (beta != 0.f) {
+        if (g.relu) write_tile(std::true_type{}, std::true_type{});
+        else write_tile(std::true_type{}, std::false_type{});
+    } else {
+        if (g.relu) write_tile(std::false_type{}, std::true_type{});
+        else write_tile(std::false_type{}, std::false_type{});
     }
 }
-
 
 // Shape-agnostic kernel: one thread per output element, 16-byte loads along K.  Used for shapes
 // the tiled kernels do not divide (the MLP's K = 32 or N = 3 for instance).
