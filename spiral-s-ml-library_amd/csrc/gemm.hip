@@ -3,6 +3,9 @@
 // A (M,K) and B (N,K) are both K-contiguous, so neither operand needs a transposing read: a
 // 32x32 MFMA fragment of either one is "32 rows x one 16-byte K-chunk per lane".
 //
+// Two tiled kernels: gemm_abt_w4_kernel (four waves, 16x16x32 MFMAs; large 16-bit shapes) and gemm_abt_kernel (eight or
+// four waves, 32x32 MFMAs; f32, small tiles, single-column outputs).
+//
 // Data movement per workgroup and K-tile (128 bytes of K per row: 64 bf16/f16 or 32 f32):
 //   global --global_load_lds_dwordx4 (DMA, no registers)--> LDS (double buffered, XOR-swizzled
 //   16-byte chunks) --ds_read_b128--> MFMA operands.  One barrier per K-tile; the DMA of tile k+1
