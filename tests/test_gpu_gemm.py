@@ -224,6 +224,8 @@ def test_device_and_kernel_info():
     assert info["arch"].startswith("gfx950") and info["compute_units"] >= 64 and info["wavefront_size"] == 64
     k = _lib.kernel_info("gemm_bf16_256x256")
     assert k["threads_per_block"] == 512 and k["vgprs"] > 64
+    k4 = _lib.kernel_info("gemm_bf16_256x256_4w")
+    assert k4["threads_per_block"] == 256 and k4["vgprs"] > 128
     with pytest.raises(_lib.SpiralError):
         _lib.kernel_info("no_such_kernel")
 
