@@ -705,7 +705,17 @@ struct TileCfg {
 static const TileCfg kTileCfgs[] = {{256, 256, 2, 4}, {128, 128, 2, 2}, {64, 64, 2, 2}};
 constexpr int kNumCfgs = 3;
 
-// Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.
+// The four-wave kernel takes the 256 x 256 tiles of 16-bit GEMMs whose K is a whole number of K-tile pairs and whose
+// B matrix spans more than one tile column; with a single column every A panel is read once, straight from HBM, and
+// two waves per SIMD hide that latency better (65536 x 256 x 2048: 85 us against 89-93 us).
+static bool use_four_waves(int dtype_in, long N, long K) {
+    return dtype_in != SP_F32 && K % 128 == 0 && K <= (1l << 22) && N >= 512;
+}
+
+// Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.  "Fills" is 80 %
+// of the compute units, except for the four-wave kernel, which does per unit so much more than the 128 x 128 tiles
+// that 9/16 of the units are enough (3072^3 bf16: 144 tiles of 256 x 256 take 56 us, 576 tiles of 128 x 128 76 us; at
+// 128 tiles the two are level, below that the smaller tiles win).
 static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
     const int bk = dtype_in == SP_F32 ? 32 : 64;
     if (K % bk != 0) return -1;
@@ -716,7 +726,8 @@ static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
         if (M % c.bm != 0 || N % c.bn != 0) continue;
         smallest = i;
         const long tiles = (M / c.bm) * (N / c.bn) * batch;
-        if (tiles * 5 >= (long)cus * 4) return i;
+        const bool four_waves = i == 0 && use_four_waves(dtype_in, N, K);
+        if (four_waves ? tiles * 16 >= (long)cus * 9 : tiles * 5 >= (long)cus * 4) return i;
     }
     return smallest;
 }
@@ -737,13 +748,6 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     const long tiles = (long)g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(WM * WN * 64), lds_bytes, stream, g);
     return check_launch("sp_gemm_abt");
-}
-
-// The four-wave kernel takes the 256 x 256 tiles of 16-bit GEMMs whose K is a whole number of K-tile pairs and whose
-// B matrix spans more than one tile column; with a single column every A panel is read once, straight from HBM, and
-// two waves per SIMD hide that latency better (65536 x 256 x 2048: 85 us against 89-93 us).
-static bool use_four_waves(int dtype_in, long N, long K) {
-    return dtype_in != SP_F32 && K % 128 == 0 && K <= (1l << 22) && N >= 512;
 }
 
 template <int DT, int OT>
