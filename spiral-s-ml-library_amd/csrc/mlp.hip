@@ -897,6 +897,19 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
         else
             return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x), c, 0, 0, 0);
     };
+    // The feature-split layers accumulate in architected registers, MFMAs issued from assembly: the conversion after
+    // a layer then reads the sums directly instead of copying 64 registers out of the accumulation file (with one
+    // wave per SIMD every instruction costs matrix-pipe time).  publish() supplies the wait states that the
+    // compiler would otherwise insert between the last MFMA and the first read of its result.
+    auto mfma_v = [&](f32x4& c, const u32x4& w, const u32x4& x, bool first) {
+        if (first) {
+            if constexpr (DT == SP_F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "v"(w), "v"(x));
+            else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "v"(w), "v"(x));
+        } else {
+            if constexpr (DT == SP_F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "v"(w), "v"(x));
+            else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "v"(w), "v"(x));
+        }
+    };
     f32x4 acc[4][4];                                         // [batch tile][feature tile]
     u32x4 wf[2][4], bf[2][4];                                // operands of k-step parity 0 / 1
     int r_stage = 0;                                         // ring stage of the chunk being multiplied
@@ -918,44 +931,51 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
 #pragma unroll
             for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_a(bt * 8192, 2 * KC);
         }
-        if constexpr (!half) {
-#pragma unroll
-            for (int t = 0; t < 4; ++t) wf[1][t] = read_w(r_stage, 1, t);
-#pragma unroll
-            for (int bt = 0; bt < 4; ++bt) bf[1][bt] = read_a(bt * 8192, 2 * KC + 1);
-        }
+        // operand reads of the other k-step go out one at a time behind the first MFMAs, in the order of their use
+        auto read1 = [&](int m) {
+            if (m == 0) wf[1][0] = read_w(r_stage, 1, 0);
+            else if (m < 5) bf[1][m - 1] = read_a((m - 1) * 8192, 2 * KC + 1);
+            else wf[1][m - 4] = read_w(r_stage, 1, m - 4);
+        };
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = 0; t < 4; ++t)
 #pragma unroll
-            for (int bt = 0; bt < 4; ++bt) acc[bt][t] = mfma(KC == 0 ? zero4 : acc[bt][t], wf[0][t], bf[0][bt]);
-        __builtin_amdgcn_sched_barrier(0);
+            for (int bt = 0; bt < 4; ++bt) {
+                mfma_v(acc[bt][t], wf[0][t], bf[0][bt], KC == 0);
+                if (!half && 4 * t + bt < 8) read1(4 * t + bt);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         if constexpr (issue) issue_chunk(IC<0>{});
         if constexpr (want_bias) load_bias(bias, valid);
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(WAITN) : "memory");
         const int next_stage = (r_stage + 1) & (SPLIT_STAGES - 1);
-        if constexpr (nextw) {
+        auto read0 = [&](int m) {
+            if (m == 0) { if constexpr (nextw) wf[0][0] = read_w(next_stage, 0, 0); }
+            else if (m < 5) { if constexpr (!lastk) bf[0][m - 1] = read_a((m - 1) * 8192, 2 * KC + 2); }
+            else { if constexpr (nextw) wf[0][m - 4] = read_w(next_stage, 0, m - 4); }
+        };
+        if constexpr (half) {
 #pragma unroll
-            for (int t = 0; t < 4; ++t) wf[0][t] = read_w(next_stage, 0, t);
-        }
-        if constexpr (!lastk) {
-#pragma unroll
-            for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_a(bt * 8192, 2 * KC + 2);
+            for (int m = 0; m < 8; ++m) read0(m);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (!half) {
 #pragma unroll
             for (int t = 0; t < 4; ++t)
 #pragma unroll
-                for (int bt = 0; bt < 4; ++bt) acc[bt][t] = mfma(acc[bt][t], wf[1][t], bf[1][bt]);
+                for (int bt = 0; bt < 4; ++bt) {
+                    mfma_v(acc[bt][t], wf[1][t], bf[1][bt], false);
+                    if (4 * t + bt < 8) read0(4 * t + bt);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
         }
-        __builtin_amdgcn_sched_barrier(0);
         r_stage = next_stage;
     };
     // the layer's outputs replace its inputs: barrier (every wave is done reading), bias, relu, rounding,
     // 16 bytes per (batch tile, tile pair), barrier
     auto publish = [&]() {
-        asm volatile("s_barrier" ::: "memory");
+        asm volatile("s_nop 15\n\ts_nop 3\n\ts_barrier" ::: "memory");   // the last MFMAs have written their results
 #pragma unroll
         for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(bias_r[i]));
         auto convert = [&](auto HAS_BIAS_) {
