@@ -63,7 +63,8 @@ int sp_device_info(sp_device_info_t* out);
 
 /* Occupancy report for a named kernel of this library: "gemm_bf16_256x256_4w", "gemm_f16_256x256_4w"
  * (four-wave kernel of the large 16-bit shapes), "gemm_bf16_256x256", "gemm_f16_256x256",
- * "gemm_bf16_128x128", "gemm_f32_64x64", "row_ops", "row_map", "mlp_forward", "mlp_forward_wide".
+ * "gemm_bf16_128x128", "gemm_f32_64x64", "row_ops", "row_ops_scalars" (sp_row_ops without probs/cdf
+ * outputs), "row_map", "mlp_forward", "mlp_forward_wide".
  * Registers, static LDS bytes and resident workgroups per CU (dynamic LDS not included).  Stands in
  * for ml/max_blocks_per_sm.py:2-31.  Returns SP_ERR_ARG for an unknown name. */
 typedef struct {

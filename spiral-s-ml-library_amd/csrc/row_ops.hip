@@ -342,19 +342,19 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 // are computed by the same operations in the same order); what differs is the instruction count:
 // padding lanes hold -inf, whose exponential is 0, so no per-element validity tests remain, full
 // waves load and store without predicates, and the max reductions are single DPP instructions.
-template <int T, int C>
-__global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs a) {
+template <int T, int C, bool MAT>
+__device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
     const int l = lane % T;
     const int sub = lane / T;
     const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
-    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    const long stride = (long)gridDim.x * (ROW_THREADS / WAVE) * ROWS_PER_WAVE;
     const float NEG_INF = -__builtin_inff();
     const int cols = a.cols;
     const bool full_cols = cols == C * 4 * T;
 
-    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += n_waves * ROWS_PER_WAVE) {
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += stride) {
         const long row = row0 + sub;
         const bool row_ok = row < a.rows;
         const bool full = full_cols && row0 + ROWS_PER_WAVE <= a.rows;   // wave-uniform
@@ -404,9 +404,10 @@ __global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs 
             for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
 
         const bool want_sample = a.sample != nullptr;
-        float cdf[C][4];
+        float cdf[MAT ? C : 1][4];
+        float first[C], last[C];   // running sum in front of / at the end of this lane's piece of chunk c
         int pick = INT_MAX_;
-        if (want_sample || a.cdf != nullptr) {
+        if (want_sample || (MAT && a.cdf != nullptr)) {
             float carry = 0.f;
 #pragma unroll
             for (int c = 0; c < C; ++c) {
@@ -414,11 +415,13 @@ __global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs 
                 float prev = dpp_move<0x138>(incl);   // wave_shr:1 = the lane before
                 if (l == 0) prev = 0.f;
                 float run = carry + prev;
+                first[c] = run;
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     run = run + p[c][k];
-                    cdf[c][k] = run;
+                    if (MAT) cdf[c][k] = run;
                 }
+                last[c] = run;
                 if (C > 1) carry = carry + group_broadcast_last<T>(incl);
             }
             if (want_sample) {
@@ -428,27 +431,40 @@ __global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs 
                 // the largest of them over p > 0 is the last one, provided the chunk's sum is positive.
                 float m = NEG_INF;
 #pragma unroll
-                for (int c = 0; c < C; ++c) m = vmax(m, sum4(p[c]) > 0.f ? cdf[c][3] : NEG_INF);
+                for (int c = 0; c < C; ++c) m = vmax(m, sum4(p[c]) > 0.f ? last[c] : NEG_INF);
                 m = group_max<T>(m);
                 const float uu = row_ok ? a.u[row] : 1.f;
                 const float thr = uu * m;
 #pragma unroll
-                for (int c = C - 1; c >= 0; --c)
+                for (int c = C - 1; c >= 0; --c) {
+                    // When the running sums are not written out they are not kept either: the same
+                    // additions in the same order give the same bits again.
+                    float r[4];
+                    float run = first[c];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        run = run + p[c][k];
+                        r[k] = MAT ? cdf[c][k] : run;
+                    }
 #pragma unroll
                     for (int k = 3; k >= 0; --k)
-                        if (p[c][k] > 0.f && cdf[c][k] >= thr) pick = c * 4 * T + 4 * l + k;
+                        if (p[c][k] > 0.f && r[k] >= thr) pick = c * 4 * T + 4 * l + k;
+                }
                 pick = group_reduce<T>(pick, [](int x, int y) { return x < y ? x : y; });
             }
         }
 
+        if (MAT) {
 #pragma unroll
-        for (int c = 0; c < C; ++c) {
-            if (full || (row_ok && c * 4 * T + 4 * l < cols)) {
-                if (a.out != nullptr)
-                    *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) = f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
-                if (a.cdf != nullptr)
-                    *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) =
-                        f32x4{cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]};
+            for (int c = 0; c < C; ++c) {
+                if (full || (row_ok && c * 4 * T + 4 * l < cols)) {
+                    if (a.out != nullptr)
+                        *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) =
+                            f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
+                    if (a.cdf != nullptr)
+                        *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) =
+                            f32x4{cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]};
+                }
             }
         }
         if (row_ok && l == 0) {
@@ -458,6 +474,22 @@ __global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs 
             if (a.sample != nullptr) a.sample[row] = pick;
         }
     }
+}
+
+// MAT = true: probabilities and/or running sums are written out.  Held to 64 registers (8 waves per
+// SIMD): with 4 loads and up to 8 stores of 16 bytes per lane in flight, more waves hide more.
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) __attribute__((amdgpu_waves_per_eu(8, 8))) void row_softmax_kernel(
+    const RowArgs a) {
+    row_softmax_body<T, C, true>(a);
+}
+
+// MAT = false: per-row results only.  Nothing of the row is written back and the running sums
+// are recomputed where the sample is picked instead of being kept, which frees a sixth of the
+// registers; the register limit above would cost this variant three spills.
+template <int T, int C>
+__global__ __launch_bounds__(ROW_THREADS) void row_softmax_scalars_kernel(const RowArgs a) {
+    row_softmax_body<T, C, false>(a);
 }
 
 // Integer rows: identity and exact scans (two's complement wrap-around).
@@ -662,8 +694,11 @@ static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
-        if (FUSED)
+        if (FUSED && (a.out != nullptr || a.cdf != nullptr))
             hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid),
+                               dim3(ROW_THREADS), 0, stream, a);
+        else if (FUSED)   // per-row results only: nothing of the row itself is written back
+            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid),
                                dim3(ROW_THREADS), 0, stream, a);
         else
             hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
@@ -677,6 +712,7 @@ namespace {
 struct RowKernelNames {
     RowKernelNames() {
         register_kernel("row_ops", (const void*)row_softmax_kernel<16, 4>, ROW_THREADS);
+        register_kernel("row_ops_scalars", (const void*)row_softmax_scalars_kernel<16, 4>, ROW_THREADS);
         register_kernel("row_map", (const void*)row_kernel<16, 4>, ROW_THREADS);
     }
 } row_kernel_names;

@@ -226,6 +226,10 @@ def test_device_and_kernel_info():
     assert k["threads_per_block"] == 512 and k["vgprs"] > 64
     k4 = _lib.kernel_info("gemm_bf16_256x256_4w")
     assert k4["threads_per_block"] == 256 and k4["vgprs"] > 128
+    for name in ("row_ops", "row_ops_scalars", "row_map"):
+        kr = _lib.kernel_info(name)
+        assert kr["threads_per_block"] == 256 and 0 < kr["vgprs"] <= 128
+    assert _lib.kernel_info("row_ops")["vgprs"] <= 64   # 8 waves per SIMD
     with pytest.raises(_lib.SpiralError):
         _lib.kernel_info("no_such_kernel")
 
