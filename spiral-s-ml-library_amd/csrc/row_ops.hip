@@ -354,23 +354,12 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
     const int cols = a.cols;
     const bool full_cols = cols == C * 4 * T;
 
-    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += stride) {
+    // Everything that happens to one group of ROWS_PER_WAVE rows once it is in registers.
+    auto work = [&](const f32x4 (&v)[C], const float uu, const long row0) {
         const long row = row0 + sub;
         const bool row_ok = row < a.rows;
         const bool full = full_cols && row0 + ROWS_PER_WAVE <= a.rows;   // wave-uniform
         const long base = row * (long)cols + 4 * l;
-
-        f32x4 v[C];
-        if (full) {
-#pragma unroll
-            for (int c = 0; c < C; ++c) v[c] = *reinterpret_cast<const f32x4*>(a.x + base + c * 4 * T);
-        } else {
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                v[c] = f32x4{NEG_INF, NEG_INF, NEG_INF, NEG_INF};
-                if (row_ok && c * 4 * T + 4 * l < cols) v[c] = *reinterpret_cast<const f32x4*>(a.x + base + c * 4 * T);
-            }
-        }
 
         float bv = vmax(vmax(v[0][0], v[0][1]), vmax(v[0][2], v[0][3]));
 #pragma unroll
@@ -403,8 +392,16 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 #pragma unroll
             for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
 
+        // Results that are rows themselves leave as soon as they exist, so that neither the
+        // probabilities' copy for the store nor the running sums stay in registers.
+        if (MAT && a.out != nullptr) {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                if (full || (row_ok && c * 4 * T + 4 * l < cols))
+                    *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) = f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
+        }
+
         const bool want_sample = a.sample != nullptr;
-        float cdf[MAT ? C : 1][4];
         float first[C], last[C];   // running sum in front of / at the end of this lane's piece of chunk c
         int pick = INT_MAX_;
         if (want_sample || (MAT && a.cdf != nullptr)) {
@@ -416,12 +413,15 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 if (l == 0) prev = 0.f;
                 float run = carry + prev;
                 first[c] = run;
+                float r[4];
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     run = run + p[c][k];
-                    if (MAT) cdf[c][k] = run;
+                    r[k] = run;
                 }
                 last[c] = run;
+                if (MAT && a.cdf != nullptr && (full || (row_ok && c * 4 * T + 4 * l < cols)))
+                    *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) = f32x4{r[0], r[1], r[2], r[3]};
                 if (C > 1) carry = carry + group_broadcast_last<T>(incl);
             }
             if (want_sample) {
@@ -433,18 +433,17 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 #pragma unroll
                 for (int c = 0; c < C; ++c) m = vmax(m, sum4(p[c]) > 0.f ? last[c] : NEG_INF);
                 m = group_max<T>(m);
-                const float uu = row_ok ? a.u[row] : 1.f;
                 const float thr = uu * m;
 #pragma unroll
                 for (int c = C - 1; c >= 0; --c) {
-                    // When the running sums are not written out they are not kept either: the same
-                    // additions in the same order give the same bits again.
+                    // The running sums are not kept: the same additions in the same order give
+                    // the same bits again.
                     float r[4];
                     float run = first[c];
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
                         run = run + p[c][k];
-                        r[k] = MAT ? cdf[c][k] : run;
+                        r[k] = run;
                     }
 #pragma unroll
                     for (int k = 3; k >= 0; --k)
@@ -454,39 +453,61 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
             }
         }
 
-        if (MAT) {
-#pragma unroll
-            for (int c = 0; c < C; ++c) {
-                if (full || (row_ok && c * 4 * T + 4 * l < cols)) {
-                    if (a.out != nullptr)
-                        *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) =
-                            f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
-                    if (a.cdf != nullptr)
-                        *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) =
-                            f32x4{cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]};
-                }
-            }
-        }
         if (row_ok && l == 0) {
             if (a.rowmax != nullptr) a.rowmax[row] = bv;
             if (a.rowsum != nullptr) a.rowsum[row] = s;
             if (a.argmax != nullptr) a.argmax[row] = bi;
             if (a.sample != nullptr) a.sample[row] = pick;
         }
+    };
+
+    // Whole groups of complete rows: as many 16-byte loads as chunks, none of them predicated.
+    auto load_full = [&](long r0, f32x4 (&w)[C], float& uu) {
+        const long r = r0 + sub;
+        const long b = r * (long)cols + 4 * l;
+        uu = a.u[r];   // first: whoever waits for a piece of the row then has the uniform too
+#pragma unroll
+        for (int c = 0; c < C; ++c) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
+    };
+    // Any group: -inf where the row or the tensor ends.
+    auto load_any = [&](long r0, f32x4 (&w)[C], float& uu) {
+        const long r = r0 + sub;
+        const long b = r * (long)cols + 4 * l;
+#pragma unroll
+        for (int c = 0; c < C; ++c) {
+            w[c] = f32x4{NEG_INF, NEG_INF, NEG_INF, NEG_INF};
+            if (r < a.rows && c * 4 * T + 4 * l < cols) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
+        }
+        uu = r < a.rows ? a.u[r] : 1.f;
+    };
+
+    // The uniform is requested together with the row: the counter of outstanding loads runs in
+    // order, so a load issued in the middle of the work would be waited for with nothing to do.
+    const long full_rows = full_cols ? a.rows - a.rows % ROWS_PER_WAVE : 0;
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < a.rows; row0 += stride) {
+        f32x4 v[C];
+        float uu;
+        // Two copies of the work, so that the common case stays a straight line: merged, the
+        // compiler orders the loads of both cases as row, wait, uniform, wait.
+        if (row0 < full_rows) {
+            load_full(row0, v, uu);
+            __builtin_amdgcn_sched_barrier(0);
+            work(v, uu, row0);
+        } else {
+            load_any(row0, v, uu);
+            work(v, uu, row0);
+        }
     }
 }
 
-// MAT = true: probabilities and/or running sums are written out.  Held to 64 registers (8 waves per
-// SIMD): with 4 loads and up to 8 stores of 16 bytes per lane in flight, more waves hide more.
+// MAT = true: probabilities and/or running sums are written out.
 template <int T, int C>
-__global__ __launch_bounds__(ROW_THREADS) __attribute__((amdgpu_waves_per_eu(8, 8))) void row_softmax_kernel(
+__global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(
     const RowArgs a) {
     row_softmax_body<T, C, true>(a);
 }
 
-// MAT = false: per-row results only.  Nothing of the row is written back and the running sums
-// are recomputed where the sample is picked instead of being kept, which frees a sixth of the
-// registers; the register limit above would cost this variant three spills.
+// MAT = false: per-row results only; nothing of the row is written back.
 template <int T, int C>
 __global__ __launch_bounds__(ROW_THREADS) void row_softmax_scalars_kernel(const RowArgs a) {
     row_softmax_body<T, C, false>(a);
@@ -687,9 +708,13 @@ static int check_rows_cols(const char* fn, int64_t rows, int64_t cols) {
 }
 
 template <bool FUSED>
-static int launch_row(const RowArgs& a, hipStream_t stream, const char* fn) {
+static int launch_row(const RowArgs& args, hipStream_t stream, const char* fn) {
     int rc = require_gfx950(fn);
     if (rc != SP_OK) return rc;
+    RowArgs a = args;
+    // The fused kernels read one uniform per row whether a sample is wanted or not; without one
+    // they read the first `rows` inputs instead, which exist because a row has at least 4 columns.
+    if (FUSED && a.u == nullptr) a.u = a.x;
     const int t = lanes_per_row(a.cols);
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
