@@ -229,8 +229,34 @@ def main():
                 res["cpu_gbs"] = round(nbytes / t / 1e9, 2)
             return res
 
+        def elementwise_case(kind):
+            # map / reduce / grid_transpose_snd of ml/primitives.spi on the row-primitive tensor shape
+            rng = np.random.default_rng(9)
+            rows, cols = 65536, 256
+            x = rng.standard_normal((rows, cols), dtype=np.float32)
+            xd = dev(x)
+            if kind == "map_relu":
+                out = torch.empty_like(xd)
+                fn = lambda: primitives.map("relu", xd, out=out)
+                nbytes = 2 * x.nbytes
+            elif kind == "reduce_sum":
+                from ml._lib import check, lib, ptr, stream_ptr
+                ws = torch.empty(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device="cuda")
+                out = torch.empty(4, dtype=torch.float32, device="cuda")
+                fn = lambda: check(lib.sp_reduce_sum(0, ptr(xd), ptr(out), xd.numel(), ptr(ws), ws.numel(), stream_ptr()))
+                nbytes = x.nbytes + 4
+            else:
+                out = torch.empty((cols, rows), dtype=torch.float32, device="cuda")
+                fn = lambda: primitives.transpose_snd(xd, out=out)
+                nbytes = 2 * x.nbytes
+            wall, ev = time_launches(fn, K, W)
+            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "roofline": roofline_hbm(nbytes, ev), "seed": 9}
+
         cases += [("mlp_leduc_16384", mlp_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
-                  ("row_ops_65536x256_materialised", lambda: rows_case(True))]
+                  ("row_ops_65536x256_materialised", lambda: rows_case(True)),
+                  ("map_relu_65536x256", lambda: elementwise_case("map_relu")),
+                  ("reduce_sum_f32_65536x256", lambda: elementwise_case("reduce_sum")),
+                  ("transpose_65536x256", lambda: elementwise_case("transpose"))]
     for name, fn in cases:
         if args.only and name != args.only:
             continue

@@ -10,7 +10,7 @@ namespace sp {
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int EW_THREADS = 256;
-constexpr int REDUCE_MAX_BLOCKS = 1024;
+constexpr int REDUCE_MAX_BLOCKS = 2048;
 
 template <int OP>
 __device__ __forceinline__ float map_op(float x) {
@@ -47,12 +47,30 @@ __device__ __forceinline__ T block_sum(T v, T* slots) {
     return r;  // valid in wave 0
 }
 
+// Per-block partial sums: 16-byte loads, four of them in flight per lane and four independent
+// running sums; the order of the additions depends only on n and the grid, so the result is the
+// same from run to run.
 template <typename T>
 __global__ __launch_bounds__(EW_THREADS) void reduce_partial_kernel(const T* __restrict__ x, T* __restrict__ partial, long n) {
     __shared__ T slots[EW_THREADS / WAVE];
-    T acc = T(0);
+    constexpr int V = 16 / sizeof(T);
+    typedef T VT __attribute__((ext_vector_type(V)));
+    const VT* xv = reinterpret_cast<const VT*>(x);
+    const long nv = n / V;
     const long stride = (long)gridDim.x * EW_THREADS;
-    for (long i = (long)blockIdx.x * EW_THREADS + threadIdx.x; i < n; i += stride) acc += x[i];
+    const long tid = (long)blockIdx.x * EW_THREADS + threadIdx.x;
+    VT a0 = VT(0), a1 = VT(0), a2 = VT(0), a3 = VT(0);
+    long i = tid;
+    for (; i + 3 * stride < nv; i += 4 * stride) {
+        const VT v0 = xv[i], v1 = xv[i + stride], v2 = xv[i + 2 * stride], v3 = xv[i + 3 * stride];
+        a0 += v0; a1 += v1; a2 += v2; a3 += v3;
+    }
+    for (; i < nv; i += stride) a0 += xv[i];
+    const VT a = (a0 + a1) + (a2 + a3);
+    T acc = a[0];
+#pragma unroll
+    for (int k = 1; k < V; ++k) acc += a[k];
+    for (long j = nv * V + tid; j < n; j += stride) acc += x[j];   // the last n % V elements
     acc = block_sum(acc, slots);
     if (threadIdx.x == 0) partial[blockIdx.x] = acc;
 }
@@ -88,9 +106,44 @@ __global__ __launch_bounds__(EW_THREADS) void transpose_kernel(const unsigned* _
     }
 }
 
+// The same for B and C multiples of 4: 16-byte reads and writes (a quarter of the memory
+// instructions), the transposition happens between four 4-byte LDS writes and four 4-byte LDS
+// reads per lane; with rows padded to 65 words both hit 64 different banks per wave.
+__global__ __launch_bounds__(EW_THREADS) void transpose_vec4_kernel(const unsigned* __restrict__ from,
+                                                                    unsigned* __restrict__ to, long B, long C,
+                                                                    long tiles_b, long tiles_c) {
+    typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+    __shared__ unsigned tile[64][65];
+    const long t = blockIdx.x;
+    const long a = t / (tiles_b * tiles_c);
+    const long tb = (t / tiles_c) % tiles_b, tc = t % tiles_c;
+    const unsigned* src = from + a * B * C;
+    unsigned* dst = to + a * B * C;
+    const int q = threadIdx.x & 15, r0 = threadIdx.x >> 4;   // 16 lanes per 64-word row, 16 rows per pass
+    u32x4 v[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const long b = tb * 64 + 16 * p + r0, c = tc * 64 + 4 * q;
+        v[p] = u32x4{0u, 0u, 0u, 0u};
+        if (b < B && c < C) v[p] = *reinterpret_cast<const u32x4*>(src + b * C + c);
+    }
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) tile[16 * p + r0][4 * q + k] = v[p][k];
+    __syncthreads();
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int cl = 16 * p + r0;
+        const long c = tc * 64 + cl, b = tb * 64 + 4 * q;
+        const u32x4 w = {tile[4 * q][cl], tile[4 * q + 1][cl], tile[4 * q + 2][cl], tile[4 * q + 3][cl]};
+        if (b < B && c < C) *reinterpret_cast<u32x4*>(dst + c * B + b) = w;
+    }
+}
+
 template <typename T>
 static int run_reduce(const void* x, void* out, int64_t n, void* workspace, hipStream_t stream) {
-    long blocks = (n + EW_THREADS * 8 - 1) / (EW_THREADS * 8);
+    long blocks = (n + EW_THREADS * 16 - 1) / (EW_THREADS * 16);   // >= 4 vectors of 16 bytes per lane
     if (blocks > REDUCE_MAX_BLOCKS) blocks = REDUCE_MAX_BLOCKS;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL(reduce_partial_kernel<T>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x,
@@ -159,7 +212,12 @@ extern "C" int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int
     const long tiles_b = (b + 63) / 64, tiles_c = (c + 63) / 64;
     const long blocks = a * tiles_b * tiles_c;
     if (blocks > 0x7fffffffL) return fail(SP_ERR_SHAPE, "sp_transpose_inner_b32: too many tiles");
-    hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, (hipStream_t)stream,
-                       (const unsigned*)from, (unsigned*)to, (long)b, (long)c, tiles_b, tiles_c);
+    const bool vec4 = b % 4 == 0 && c % 4 == 0 && ((uintptr_t)from | (uintptr_t)to) % 16 == 0;
+    if (vec4)
+        hipLaunchKernelGGL(transpose_vec4_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, (hipStream_t)stream,
+                           (const unsigned*)from, (unsigned*)to, (long)b, (long)c, tiles_b, tiles_c);
+    else
+        hipLaunchKernelGGL(transpose_kernel, dim3((unsigned)blocks), dim3(EW_THREADS), 0, (hipStream_t)stream,
+                           (const unsigned*)from, (unsigned*)to, (long)b, (long)c, tiles_b, tiles_c);
     return check_launch(__func__);
 }

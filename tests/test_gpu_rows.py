@@ -89,6 +89,33 @@ def test_golden_reduce_and_transpose(P, golden):
     assert (host(P.transpose_snd(y)) == orow.transpose_inner(host(y))).all()
 
 
+@pytest.mark.parametrize("shape", [(1, 4, 4), (2, 64, 64), (3, 68, 132), (1, 100, 8), (2, 4, 260), (5, 7, 9),
+                                   (1, 1, 257), (1, 1024, 256), (2, 6, 64)])
+def test_transpose_shapes(P, shape):
+    """Whole and partial 64x64 tiles, through the 16-byte kernel (both dimensions multiples of 4) and the 4-byte one."""
+    announce("transpose %s" % (shape,))
+    y = dev(np.random.default_rng(1).integers(-2 ** 31, 2 ** 31 - 1, size=shape, dtype=np.int64).astype(np.int32))
+    assert (host(P.transpose_snd(y)) == orow.transpose_inner(host(y))).all()
+    f = dev(np.random.default_rng(2).standard_normal(shape[1:], dtype=np.float32))
+    back = P.grid_transpose(P.grid_transpose(f))
+    assert (host(back) == host(f)).all()
+
+
+@pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, 262144 + 3, (1 << 22) + 1, 65536 * 256])
+def test_reduce_sizes(P, n):
+    """Exact for integers at every size (vector body, scalar tail, one block to the full grid); f32 against a
+    float64 sum, tolerance = a few ulps of the sum of magnitudes."""
+    announce("reduce n=%d" % n)
+    rng = np.random.default_rng(n)
+    xi = rng.integers(-1000, 1000, size=n, dtype=np.int32)
+    assert int(P.reduce_sum(dev(xi))) == int(xi.sum(dtype=np.int64))
+    xu = rng.integers(0, 2 ** 40, size=min(n, 1 << 20), dtype=np.int64)
+    assert int(P.reduce_sum(dev(xu))) == int(xu.sum())
+    xf = rng.standard_normal(n, dtype=np.float32)
+    want = float(xf.astype(np.float64).sum())
+    assert abs(float(P.reduce_sum(dev(xf))) - want) <= 1e-6 * float(np.abs(xf).sum(dtype=np.float64)) + 1e-6
+
+
 SHAPES = [(1, 4), (3, 12), (5, 16), (130, 64), (64, 128), (257, 256), (33, 260), (9, 512), (1000, 1024), (7, 1000)]
 
 
