@@ -141,6 +141,12 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             }
         }
 
+        // The row's uniform is requested (or computed) while the row itself is on its way: the
+        // counter of outstanding loads runs in order, so a load issued in mid-work is waited for
+        // with nothing else to do.
+        float uu = 0.f;
+        if (a.sample != nullptr && row_ok) uu = a.u != nullptr ? a.u[row] : reference_row_uniform(a, row);
+
         // ---- row max of the raw input, then argmax = lowest index holding it ----
         float bv = NEG_INF;
         int bi = INT_MAX_;
@@ -262,7 +268,6 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 
         // ---- inverse-CDF sampling (local_discrete_sampling, ml/primitives.spi:782-798) ----
         int pick = INT_MAX_;
-        float uu = 0.f;
         if (want_sample) {
             float m = NEG_INF;
 #pragma unroll
@@ -271,10 +276,6 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 for (int k = 0; k < 4; ++k)
                     if (p[c][k] > 0.f) m = fmaxf(m, cdf[c][k]);
             m = group_reduce<T>(m, [](float x, float y) { return fmaxf(x, y); });
-            if (row_ok) {
-                if (a.u != nullptr) uu = a.u[row];
-                else uu = reference_row_uniform(a, row);
-            }
             const float thr = uu * m;
 #pragma unroll
             for (int c = C - 1; c >= 0; --c)
@@ -458,6 +459,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
             if (a.rowsum != nullptr) a.rowsum[row] = s;
             if (a.argmax != nullptr) a.argmax[row] = bi;
             if (a.sample != nullptr) a.sample[row] = pick;
+            if (a.u_out != nullptr) a.u_out[row] = uu;
         }
     };
 
@@ -465,7 +467,8 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
     auto load_full = [&](long r0, f32x4 (&w)[C], float& uu) {
         const long r = r0 + sub;
         const long b = r * (long)cols + 4 * l;
-        uu = a.u[r];   // first: whoever waits for a piece of the row then has the uniform too
+        // first: whoever waits for a piece of the row then has the uniform too
+        uu = a.philox_mode >= 0 ? reference_row_uniform(a, r) : a.u[r];
 #pragma unroll
         for (int c = 0; c < C; ++c) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
     };
@@ -478,7 +481,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
             w[c] = f32x4{NEG_INF, NEG_INF, NEG_INF, NEG_INF};
             if (r < a.rows && c * 4 * T + 4 * l < cols) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
         }
-        uu = r < a.rows ? a.u[r] : 1.f;
+        uu = r < a.rows ? (a.philox_mode >= 0 ? reference_row_uniform(a, r) : a.u[r]) : 1.f;
     };
 
     // The uniform is requested together with the row: the counter of outstanding loads runs in
@@ -845,6 +848,8 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
         rc = set_philox(a, philox, rows, cols, __func__);
         if (rc != SP_OK) return rc;
     }
+    // Plain softmax sampling is what the fused pipeline does (same operations, same order, same bits).
+    if (op == SP_ROW_SOFTMAX && prob_out == nullptr) return launch_row<true>(a, (hipStream_t)stream, __func__);
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 

@@ -101,6 +101,24 @@ def test_transpose_shapes(P, shape):
     assert (host(back) == host(f)).all()
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 4), (5, 16), (130, 64), (257, 256), (33, 260), (1000, 1024), (7, 1000),
+                                       (4099, 256)])
+def test_fused_and_general_kernels_agree(P, rows, cols):
+    """Plain softmax sampling runs on the fused kernel, a mask that covers every column on the general one:
+    probabilities, running sums, uniforms and samples must agree bit for bit, with given and with device uniforms."""
+    announce("fused vs general %dx%d" % (rows, cols))
+    rng = np.random.default_rng(rows * 1000 + cols)
+    x = dev((rng.standard_normal((rows, cols), dtype=np.float32) * 2).astype(np.float32))
+    u = dev((1 - rng.random(rows, dtype=np.float32)).astype(np.float32))
+    for kw in (dict(u=u), dict(rng=P.philox())):
+        if "rng" in kw and (256 % (cols // 4) != 0):
+            continue   # the reference's generator needs threads_per_block to be a multiple of cols/4
+        a = P.softmax_and_discrete_sampling(x, want_cdf=True, want_u=True, **kw)
+        b = P.masked_softmax_and_discrete_sampling(x, cols, want_cdf=True, want_u=True, **kw)
+        for fa, fb in zip(a, b):
+            assert torch.equal(fa, fb)
+
+
 @pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, 262144 + 3, (1 << 22) + 1, 65536 * 256])
 def test_reduce_sizes(P, n):
     """Exact for integers at every size (vector body, scalar tail, one block to the full grid); f32 against a
