@@ -112,9 +112,10 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
     return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN>
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS = 2>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g) {
     constexpr int NT = WM * WN * 64;
+    static_assert(NS >= 2, "at least two LDS stages");
     constexpr int ES = (DT == SP_F32) ? 4 : 2;          // element size
     constexpr int BK = ROW_BYTES / ES;                   // elements of K per tile
     constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile
@@ -189,14 +190,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         for (int j = 0; j < TN; ++j)
             fb[j] = *reinterpret_cast<const u32x4*>(lds + vb[ks ^ (2 * (j & 1))] + j * 32 * ROW_BYTES);
     };
+    // NS stages form a ring; `cur` is the one being multiplied (two stages: a sign flip does it).
+    int cur = 0;
     int stage_delta = STAGE_BYTES;
-    auto toggle_stage = [&]() {
+    auto next_stage = [&](int kt) {
+        int released, delta;
+        if constexpr (NS == 2) {
+            released = kt & 1;
+            delta = stage_delta;
+            stage_delta = -stage_delta;
+        } else {
+            released = cur;
+            cur = (cur + 1 == NS) ? 0 : cur + 1;
+            delta = (cur == 0) ? -(NS - 1) * STAGE_BYTES : STAGE_BYTES;
+        }
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            va[t] += stage_delta;
-            vb[t] += stage_delta;
+            va[t] += delta;
+            vb[t] += delta;
         }
-        stage_delta = -stage_delta;
+        return released;
     };
     // The B fragment is the MFMA's first operand, so the result fragment is (n, m): register r of
     // lane l holds C[m = l % 32][n = 8 * (r / 4) + 4 * (l / 32) + r % 4], 4 consecutive columns per
@@ -232,15 +245,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     // that was just released.
     const int nk = (int)(K / BK);
     u32x4 fa[2][TM], fb[2][TN];
+    // Prologue: the first NS K-tiles (as many as there are) go out at once, one per stage.
 #pragma unroll
-    for (int q = 0; q < NI; ++q) dma_to_lds(src[q], lane_off[q], dst[q]);
-    if (nk > 1) {
+    for (int st = 0; st < NS; ++st) {
+        if (st < nk) {
 #pragma unroll
-        for (int q = 0; q < NI; ++q) {
-            src[q] += ROW_BYTES;
-            dma_to_lds(src[q], lane_off[q], dst[q] + STAGE_BYTES);
+            for (int q = 0; q < NI; ++q) {
+                if (st > 0) src[q] += ROW_BYTES;
+                dma_to_lds(src[q], lane_off[q], dst[q] + st * STAGE_BYTES);
+            }
         }
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");  // tile 0 landed, tile 1 may be in flight
+    }
+    if (nk >= NS) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * NI) : "memory");  // tile 0 landed, NS - 1 tiles may be in flight
     } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
@@ -259,17 +276,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     const bool dma_first = __builtin_amdgcn_readfirstlane(wave) < NW / 2;
     for (int kt = 0; kt + 1 < nk; ++kt) {
         first_three_steps();
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        // Tile kt + 1 must have landed.  While every stage behind it is still being filled that is
+        // "at most NS - 2 tiles outstanding" (the counter runs in order); near the end fewer tiles
+        // are in flight and only "none outstanding" says it.
+        if (NS > 2 && kt + NS <= nk) {
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NS - 2) * NI) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        }
         __syncthreads();
-        toggle_stage();
+        const int released = next_stage(kt);
         // The two waves of a SIMD take turns: a wave issuing its DMA instructions waits at the texture
         // path's queue (one 1 KiB instruction per ~16 cycles, 8 waves x NI of them per tile: measured
         // ~600 cycles per wave and tile) and issues no MFMA meanwhile, so one wave of each pair fetches
         // before the last k-step's MFMAs and the other one after them.  Only the DMA issue sits in the
         // (wave-uniform) branches: MFMAs in both arms would make the compiler copy the accumulators.
         auto issue_dma = [&]() {
-            if (kt + 2 < nk) {
-                const unsigned stage_off = (kt & 1) * STAGE_BYTES;
+            if (kt + NS < nk) {
+                const unsigned stage_off = (unsigned)released * STAGE_BYTES;
 #pragma unroll
                 for (int q = 0; q < NI; ++q) {
                     src[q] += ROW_BYTES;
@@ -732,10 +756,10 @@ static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
     return smallest;
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN>
-static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
-    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN>;
-    const int lds_bytes = 2 * (BM + BN) * ROW_BYTES;
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS>
+static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
+    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS>;
+    const int lds_bytes = NS * (BM + BN) * ROW_BYTES;
     static bool attr_set[64] = {false};
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -748,6 +772,24 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     const long tiles = (long)g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(WM * WN * 64), lds_bytes, stream, g);
     return check_launch("sp_gemm_abt");
+}
+
+// Two LDS stages keep several small workgroups on a compute unit.  When the grid has at most one
+// workgroup per unit anyway, 16-bit GEMMs with a long K give the whole LDS to one deep ring instead
+// (128 KiB: 4 stages of a 128 x 128 tile, 8 of a 64 x 64 tile): a K-tile of a small 16-bit tile is
+// multiplied in far less time than a load takes to arrive, and with two stages every tile waits
+// for its data (1024 x 1024 x 8192 bf16: 51.7 -> 34.2 us).  Measured and left on two stages: f32
+// (its K-tile takes 1024 cycles of MFMA and the deep ring was 5-9 % slower) and short K (the burst
+// of the prologue delays the first tile: 2048 x 2048 x 512 bf16 9.7 -> 10.4 us).
+template <int DT, int OT, int BM, int BN, int WM, int WN>
+static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
+    constexpr int DEEP = (128 * 1024) / ((BM + BN) * ROW_BYTES);
+    if constexpr (DEEP > 2 && DT != SP_F32) {
+        constexpr int BK = ROW_BYTES / 2;
+        if ((long)g.tiles_m * g.tiles_n * g.batch <= (long)device_cu_count() && g.K / BK >= 32)
+            return launch_tiled_stages<DT, OT, BM, BN, WM, WN, DEEP>(g, stream);
+    }
+    return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2>(g, stream);
 }
 
 template <int DT, int OT>

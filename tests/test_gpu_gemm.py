@@ -44,6 +44,25 @@ def test_tiled_shapes(MM, dtype, m, n, k):
     assert ogemm.rel_frobenius(generic, ogemm.gemm_abt(a, b)) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(512, 512, 4096), (1024, 1024, 2048), (2048, 2048, 2048), (512, 512, 2112),
+                                   (1024, 2048, 2240), (256, 256, 8192)])
+def test_long_k_small_grids(MM, dtype, m, n, k):
+    """16-bit shapes with at most one workgroup per compute unit and >= 32 K-tiles run on the deep LDS ring
+    (8 stages of 64 x 64 tiles, 4 of 128 x 128), including K-tile counts that are no multiple of the ring length.
+    Integer operands make the comparison exact, so a tile read from the wrong stage cannot hide in a tolerance."""
+    announce("gemm deep ring %s %dx%dx%d" % (dtype, m, n, k))
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a, b = make(rng, m, n, k, dtype)
+    assert ogemm.rel_frobenius(run(MM, a, b, dtype), ogemm.gemm_abt(a, b)) < TOL[dtype]
+    ai = rng.integers(-2, 3, size=(m, k)).astype(np.float32)
+    bi = rng.integers(-2, 3, size=(n, k)).astype(np.float32)
+    # every K-tile of 64 gets its own weight so that a swapped or repeated tile changes the sum
+    w = (np.arange(k) // 64 % 5 + 1).astype(np.float32)
+    want = (ai * w).astype(np.int64) @ bi.astype(np.int64).T
+    assert (run(MM, ai * w, bi, dtype).astype(np.int64) == want).all()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 def test_integer_inputs_are_exact(MM, dtype):
     """Small integers are exact in every dtype and every partial sum fits f32: any indexing slip
