@@ -92,8 +92,14 @@ def check(rc):
         raise SpiralError(rc, lib.sp_last_error_string().decode())
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr():
-    """torch's current HIP stream as a hipStream_t."""
+    """torch's current HIP stream as a hipStream_t.  The raw query skips the Stream object, which costs
+    several microseconds per call: as much as a small kernel."""
+    if _raw_stream is not None:
+        return C.c_void_p(_raw_stream(torch.cuda.current_device()))
     return C.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
