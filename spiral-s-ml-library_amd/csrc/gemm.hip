@@ -40,6 +40,7 @@ struct GemmArgs {
     long stride_a, stride_b, stride_c;   // bytes between the matrices of a batch (0: shared)
     int batch;
     int group_m;   // tile rows per group of the block -> tile walk (4: an XCD's 32 concurrent tiles form a 4 x 8 patch)
+    int k_rotate;  // workgroup t starts its K loop at K-tile (t * k_rotate) % nk and wraps around (0: everyone at 0)
 };
 
 constexpr int ROW_BYTES = 128;  // bytes of K per LDS row and K-tile
@@ -112,10 +113,16 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
     return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN, int NS = 2>
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS = 2, int NSA = NS>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g) {
     constexpr int NT = WM * WN * 64;
     static_assert(NS >= 2, "at least two LDS stages");
+    // NSA != NS: the A tiles have a ring of their own, longer than B's (which then has two stages).  A is what
+    // comes from HBM when B is a single tile column that every workgroup shares through the L2.
+    constexpr bool SPLIT_RING = NSA != NS;
+    static_assert(!SPLIT_RING || (NS == 2 && NSA > NS), "a separate A ring goes with a two-stage B ring");
+    constexpr int ABYTES = BM * ROW_BYTES, BBYTES = BN * ROW_BYTES;
+    constexpr int B_BASE = SPLIT_RING ? NSA * ABYTES : ABYTES;   // where the B tile of stage 0 starts
     constexpr int ES = (DT == SP_F32) ? 4 : 2;          // element size
     constexpr int BK = ROW_BYTES / ES;                   // elements of K per tile
     constexpr int WTM = BM / WM, WTN = BN / WN;          // wave tile
@@ -158,7 +165,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         const unsigned char* origin = is_a ? Ab + (m0 + blk * 8) * K * ES : Bb + (n0 + blk * 8) * K * ES;
         src[q] = uniform_ptr(origin);
         lane_off[q] = (unsigned)(r * K * ES + kc * 16);
-        dst[q] = __builtin_amdgcn_readfirstlane(lds_base + (is_a ? 0 : BM * ROW_BYTES) + blk * 8 * ROW_BYTES);
+        dst[q] = __builtin_amdgcn_readfirstlane(lds_base + (is_a ? 0 : B_BASE) + blk * 8 * ROW_BYTES);
     }
 
     f32x16 acc[TM][TN];
@@ -180,7 +187,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         va[t] = lds_offset(wm * WTM + frag_row, 2 * t + frag_half);
-        vb[t] = BM * ROW_BYTES + lds_offset(wn * WTN + frag_row, 2 * t + frag_half);
+        vb[t] = B_BASE + lds_offset(wn * WTN + frag_row, 2 * t + frag_half);
     }
     auto load_frags = [&](int ks, u32x4(&fa)[TM], u32x4(&fb)[TN]) {
 #pragma unroll
@@ -195,7 +202,18 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     int stage_delta = STAGE_BYTES;
     auto next_stage = [&](int kt) {
         int released, delta;
-        if constexpr (NS == 2) {
+        if constexpr (SPLIT_RING) {
+            released = cur;                                   // the A stage; B's is kt & 1
+            cur = (cur + 1 == NSA) ? 0 : cur + 1;
+            const int da = (cur == 0) ? -(NSA - 1) * ABYTES : ABYTES;
+            const int db = (kt & 1) ? -BBYTES : BBYTES;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                va[t] += da;
+                vb[t] += db;
+            }
+            return released;
+        } else if constexpr (NS == 2) {
             released = kt & 1;
             delta = stage_delta;
             stage_delta = -stage_delta;
@@ -245,6 +263,46 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     // that was just released.
     const int nk = (int)(K / BK);
     u32x4 fa[2][TM], fb[2][TN];
+    // Where this workgroup's K loop starts (split ring only): all workgroups walking K in step would ask the
+    // memory system for the same column offsets of 256 different rows each at the same time.
+    int left_a = nk, left_b = nk;      // tiles until the walk wraps around to K-tile 0
+    if constexpr (SPLIT_RING) {
+        const int kt0 = (int)(((long)blockIdx.x * g.k_rotate) % nk);
+#pragma unroll
+        for (int q = 0; q < NI; ++q) src[q] += (long)kt0 * ROW_BYTES;
+        left_a = left_b = nk - kt0;
+    }
+    auto next_a = [&]() { return --left_a == 0 ? -(long)(nk - 1) * ROW_BYTES : (long)ROW_BYTES; };
+    auto next_b = [&]() { return --left_b == 0 ? -(long)(nk - 1) * ROW_BYTES : (long)ROW_BYTES; };
+    if constexpr (SPLIT_RING) {
+        // Issue order, here and in the loop: B tile j + 2, then A tile j + NSA, for j = -NSA, -NSA + 1, ...  The
+        // counter of outstanding loads runs in order; with B ahead of A in every pair, "B tile kt + 1 has landed"
+        // leaves exactly the NIA instructions of the A tile issued behind it outstanding.
+#pragma unroll
+        for (int j = -NSA; j < 0; ++j) {
+            if (j + 2 >= 0 && j + 2 < nk) {
+                const long step = j + 2 > 0 ? next_b() : 0;
+#pragma unroll
+                for (int q = NIA; q < NI; ++q) {
+                    src[q] += step;
+                    dma_to_lds(src[q], lane_off[q], dst[q] + (j + 2) * BBYTES);
+                }
+            }
+            if (j + NSA < nk) {
+                const long step = j + NSA > 0 ? next_a() : 0;
+#pragma unroll
+                for (int q = 0; q < NIA; ++q) {
+                    src[q] += step;
+                    dma_to_lds(src[q], lane_off[q], dst[q] + (j + NSA) * ABYTES);
+                }
+            }
+        }
+        if (nk >= NSA) {   // behind B tile 0: A tile NSA - 2, B tile 1, A tile NSA - 1
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NIA + NI) : "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+    } else {
     // Prologue: the first NS K-tiles (as many as there are) go out at once, one per stage.
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
@@ -260,6 +318,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * NI) : "memory");  // tile 0 landed, NS - 1 tiles may be in flight
     } else {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
     }
     __syncthreads();
     load_frags(0, fa[0], fb[0]);
@@ -279,7 +338,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         // Tile kt + 1 must have landed.  While every stage behind it is still being filled that is
         // "at most NS - 2 tiles outstanding" (the counter runs in order); near the end fewer tiles
         // are in flight and only "none outstanding" says it.
-        if (NS > 2 && kt + NS <= nk) {
+        if (SPLIT_RING && kt + NSA <= nk) {
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(NIA) : "memory");
+        } else if (!SPLIT_RING && NS > 2 && kt + NS <= nk) {
             asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"((NS - 2) * NI) : "memory");
         } else {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -292,7 +353,26 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
         // before the last k-step's MFMAs and the other one after them.  Only the DMA issue sits in the
         // (wave-uniform) branches: MFMAs in both arms would make the compiler copy the accumulators.
         auto issue_dma = [&]() {
-            if (kt + NS < nk) {
+            if constexpr (SPLIT_RING) {
+                if (kt + 2 < nk) {
+                    const unsigned stage_off = (unsigned)(kt & 1) * BBYTES;
+                    const long step = next_b();
+#pragma unroll
+                    for (int q = NIA; q < NI; ++q) {
+                        src[q] += step;
+                        dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
+                    }
+                }
+                if (kt + NSA < nk) {
+                    const unsigned stage_off = (unsigned)released * ABYTES;
+                    const long step = next_a();
+#pragma unroll
+                    for (int q = 0; q < NIA; ++q) {
+                        src[q] += step;
+                        dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
+                    }
+                }
+            } else if (kt + NS < nk) {
                 const unsigned stage_off = (unsigned)released * STAGE_BYTES;
 #pragma unroll
                 for (int q = 0; q < NI; ++q) {
@@ -756,10 +836,10 @@ static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
     return smallest;
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN, int NS>
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS, int NSA = NS>
 static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
-    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS>;
-    const int lds_bytes = NS * (BM + BN) * ROW_BYTES;
+    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS, NSA>;
+    const int lds_bytes = (NSA * BM + NS * BN) * ROW_BYTES;
     static bool attr_set[64] = {false};
     int dev = 0;
     (void)hipGetDevice(&dev);
@@ -784,6 +864,12 @@ static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
 template <int DT, int OT, int BM, int BN, int WM, int WN>
 static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     constexpr int DEEP = (128 * 1024) / ((BM + BN) * ROW_BYTES);
+    if constexpr (BM == 256 && BN == 256 && DT != SP_F32) {
+        // B is a single tile column: every A panel comes straight from HBM, once, and one 32 KiB stage of it in
+        // flight per compute unit is too little to cover that latency (8 MiB over the chip).  The 32 KiB of LDS that
+        // two 64 KiB stages leave over become a third A stage.
+        if (g.tiles_n == 1 && g.K / (ROW_BYTES / 2) >= 4) return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2, 3>(g, stream);
+    }
     if constexpr (DEEP > 2 && DT != SP_F32) {
         constexpr int BK = ROW_BYTES / 2;
         if ((long)g.tiles_m * g.tiles_n * g.batch <= (long)device_cu_count() && g.K / BK >= 32)
@@ -897,6 +983,7 @@ static int gemm_entry(const char* fn, int dtype_in, int dtype_out, const void* A
     g.relu = (flags & SP_GEMM_RELU) ? 1 : 0;
     g.out_dtype = dtype_out;
     g.group_m = 4;
+    g.k_rotate = 7;   // odd: coprime with the power-of-two K-tile counts of the usual shapes (measured: 1, 3, ..., 13 all within 1 %)
     g.batch = (int)batch;
     g.stride_a = stride_a * es_in; g.stride_b = stride_b * es_in; g.stride_c = stride_c * es_out;
     if (cfg >= 0) {

@@ -63,6 +63,23 @@ def test_long_k_small_grids(MM, dtype, m, n, k):
     assert (run(MM, ai * w, bi, dtype).astype(np.int64) == want).all()
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("k", [256, 320, 384, 448, 2048])
+def test_single_tile_column_a_ring(MM, dtype, k):
+    """N = 256 with enough rows for 256 x 256 tiles: the A tiles run through a three-stage ring of their own next to
+    B's two stages.  K-tile counts 4..7 and 32 cover every phase of both rings and the drain at the end; integer
+    operands with a weight per K-tile make a tile read from the wrong stage change the exact result."""
+    announce("gemm A ring %s 65536x256x%d" % (dtype, k))
+    m, n = 65536, 256
+    rng = np.random.default_rng(k)
+    w = (np.arange(k) // 64 % 5 + 1).astype(np.float32)
+    ai = rng.integers(-2, 3, size=(m, k)).astype(np.float32) * w
+    bi = rng.integers(-2, 3, size=(n, k)).astype(np.float32)
+    want = ai.astype(np.float64) @ bi.astype(np.float64).T     # exact: |sum| < 2^53
+    got = run(MM, ai, bi, dtype)
+    assert (got.astype(np.float64) == want).all()
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 def test_integer_inputs_are_exact(MM, dtype):
     """Small integers are exact in every dtype and every partial sum fits f32: any indexing slip
