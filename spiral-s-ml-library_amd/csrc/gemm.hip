@@ -868,7 +868,7 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
         // B is a single tile column: every A panel comes straight from HBM, once, and one 32 KiB stage of it in
         // flight per compute unit is too little to cover that latency (8 MiB over the chip).  The 32 KiB of LDS that
         // two 64 KiB stages leave over become a third A stage.
-        if (g.tiles_n == 1 && g.K / (ROW_BYTES / 2) >= 4) return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2, 3>(g, stream);
+        if (g.tiles_n == 1 && g.K / (ROW_BYTES / 2) >= 8) return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2, 3>(g, stream);
     }
     if constexpr (DEEP > 2 && DT != SP_F32) {
         constexpr int BK = ROW_BYTES / 2;

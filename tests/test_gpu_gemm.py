@@ -64,10 +64,10 @@ def test_long_k_small_grids(MM, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("k", [256, 320, 384, 448, 2048])
+@pytest.mark.parametrize("k", [512, 576, 640, 704, 2048])
 def test_single_tile_column_a_ring(MM, dtype, k):
     """N = 256 with enough rows for 256 x 256 tiles: the A tiles run through a three-stage ring of their own next to
-    B's two stages.  K-tile counts 4..7 and 32 cover every phase of both rings and the drain at the end; integer
+    B's two stages.  K-tile counts 8..11 and 32 cover every phase of both rings and the drain at the end; integer
     operands with a weight per K-tile make a tile read from the wrong stage change the exact result."""
     announce("gemm A ring %s 65536x256x%d" % (dtype, k))
     m, n = 65536, 256
