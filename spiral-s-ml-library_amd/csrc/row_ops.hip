@@ -820,6 +820,7 @@ extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, 
     RowArgs a{};
     a.x = x; a.out = out; a.rows = rows; a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols;
     a.philox_mode = -1;
+    if (op == SP_ROW_SOFTMAX) return launch_row<true>(a, (hipStream_t)stream, __func__);   // the fused kernel's first half
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 

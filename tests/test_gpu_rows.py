@@ -117,6 +117,7 @@ def test_fused_and_general_kernels_agree(P, rows, cols):
         b = P.masked_softmax_and_discrete_sampling(x, cols, want_cdf=True, want_u=True, **kw)
         for fa, fb in zip(a, b):
             assert torch.equal(fa, fb)
+    assert torch.equal(P.softmax(x), P.masked_softmax(x, cols))     # the map alone: fused kernel vs general kernel
 
 
 @pytest.mark.parametrize("n", [1, 3, 4, 5, 1023, 4096, 262144 + 3, (1 << 22) + 1, 65536 * 256])
