@@ -97,8 +97,9 @@ int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
  *   type of C (SP_F32, or the same 16-bit type as the input).  bias (N,) f32 may be NULL.
  *   alpha must be non-zero (kernel.spi:49).  beta == 0 means C is never read, so NaNs in the
  *   old C do not propagate (kernel.spi:152-154).
- *   Fast MFMA path: M, N multiples of 64 and K a multiple of 64 (16-bit) / 32 (f32); any other
- *   positive shape with K a multiple of 8 (16-bit) / 4 (f32) runs on a slower general kernel.
+ *   K must be a multiple of 8 (16-bit) / 4 (f32): rows of A and B are whole 16-byte chunks.  Every such
+ *   shape with N a multiple of 4 runs on the tiled MFMA kernels (tiles that overhang M, N or K are
+ *   masked); only N not a multiple of 4 falls back to a slow one-thread-per-output kernel.
  */
 int sp_gemm_abt(int dtype_in, int dtype_out, const void* A, const void* B, void* C, const float* bias,
                 int64_t M, int64_t N, int64_t K, float alpha, float beta, uint32_t flags, void* stream);

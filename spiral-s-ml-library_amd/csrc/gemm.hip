@@ -40,6 +40,7 @@ struct GemmArgs {
     long stride_a, stride_b, stride_c;   // bytes between the matrices of a batch (0: shared)
     int batch;
     int group_m;   // tile rows per group of the block -> tile walk (4: an XCD's 32 concurrent tiles form a 4 x 8 patch)
+    int ragged;    // M or N is not a multiple of the tile: tiles_m / tiles_n are rounded up
     int k_rotate;  // workgroup t starts its K loop at K-tile (t * k_rotate) % nk and wraps around (0: everyone at 0)
 };
 
@@ -106,6 +107,13 @@ __device__ __forceinline__ void dma_to_lds(const unsigned char* base, unsigned l
                  : "memory");
 }
 
+// The same with a full address per lane (the last, partial K-tile of a ragged K: chunks past the end of a row
+// are fetched from a block of zeros instead).
+__device__ __forceinline__ void dma_to_lds_addr(const unsigned char* addr, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(addr), "s"(lds_addr) : "memory");
+}
+__device__ __attribute__((aligned(16))) const unsigned kZeroChunk[4] = {0u, 0u, 0u, 0u};
+
 __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char* p) {
     const unsigned long long v = (unsigned long long)p;
     const unsigned lo = __builtin_amdgcn_readfirstlane((unsigned)v);
@@ -113,7 +121,10 @@ __device__ __forceinline__ const unsigned char* uniform_ptr(const unsigned char*
     return (const unsigned char*)(((unsigned long long)hi << 32) | lo);
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN, int NS = 2, int NSA = NS>
+// RAGGED: M, N and K need not be multiples of the tile (N a multiple of 4, K of 16 bytes).  Rows past the end are
+// fetched as copies of the last row and the chunks of the last K-tile that lie past the end of a row as zeros, so
+// every load stays inside the matrices, and the epilogue skips what lies outside C.
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS = 2, int NSA = NS, bool RAGGED = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g) {
     constexpr int NT = WM * WN * 64;
     static_assert(NS >= 2, "at least two LDS stages");
@@ -156,15 +167,25 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     const unsigned char* src[NI];
     unsigned lane_off[NI];
     unsigned dst[NI];
+    const int nk = RAGGED ? (int)((K + BK - 1) / BK) : (int)(K / BK);
+    const bool k_tail = RAGGED && K % BK != 0;   // the last K-tile is partial
+    unsigned tail_in = 0;                        // bit q: this lane's chunk of the last K-tile lies inside the row
 #pragma unroll
     for (int q = 0; q < NI; ++q) {
         const bool is_a = q < NIA;
         const int blk = (is_a ? q : q - NIA) * NW + wave;           // row block inside the A (or B) tile
         const int r = lane >> 3;                                    // row inside the block
         const int kc = (lane & 7) ^ ((r ^ blk) & 7);                // global chunk that belongs in slot lane & 7
-        const unsigned char* origin = is_a ? Ab + (m0 + blk * 8) * K * ES : Bb + (n0 + blk * 8) * K * ES;
+        long first = (is_a ? m0 : n0) + blk * 8, mine = first + r;      // first row of the block, this lane's row
+        if constexpr (RAGGED) {
+            const long last = (is_a ? g.M : g.N) - 1;
+            first = first < last ? first : last;
+            mine = first + r < last ? first + r : last;
+        }
+        const unsigned char* origin = (is_a ? Ab : Bb) + first * K * ES;
         src[q] = uniform_ptr(origin);
-        lane_off[q] = (unsigned)(r * K * ES + kc * 16);
+        lane_off[q] = (unsigned)((mine - first) * K * ES + kc * 16);
+        if ((long)(nk - 1) * CHUNKS + kc < K * ES / 16) tail_in |= 1u << q;
         dst[q] = __builtin_amdgcn_readfirstlane(lds_base + (is_a ? 0 : B_BASE) + blk * 8 * ROW_BYTES);
     }
 
@@ -261,8 +282,25 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     // share of the next tile has landed), request the next tile's first fragments, run the last
     // step's MFMAs under that latency, then start the DMA of the tile after next into the stage
     // that was just released.
-    const int nk = (int)(K / BK);
     u32x4 fa[2][TM], fb[2][TN];
+    // The next K-tile of every DMA instruction of this wave (src[] is advanced to it first) into the stage at
+    // byte offset `stage_off`; one branch per tile, not per instruction.
+    auto fetch_tile = [&](int tile, unsigned stage_off, bool advance) {
+        if (k_tail && tile == nk - 1) {
+#pragma unroll
+            for (int q = 0; q < NI; ++q) {
+                if (advance) src[q] += ROW_BYTES;
+                const unsigned char* inside = src[q] + lane_off[q];
+                dma_to_lds_addr((tail_in >> q) & 1u ? inside : (const unsigned char*)kZeroChunk, dst[q] + stage_off);
+            }
+        } else {
+#pragma unroll
+            for (int q = 0; q < NI; ++q) {
+                if (advance) src[q] += ROW_BYTES;
+                dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
+            }
+        }
+    };
     // Where this workgroup's K loop starts (split ring only): all workgroups walking K in step would ask the
     // memory system for the same column offsets of 256 different rows each at the same time.
     int left_a = nk, left_b = nk;      // tiles until the walk wraps around to K-tile 0
@@ -306,13 +344,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
     // Prologue: the first NS K-tiles (as many as there are) go out at once, one per stage.
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
-        if (st < nk) {
-#pragma unroll
-            for (int q = 0; q < NI; ++q) {
-                if (st > 0) src[q] += ROW_BYTES;
-                dma_to_lds(src[q], lane_off[q], dst[q] + st * STAGE_BYTES);
-            }
-        }
+        if (st < nk) fetch_tile(st, st * STAGE_BYTES, st > 0);
     }
     if (nk >= NS) {
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NS - 1) * NI) : "memory");  // tile 0 landed, NS - 1 tiles may be in flight
@@ -373,12 +405,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
                     }
                 }
             } else if (kt + NS < nk) {
-                const unsigned stage_off = (unsigned)released * STAGE_BYTES;
-#pragma unroll
-                for (int q = 0; q < NI; ++q) {
-                    src[q] += ROW_BYTES;
-                    dma_to_lds(src[q], lane_off[q], dst[q] + stage_off);
-                }
+                fetch_tile(kt + NS, (unsigned)released * STAGE_BYTES, true);
             }
         };
         if (dma_first) issue_dma();
@@ -422,8 +449,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
 #pragma unroll
             for (int js = 0; js < TN / SF; ++js) {
                 const long col = n0 + wn * WTN + js * SW + ec;
+                const bool col_ok = !RAGGED || col < g.N;
                 f32x4 bias4 = {0.f, 0.f, 0.f, 0.f};
-                if (g.bias) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
+                if (g.bias && col_ok) bias4 = *reinterpret_cast<const f32x4*>(g.bias + col);
 #pragma unroll
                 for (int jj = 0; jj < SF; ++jj)
 #pragma unroll
@@ -432,11 +460,13 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(const GemmArgs g)
                         f32x4 v = {c16[4 * gq], c16[4 * gq + 1], c16[4 * gq + 2], c16[4 * gq + 3]};
                         *reinterpret_cast<f32x4*>(stg + frag_row * EPI_STRIDE + (jj * 32 + gq * 8 + frag_half * 4) * 4) = v;
                     }
-                long idx = (m0 + wm * WTM + i * 32 + er) * g.N + col;     // advanced by RPP rows per pass
+                const long row_first = m0 + wm * WTM + i * 32 + er;
+                long idx = row_first * g.N + col;     // advanced by RPP rows per pass
 #pragma unroll
                 for (int p = 0; p < 32 / RPP; ++p, idx += row_step) {
                     const int rl = p * RPP + er;
                     const f32x4 v = *reinterpret_cast<const f32x4*>(stg + rl * EPI_STRIDE + ec * 4);
+                    if (RAGGED && !(col_ok && row_first + p * RPP < g.M)) continue;
                     f32x4 old = {0.f, 0.f, 0.f, 0.f};
                     if constexpr (OT == SP_F32) {
                         f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
@@ -836,9 +866,24 @@ static int choose_cfg(int dtype_in, long M, long N, long K, long batch = 1) {
     return smallest;
 }
 
-template <int DT, int OT, int BM, int BN, int WM, int WN, int NS, int NSA = NS>
+// Shapes no tile divides: the same tiled kernels with rows clamped in the loader, zeros for the missing part of the
+// last K-tile and a masked epilogue, provided N is a multiple of 4 (16-byte accesses to C and the bias).  Tile choice
+// as above, on tile counts rounded up.
+static int choose_cfg_ragged(int dtype_in, long M, long N, long K, long batch) {
+    (void)K;   // any K that passed validation (a multiple of 16 bytes)
+    if (N % 4 != 0) return -1;
+    const int cus = device_cu_count();
+    for (int i = 0; i < kNumCfgs; ++i) {
+        const TileCfg& c = kTileCfgs[i];
+        const long tiles = ((M + c.bm - 1) / c.bm) * ((N + c.bn - 1) / c.bn) * batch;
+        if (tiles * 5 >= (long)cus * 4) return i;
+    }
+    return kNumCfgs - 1;
+}
+
+template <int DT, int OT, int BM, int BN, int WM, int WN, int NS, int NSA = NS, bool RAGGED = false>
 static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
-    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS, NSA>;
+    auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS, NSA, RAGGED>;
     const int lds_bytes = (NSA * BM + NS * BN) * ROW_BYTES;
     static bool attr_set[64] = {false};
     int dev = 0;
@@ -863,6 +908,7 @@ static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
 // of the prologue delays the first tile: 2048 x 2048 x 512 bf16 9.7 -> 10.4 us).
 template <int DT, int OT, int BM, int BN, int WM, int WN>
 static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
+    if (g.ragged) return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2, 2, true>(g, stream);
     constexpr int DEEP = (128 * 1024) / ((BM + BN) * ROW_BYTES);
     if constexpr (BM == 256 && BN == 256 && DT != SP_F32) {
         // B is a single tile column: every A panel comes straight from HBM, once, and one 32 KiB stage of it in
@@ -904,7 +950,7 @@ template <int DT, int OT>
 static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
     switch (cfg) {
         case 0:
-            if (use_four_waves(DT, g.N, g.K)) return launch_four_waves<DT, OT>(g, stream);
+            if (!g.ragged && use_four_waves(DT, g.N, g.K)) return launch_four_waves<DT, OT>(g, stream);
             return launch_tiled<DT, OT, 256, 256, 2, 4>(g, stream);
         case 1: return launch_tiled<DT, OT, 128, 128, 2, 2>(g, stream);
         case 2: return launch_tiled<DT, OT, 64, 64, 2, 2>(g, stream);
@@ -952,13 +998,18 @@ extern "C" int sp_gemm_config(int dtype_in, int64_t M, int64_t N, int64_t K, int
     if (!tile_m || !tile_n || !tile_k || !threads) return fail(SP_ERR_NULL, "sp_gemm_config: NULL output");
     int rc = validate_gemm(dtype_in, SP_F32, M, N, K);
     if (rc != SP_OK) return rc;
-    const int cfg = choose_cfg(dtype_in, M, N, K);
+    int cfg = choose_cfg(dtype_in, M, N, K);
+    bool ragged = false;
+    if (cfg < 0) {
+        cfg = choose_cfg_ragged(dtype_in, M, N, K, 1);
+        ragged = cfg >= 0;
+    }
     if (cfg < 0) {
         *tile_m = 0; *tile_n = 0; *tile_k = 0; *threads = 256;
     } else {
         *tile_m = kTileCfgs[cfg].bm; *tile_n = kTileCfgs[cfg].bn; *tile_k = dtype_in == SP_F32 ? 32 : 64;
         *threads = kTileCfgs[cfg].wm * kTileCfgs[cfg].wn * 64;
-        if (cfg == 0 && use_four_waves(dtype_in, N, K)) *threads = 256;
+        if (cfg == 0 && !ragged && use_four_waves(dtype_in, N, K)) *threads = 256;
     }
     return SP_OK;
 }
@@ -986,9 +1037,13 @@ static int gemm_entry(const char* fn, int dtype_in, int dtype_out, const void* A
     g.k_rotate = 7;   // odd: coprime with the power-of-two K-tile counts of the usual shapes (measured: 1, 3, ..., 13 all within 1 %)
     g.batch = (int)batch;
     g.stride_a = stride_a * es_in; g.stride_b = stride_b * es_in; g.stride_c = stride_c * es_out;
+    if (cfg < 0 && !(flags & SP_GEMM_FORCE_GENERIC)) {
+        cfg = choose_cfg_ragged(dtype_in, M, N, K, batch);
+        g.ragged = cfg >= 0;
+    }
     if (cfg >= 0) {
-        g.tiles_m = (int)(M / kTileCfgs[cfg].bm);
-        g.tiles_n = (int)(N / kTileCfgs[cfg].bn);
+        g.tiles_m = (int)((M + kTileCfgs[cfg].bm - 1) / kTileCfgs[cfg].bm);
+        g.tiles_n = (int)((N + kTileCfgs[cfg].bn - 1) / kTileCfgs[cfg].bn);
     }
     hipStream_t s = (hipStream_t)stream;
     switch (dtype_in) {

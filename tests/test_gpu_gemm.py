@@ -81,6 +81,35 @@ def test_single_tile_column_a_ring(MM, dtype, k):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("m,n,k", [(1000, 1000, 1024), (1, 4, 64), (7, 12, 128), (63, 68, 64), (65, 60, 192), (300, 1000, 256),
+                                   (16384, 4, 256), (129, 132, 320), (4000, 260, 512), (2100, 2052, 128), (20000, 300, 64),
+                                   (1000, 1000, 1000), (64, 64, 40), (128, 128, 72), (100, 36, 8), (256, 256, 200),
+                                   (1024, 1024, 1000), (16384, 256, 32), (77, 4, 24)])
+def test_ragged_m_and_n(MM, dtype, m, n, k):
+    """M, N and K that no tile divides (N a multiple of 4, K of 16 bytes) run on the tiled kernels with clamped
+    loads, a zero-filled last K-tile and a masked epilogue: against the oracle, exactly on integer operands, with bias + ReLU and beta,
+    and without touching anything outside C (the output sits inside a larger buffer of sentinels)."""
+    announce("gemm ragged %s %dx%dx%d" % (dtype, m, n, k))
+    assert MM.matmul_config_tf32(False, True, m, n, k, TORCH[dtype])["m_tile"] > 0
+    rng = np.random.default_rng(m + 3 * n + 7 * k)
+    a, b = make(rng, m, n, k, dtype)
+    assert ogemm.rel_frobenius(run(MM, a, b, dtype), ogemm.gemm_abt(a, b)) < TOL[dtype]
+    ai = rng.integers(-3, 4, size=(m, k)).astype(np.float32)
+    bi = rng.integers(-3, 4, size=(n, k)).astype(np.float32)
+    want = ai.astype(np.float64) @ bi.astype(np.float64).T
+    bias = rng.integers(-5, 6, size=n).astype(np.float32)
+    c0 = rng.integers(-4, 5, size=(m, n)).astype(np.float32)
+    pad = 64
+    buf = torch.full((pad + m * n + pad,), -77.0, dtype=torch.float32, device="cuda")
+    c = buf[pad:pad + m * n].view(m, n)
+    c.copy_(dev(c0))
+    MM.matmul_abt(dev(ai, TORCH[dtype]), dev(bi, TORCH[dtype]), c=c, bias=dev(bias), relu=True, alpha=1.0, beta=2.0)
+    got = host(buf)
+    assert (got[:pad] == -77).all() and (got[pad + m * n:] == -77).all()
+    assert (got[pad:pad + m * n].reshape(m, n).astype(np.float64) == np.maximum(want + 2 * c0 + bias, 0)).all()
+
+
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 def test_integer_inputs_are_exact(MM, dtype):
     """Small integers are exact in every dtype and every partial sum fits f32: any indexing slip
     (transposed operand, wrong fragment row, dropped K-chunk) changes the integer result."""
