@@ -252,7 +252,29 @@ def main():
             wall, ev = time_launches(fn, K, W)
             return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "roofline": roofline_hbm(nbytes, ev), "seed": 9}
 
-        cases += [("mlp_leduc_16384", mlp_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
+        def graph_case():
+            # The same policy step through the reference's host surface: a layer graph (input -> matmul/relu x3 ->
+            # matmul -> masked softmax + sample, device Philox uniforms) run by layers.graph_run_host.  The head is 64
+            # wide with 3 valid columns because the reference's row ops need 16-byte rows.
+            q = layers.blocks_per_grid()
+            batch = 16384
+            g = layers.pipe(layers.input("input", (q, batch // q, 32), "f16"), layers.matmul((32, 256)), layers.relu,
+                            layers.matmul((256, 256)), layers.relu, layers.matmul((256, 256)), layers.relu,
+                            layers.matmul((256, 64)), layers.masked_softmax_and_discrete_sample(3))
+            m = layers.create_model(g)
+            rng = np.random.default_rng(10)
+            xin = layers.key_extract(m, "input")
+            xin.copy_(dev((rng.random(tuple(xin.shape)) < 0.2).astype(np.float32), torch.float16))
+            for _, t, _ in layers.extract_layers_(m, layers.weight_id()):
+                t.copy_(dev(olayers.weight_init(rng, t.shape[0], t.shape[1]), torch.float16))
+            fn = lambda: layers.graph_run_host(m)
+            wall, ev = time_launches(fn, max(K, 200), W)
+            fl = 2.0 * batch * (32 * 256 + 256 * 256 + 256 * 256 + 256 * 64)
+            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
+                    "roofline": roofline_mfma(fl, ev, "f16"), "seed": 10,
+                    "timing": "mean over back-to-back graph_run_host calls (two launches each: uniforms, fused MLP)"}
+
+        cases += [("mlp_leduc_16384", mlp_case), ("layers_graph_leduc_16384", graph_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
                   ("row_ops_65536x256_materialised", lambda: rows_case(True)),
                   ("map_relu_65536x256", lambda: elementwise_case("map_relu")),
                   ("reduce_sum_f32_65536x256", lambda: elementwise_case("reduce_sum")),

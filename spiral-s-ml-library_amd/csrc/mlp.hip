@@ -59,6 +59,7 @@ struct MlpArgs {
     int head;
     int mask_size;
     int k0, nout;        // dims[0] and dims[n_layers] once more, so that a kernel needs no dependent load for them
+    int out_stride;      // floats between two rows of policy / logits (= dims[n_layers]; nout may be smaller, see sp_mlp_forward)
 };
 
 // max(x, 0) and rounding of two f32 values to the 16-bit storage type, packed into one register
@@ -97,8 +98,11 @@ struct HeadOut {
     int* action;
     float* logits;
     int head;
+    int stride;   // floats between two rows of policy / logits; columns N .. stride - 1 of policy are written as zeros
 };
-__device__ __forceinline__ HeadOut head_out(const MlpArgs& a) { return HeadOut{a.policy, a.action, a.logits, a.head}; }
+__device__ __forceinline__ HeadOut head_out(const MlpArgs& a) {
+    return HeadOut{a.policy, a.action, a.logits, a.head, a.out_stride};
+}
 
 template <int MAXN>
 __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, long row, int N, int limit, float u) {
@@ -108,7 +112,7 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
     if (o.logits != nullptr) {
 #pragma unroll
         for (int n = 0; n < MAXN; ++n)
-            if (n < N) o.logits[row * N + n] = p[n];
+            if (n < N) o.logits[row * o.stride + n] = p[n];
     }
     // exp on the hardware exp2 unit and one hardware reciprocal (1 ulp) per normalisation: a 16-lane
     // serial head is otherwise a visible part of a forward pass that takes a few microseconds
@@ -143,7 +147,13 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
     }
 #pragma unroll
     for (int n = 0; n < MAXN; ++n)
-        if (n < N) o.policy[row * N + n] = p[n];
+        if (n < N) o.policy[row * o.stride + n] = p[n];
+    if (o.stride > N) {   // a masked head computed for its valid columns only: the rest of the row is exact zeros
+        float* tail = o.policy + row * o.stride;
+        int c = N;
+        for (; c < o.stride && ((c & 3) != 0 || (o.stride & 3) != 0); ++c) tail[c] = 0.f;
+        for (; c + 4 <= o.stride; c += 4) *reinterpret_cast<float4*>(tail + c) = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     if (o.action != nullptr) {
         float run = 0.f, m = -__builtin_inff();
         float cdf[MAXN];
@@ -1136,6 +1146,7 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     if (rc != SP_OK) return rc;
     a.x = x; a.n_layers = n_layers; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.nout = dims[n_layers];
+    a.out_stride = dims[n_layers];
     // 4 waves (64 rows) per workgroup while such workgroups fit the compute units in one round: every
     // wave reads all weights from LDS, so 8 waves on a unit are LDS-bandwidth bound (2048 cycles per
     // 32 KiB chunk) where 4 are not; beyond one round, 8 waves (128 rows) halve the rounds
@@ -1144,12 +1155,20 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     const int nw = wide ? 8 : 4;
     bool h256 = n_layers >= 2;   // all hidden layers 256 wide: the lean kernel
     for (int i = 1; i < n_layers; ++i) h256 = h256 && dims[i] == 256;
+    // A masked head gives probability zero to the columns past the mask whatever their logits are: when the logits
+    // themselves are not asked for, the last layer is computed for the valid columns only (the first rows of its
+    // weight matrix) and the head fills the rest of each policy row with zeros.  A 64-wide layer with 3 valid
+    // columns, the shape the reference's 16-byte row primitives force on a 3-action game, then runs on the
+    // narrow-head kernels.
+    if (h256 && head != SP_HEAD_NONE && logits_out == nullptr && mask_size > 0 && mask_size <= 16 &&
+        mask_size < dims[n_layers])
+        a.nout = mask_size;
     const void* kernel;
     int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
     int rows_per_block = nw * 16;
     int threads = nw * 64;
     // at most one 64-row workgroup per compute unit and a narrow head: hidden layers split by output features
-    const bool split = h256 && n_layers >= 3 && !wide && dims[n_layers] <= 16;
+    const bool split = h256 && n_layers >= 3 && !wide && a.nout <= 16;
     if (split) {
         const int ks0 = dims[0] <= 32 ? 1 : dims[0] <= 64 ? 2 : 8;
         kernel = pick_split_kernel(dtype, ks0);

@@ -122,3 +122,34 @@ def test_bias_extension(LY):
     biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
     biases[1] = None
     check(LY, x, ws, u, "bf16", biases=biases)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("batch,dims,head,mask", [(16384, [32, 256, 256, 256, 64], "softmax", 3),
+                                                  (1000, [128, 256, 256, 64], "regret_matching", 3),
+                                                  (333, [32, 256, 256, 256, 64], "softmax_regret_matching", 11),
+                                                  (40000, [32, 256, 256, 32], "softmax", 16),
+                                                  (257, [64, 256, 256, 6], "softmax", 5)])
+def test_masked_head_without_logits(LY, dtype, batch, dims, head, mask):
+    """Without the logits output a masked head is computed for its valid columns only and the rest of every policy
+    row is written as zeros (a 64-wide layer with 3 valid columns is the reference's shape for a 3-action game).
+    The policy must match the oracle and the run that does write the logits, the masked columns must be exact zeros
+    inside a buffer of sentinels, and the action must be the one the kernel's own policy and the uniforms give."""
+    announce("mlp masked head, no logits: %s %s batch=%d mask=%d %s" % (dims, head, batch, mask, dtype))
+    rng = np.random.default_rng(batch + mask)
+    x, ws, u = make_problem(rng, batch, dims, dtype)
+    t = TORCH[dtype]
+    xd, wd, ud = dev(x, t), [dev(w, t) for w in ws], dev(u)
+    n = dims[-1]
+    buf = torch.full((64 + batch * n + 64,), -9.0, dtype=torch.float32, device="cuda")
+    policy_t = buf[64:64 + batch * n].view(batch, n)
+    action_t = torch.full((batch,), -1, dtype=torch.int32, device="cuda")
+    LY.mlp_forward(xd, wd, None, head, ud, mask, False, policy_out=policy_t, action_out=action_t)
+    raw = host(buf)
+    assert (raw[:64] == -9).all() and (raw[-64:] == -9).all()
+    policy, action = raw[64:-64].reshape(batch, n), host(action_t)
+    full_p, full_a, _ = LY.mlp_forward(xd, wd, None, head, ud, mask, True)
+    want_p, _, _ = olayers.mlp_forward(x, ws, None, HEAD_CODE[head], u, dtype, mask)
+    assert (policy[:, mask:] == 0).all() and np.abs(policy.sum(axis=1) - 1).max() < 1e-5
+    assert ogemm.rel_frobenius(policy, want_p) < 2e-4 and ogemm.rel_frobenius(policy, host(full_p)) < 2e-4
+    assert (action == orow.discrete_sampling(policy, u)).all() and (action < mask).all() and (action >= 0).all()
