@@ -272,7 +272,8 @@ def main():
             fl = 2.0 * batch * (32 * 256 + 256 * 256 + 256 * 256 + 256 * 64)
             return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
                     "roofline": roofline_mfma(fl, ev, "f16"), "seed": 10,
-                    "timing": "mean over back-to-back graph_run_host calls (two launches each: uniforms, fused MLP)"}
+                    "timing": "mean over back-to-back graph_run_host calls (one fused-MLP launch each; the run's Philox "
+                              "uniforms depend on (model, seed) only and are drawn when the plan is built)"}
 
         cases += [("mlp_leduc_16384", mlp_case), ("layers_graph_leduc_16384", graph_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
                   ("row_ops_65536x256_materialised", lambda: rows_case(True)),

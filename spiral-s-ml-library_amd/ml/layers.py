@@ -621,10 +621,12 @@ def _build_fused_run(model, plan, ls):
     rows = q * w
     keep = (x, ws, probs, action, u, policy, act)   # the views stay alive as long as the closure does
 
+    # A run restarts the generator from the same seed (ml/layers.spi:339-344), so the uniforms of a (model, seed)
+    # pair are the same in every run: they are drawn once, here.
+    check(lib.sp_philox_uniforms(C.byref(rng), args[6], rows, cols, stream_ptr()))
+
     def run():
-        stream = stream_ptr()
-        check(lib.sp_philox_uniforms(C.byref(rng), args[6], rows, cols, stream))
-        check(lib.sp_mlp_forward(*args, stream))
+        check(lib.sp_mlp_forward(*args, stream_ptr()))
         return keep
 
     return run
