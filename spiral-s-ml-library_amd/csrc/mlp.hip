@@ -105,7 +105,8 @@ __device__ __forceinline__ HeadOut head_out(const MlpArgs& a) {
 }
 
 template <int MAXN>
-__device__ __forceinline__ void head_row(const HeadOut& o, const float* src, long row, int N, int limit, float u) {
+__device__ __forceinline__ void head_row(const HeadOut& o, const float* src, long row, int N, int limit, float u,
+                                         int fill_end = 1 << 30) {
     float p[MAXN];
 #pragma unroll
     for (int n = 0; n < MAXN; ++n) p[n] = n < N ? src[n] : 0.f;
@@ -149,10 +150,11 @@ __device__ __forceinline__ void head_row(const HeadOut& o, const float* src, lon
     for (int n = 0; n < MAXN; ++n)
         if (n < N) o.policy[row * o.stride + n] = p[n];
     if (o.stride > N) {   // a masked head computed for its valid columns only: the rest of the row is exact zeros
-        float* tail = o.policy + row * o.stride;
+        float* tail = o.policy + row * o.stride;   // (up to fill_end: the caller may fill the rest with whole waves)
+        const int end = o.stride < fill_end ? o.stride : fill_end;
         int c = N;
-        for (; c < o.stride && ((c & 3) != 0 || (o.stride & 3) != 0); ++c) tail[c] = 0.f;
-        for (; c + 4 <= o.stride; c += 4) *reinterpret_cast<float4*>(tail + c) = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (; c < end && ((c & 3) != 0 || (o.stride & 3) != 0); ++c) tail[c] = 0.f;
+        for (; c + 4 <= end; c += 4) *reinterpret_cast<float4*>(tail + c) = make_float4(0.f, 0.f, 0.f, 0.f);
     }
     if (o.action != nullptr) {
         float run = 0.f, m = -__builtin_inff();
@@ -1058,6 +1060,20 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
     const __attribute__((address_space(1))) float* bias =
         (const __attribute__((address_space(1))) float*)(unsigned long long)table_ptr(tab_b, NL - 1);
     const int limit = mask_size > 0 ? mask_size : NOUT;
+    // A masked head that was computed for its valid columns only: the wave's 16 policy rows are one contiguous
+    // block, and whole waves write its zeros (16 bytes per lane) instead of 16 lanes writing a row each.
+    int fill_end = 1 << 30;
+    if (out.stride > NOUT && (out.stride & 3) == 0) {
+        const int s4 = out.stride >> 2, c0 = (NOUT + 3) >> 2;    // float4 groups per row; the first one that is all zeros
+        fill_end = 4 * c0;
+        const long first_row = row0 + wave * 16;
+        float* block = out.policy + first_row * out.stride;
+        for (int idx = lane; idx < 16 * s4; idx += 64) {
+            const int r = idx / s4, c = idx - r * s4;
+            if (c >= c0 && first_row + r < batch)
+                *reinterpret_cast<float4*>(block + (long)r * out.stride + 4 * c) = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     if (NOUT <= 4) {
         // lane (j, q = 0) holds outputs 0..3 of batch row j; those are lanes 0..15 of the wave
         float p[4];
@@ -1066,7 +1082,7 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
             p[n] = d[n];
             if (bias != nullptr && n < NOUT) p[n] += bias[n];
         }
-        if (head_ok) head_row<4>(out, p, head_row_idx, NOUT, limit, u_row);
+        if (head_ok) head_row<4>(out, p, head_row_idx, NOUT, limit, u_row, fill_end);
     } else {
         // every chunk of this wave's ring has been consumed: its first stage stages the 16 x NOUT outputs
         float* head_rows = reinterpret_cast<float*>(lds + SPLIT_ACT_BYTES + wave * SPLIT_RING_BYTES);
@@ -1077,7 +1093,7 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
                 if (4 * q + r < NOUT) v[r] += bias[4 * q + r];
         }
         *reinterpret_cast<f32x4*>(head_rows + j * 16 + 4 * q) = v;
-        if (head_ok) head_row<16>(out, head_rows + lane * 16, head_row_idx, NOUT, limit, u_row);
+        if (head_ok) head_row<16>(out, head_rows + lane * 16, head_row_idx, NOUT, limit, u_row, fill_end);
     }
 }
 

@@ -820,21 +820,32 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
     (ml/layers.spi:336-344).  Uniforms come from the reference's per-thread Philox streams.  A loop over
     one key that only indexes leading dimensions runs as a single batched pass with the same results
     (`batched=False` keeps the member-by-member loop)."""
-    ls = create_layer_state(seed)
-    sizes = sizes or {}
     if fuse and not sizes:
         # The plan of a model does not change between runs: the tensors are views of its arenas and the
-        # generator restarts with every run.  It is built once per (model, seed); a call then costs two
-        # C-ABI calls instead of a walk over the graph (which took several times as long as the kernels).
-        cache = model.__dict__.setdefault("_fused_runs", {})
-        key = (seed,) + tuple(d["array"].data_ptr() for d in model.data)
-        run = cache.get(key)
-        if run is None:
+        # generator restarts with every run.  It is built once per (model, seed); a call then costs one
+        # C-ABI call instead of a walk over the graph (which took several times as long as the kernel).
+        cache = model.__dict__.get("_fused_runs")
+        if cache is None:
+            cache = model.__dict__["_fused_runs"] = {}
+        entry = cache.get(seed)
+        if entry is not None:
+            arenas, run = entry
+            data = model.data
+            if arenas[0] is data[0]["array"] and arenas[1] is data[1]["array"] and arenas[2] is data[2]["array"]:
+                if run:
+                    run()
+                    return
+            else:
+                entry = None    # the model was given other arenas: plan again
+        if entry is None:
             plan = _fused_plan(model)
-            run = cache[key] = _build_fused_run(model, plan, ls) if plan is not None else False
-        if run:
-            run()
-            return
+            run = _build_fused_run(model, plan, create_layer_state(seed)) if plan is not None else False
+            cache[seed] = (tuple(d["array"] for d in model.data), run)
+            if run:
+                run()
+                return
+    ls = create_layer_state(seed)
+    sizes = sizes or {}
     key = _batchable_key(model, sizes) if batched and sizes else None
     if key is not None and sizes[key] > 1:
         _graph_run_batched(model, key, sizes[key], ls)
