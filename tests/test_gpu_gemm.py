@@ -109,6 +109,29 @@ def test_ragged_m_and_n(MM, dtype, m, n, k):
     assert (got[pad:pad + m * n].reshape(m, n).astype(np.float64) == np.maximum(want + 2 * c0 + bias, 0)).all()
 
 
+def test_random_small_shapes_are_exact(MM):
+    """120 seeded shapes around the tile boundaries (M, N up to 330, K up to 45 chunks), all three dtypes, integer
+    operands: the tiled kernels' masking of M, N and K must give the exact product, with and without bias + ReLU."""
+    announce("gemm random small shapes")
+    rng = np.random.default_rng(2024)
+    edges = np.array([1, 2, 7, 8, 9, 63, 64, 65, 127, 128, 129, 255, 256, 257, 300, 330])
+    for case in range(120):
+        dtype = ("f32", "f16", "bf16")[case % 3]
+        per = 4 if dtype == "f32" else 8
+        m = int(rng.choice(edges)) if case % 2 else int(rng.integers(1, 331))
+        n = 4 * int(rng.integers(1, 84))
+        k = per * int(rng.integers(1, 46))
+        ai = rng.integers(-3, 4, size=(m, k)).astype(np.float32)
+        bi = rng.integers(-3, 4, size=(n, k)).astype(np.float32)
+        want = ai.astype(np.float64) @ bi.astype(np.float64).T
+        got = run(MM, ai, bi, dtype)
+        assert (got.astype(np.float64) == want).all(), (dtype, m, n, k)
+        if case % 4 == 0:
+            bias = rng.integers(-5, 6, size=n).astype(np.float32)
+            got = host(MM.matmul_abt(dev(ai, TORCH[dtype]), dev(bi, TORCH[dtype]), bias=dev(bias), relu=True))
+            assert (got.astype(np.float64) == np.maximum(want + bias, 0)).all(), (dtype, m, n, k, "bias+relu")
+
+
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 def test_integer_inputs_are_exact(MM, dtype):
     """Small integers are exact in every dtype and every partial sum fits f32: any indexing slip
