@@ -84,7 +84,64 @@ def load(path=LIB_PATH):
     return lib
 
 
-lib = load()
+# Entry points that launch work; their last argument is the stream.
+LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_row_map_f32", "sp_row_map_i32",
+                      "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_update_mask",
+                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_transpose_inner_b32", "sp_mlp_forward"))
+
+
+class Tape:
+    """The launches of one pass over a fixed set of tensors, recorded while they ran and replayable with a fresh stream
+    argument.  `keep` holds every tensor whose address went into a call, so temporaries the host functions allocated
+    stay alive as long as the tape does."""
+
+    def __init__(self):
+        self.calls, self.keep = [], []
+
+    def replay(self):
+        stream = stream_ptr()
+        for fn, args in self.calls:
+            rc = fn(*args, stream)
+            if rc != 0:
+                check(rc)
+
+
+_tape = None
+
+
+def start_tape():
+    """Every launch through `lib` from now until stop_tape() is also recorded."""
+    global _tape
+    _tape = Tape()
+    return _tape
+
+
+def stop_tape():
+    global _tape
+    _tape = None
+
+
+class _Library:
+    """The C-ABI library; launches pass through a thin wrapper that feeds the active tape, if any."""
+
+    def __init__(self, cdll):
+        self._cdll = cdll
+
+    def __getattr__(self, name):
+        fn = getattr(self._cdll, name)
+        if name in LAUNCHES:
+            raw = fn
+
+            def fn(*args):
+                rc = raw(*args)
+                if _tape is not None and rc == 0:
+                    _tape.calls.append((raw, args[:-1]))
+                return rc
+        setattr(self, name, fn)     # looked up once
+        return fn
+
+
+lib = _Library(load())
 
 
 def check(rc):
@@ -118,6 +175,8 @@ def ptr(t, dtype=None, name="tensor"):
         raise ValueError("%s must be contiguous (row-major, innermost stride 1)" % name)
     if dtype is not None and t.dtype != dtype:
         raise TypeError("%s must have dtype %s, got %s" % (name, dtype, t.dtype))
+    if _tape is not None:
+        _tape.keep.append(t)
     return C.c_void_p(t.data_ptr())
 
 

@@ -435,11 +435,22 @@ def graph_extract_(layer_state, model, indices):
     """ml/layers.spi:181-252.  With a layer state the nodes are computed on the way; without one the
     tensors are only looked up."""
     data = model.data
+    # The tensors of a node are views of the arenas: they are built once per model and arena set (building them on
+    # every run cost more host time than the kernels of a small graph take).
+    arenas = tuple(x["array"] for x in data)
+    cached = model.__dict__.get("_node_views")
+    if cached is None or len(cached[0]) != len(arenas) or any(a is not b for a, b in zip(cached[0], arenas)):
+        cached = model.__dict__["_node_views"] = (arenas, {})
+    views = cached[1]
 
     def extract_current(node):
+        v = views.get(node)
+        if v is not None:
+            return v
         for x in data:
             if node in x["partition"]:
-                return _from_offsets(x["array"], x["partition"][node])
+                v = views[node] = _from_offsets(x["array"], x["partition"][node])
+                return v
         raise KeyError("Cannot find the offset in the dictionaries for node %r." % (node,))
 
     def try_out(node):
@@ -449,7 +460,14 @@ def graph_extract_(layer_state, model, indices):
         if isinstance(graph, BlockMap):
             out = try_out(graph)
             if layer_state is not None:
-                _prim.map(graph.f, loop(graph.a), out)
+                inner = graph.a
+                if graph.f == "relu" and isinstance(inner, BlockMatmul) and out.dtype == extract_current(inner).dtype:
+                    # relu of a product: the GEMM's epilogue applies it and writes the map's tensor directly (one
+                    # launch and one pass over the activations less; the product's own tensor is not written)
+                    a, b = loop(inner.a), loop(inner.b)
+                    _matmul.matmul_abt(_flat(a), b, c=_flat(out), alpha=1.0, beta=0.0, relu=True)
+                else:
+                    _prim.map(graph.f, loop(inner), out)
             return out
         if isinstance(graph, BlockRowMap):
             out = try_out(graph)
@@ -844,8 +862,26 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
             if run:
                 run()
                 return
+    if not sizes:
+        # Node by node: what a run launches depends on the graph, the arenas and the seed only (every sampling node
+        # draws from a generator that restarts with the run), so the first run is recorded and later runs replay
+        # its launches; walking the graph took longer than the kernels of a small graph.
+        tapes = model.__dict__.get("_tapes")
+        if tapes is None:
+            tapes = model.__dict__["_tapes"] = {}
+        entry = tapes.get((seed, fuse))
+        data = model.data
+        if entry is not None and len(entry[0]) == len(data) and all(a is d["array"] for a, d in zip(entry[0], data)):
+            entry[1].replay()
+            return
+        tape = _lib.start_tape()
+        try:
+            graph_run_device(model, create_layer_state(seed), {})
+        finally:
+            _lib.stop_tape()
+        tapes[(seed, fuse)] = (tuple(d["array"] for d in data), tape)
+        return
     ls = create_layer_state(seed)
-    sizes = sizes or {}
     key = _batchable_key(model, sizes) if batched and sizes else None
     if key is not None and sizes[key] > 1:
         _graph_run_batched(model, key, sizes[key], ls)
