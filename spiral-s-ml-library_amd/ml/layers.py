@@ -862,25 +862,30 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
             if run:
                 run()
                 return
-    if not sizes:
-        # Node by node: what a run launches depends on the graph, the arenas and the seed only (every sampling node
-        # draws from a generator that restarts with the run), so the first run is recorded and later runs replay
-        # its launches; walking the graph took longer than the kernels of a small graph.
-        tapes = model.__dict__.get("_tapes")
-        if tapes is None:
-            tapes = model.__dict__["_tapes"] = {}
-        entry = tapes.get((seed, fuse))
-        data = model.data
-        if entry is not None and len(entry[0]) == len(data) and all(a is d["array"] for a, d in zip(entry[0], data)):
-            entry[1].replay()
-            return
-        tape = _lib.start_tape()
-        try:
-            graph_run_device(model, create_layer_state(seed), {})
-        finally:
-            _lib.stop_tape()
-        tapes[(seed, fuse)] = (tuple(d["array"] for d in data), tape)
+    sizes = sizes or {}
+    # What a run launches depends on the graph, the arenas, the key sizes and the seed only (every sampling node draws
+    # from a generator that restarts with the run), so the first run is recorded and later runs replay its launches;
+    # walking the graph took longer than the kernels of a small graph.
+    tapes = model.__dict__.get("_tapes")
+    if tapes is None:
+        tapes = model.__dict__["_tapes"] = {}
+    tape_key = (seed, fuse, batched, tuple(sorted(sizes.items())))
+    entry = tapes.get(tape_key)
+    data = model.data
+    if entry is not None and len(entry[0]) == len(data) and all(a is d["array"] for a, d in zip(entry[0], data)):
+        entry[1].replay()
         return
+    tape = _lib.start_tape()
+    try:
+        _graph_run_walk(model, sizes, seed, batched)
+    finally:
+        _lib.stop_tape()
+    tapes[tape_key] = (tuple(d["array"] for d in data), tape)
+
+
+def _graph_run_walk(model, sizes, seed, batched):
+    """One run by walking the graph: a single batched pass over one key where that is possible, else every
+    combination of the key indices in turn."""
     ls = create_layer_state(seed)
     key = _batchable_key(model, sizes) if batched and sizes else None
     if key is not None and sizes[key] > 1:

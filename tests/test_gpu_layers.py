@@ -185,3 +185,60 @@ def test_main_body_writes_the_reference_files(L, tmp_path):
     t5 = open(os.path.join(root, "test5", "layers.txt")).read()
     idx = np.array([int(v) for v in t5.replace("[", " ").replace("]", " ").replace(";", " ").split()])
     assert idx.size == 4 * Q * 64 and idx.min() >= 0 and idx.max() <= 10
+
+
+@pytest.mark.parametrize("kind", ["nodes_f32", "fused_f16", "ensemble", "ensemble_loop"])
+def test_replayed_runs_see_new_inputs_and_weights(L, kind):
+    """graph_run_host records what its first run of a model launches and replays that afterwards.  A replay must read
+    the tensors as they are NOW: inputs and weights are rewritten in place between runs, and every run is compared
+    with the oracle and with the first (recording) run of a fresh model that holds the same values."""
+    announce("layers replay " + kind)
+    ensemble = 3
+
+    def build():
+        if kind == "fused_f16":
+            g = L.pipe(L.input("input", (Q, 64, 32), "f16"), L.matmul((32, 256)), L.relu, L.matmul((256, 256)), L.relu,
+                       L.matmul((256, 64)), L.masked_softmax_and_discrete_sample(5))
+        elif kind == "nodes_f32":
+            g = L.pipe(L.input("input", (Q, 64, 64)), L.matmul((64, 128)), L.relu, L.matmul((128, 64)), L.ln_l2, L.relu,
+                       L.matmul((64, 64)), L.softmax_and_discrete_sample)
+        else:
+            out = L.pair(L.apply("ensemble", L.input("output_probs", (ensemble, Q, 64, 64))),
+                         L.apply("ensemble", L.input("output_indices", (ensemble, Q, 64), "int")))
+            x = L.pipe(L.input("input", (Q, 64, 64)), L.matmul_ensemble((ensemble, 64, 64)), L.relu,
+                       L.matmul_ensemble((ensemble, 64, 64)))
+            g = L.softmax_and_discrete_sample_(out, x)
+        return L.create_model(g)
+
+    sizes = {"ensemble": ensemble} if kind.startswith("ensemble") else {}
+    kw = {"batched": False} if kind == "ensemble_loop" else {}
+
+    def tensors(m):
+        ws = L.key_extract_list(m, "weights") if sizes else [t for _, t, _ in L.extract_layers_(m, L.weight_id())]
+        return [L.key_extract(m, "input")] + list(ws)
+
+    def outputs(m):
+        if sizes:
+            return host(L.key_extract(m, "output_probs")), host(L.key_extract(m, "output_indices"))
+        return tuple(host(t) for t in L.graph_extract(m, {}))
+
+    m = build()
+    previous = None
+    for round_ in range(3):
+        rng = np.random.default_rng(100 + round_)
+        values = [(rng.standard_normal(tuple(t.shape)) * (1.0 if i == 0 else 0.1)).astype(np.float32)
+                  for i, t in enumerate(tensors(m))]
+        for t, v in zip(tensors(m), values):
+            t.copy_(torch.from_numpy(v).to(t.dtype))
+        L.graph_run_host(m, sizes, **kw)          # round 0 records, rounds 1 and 2 replay
+        got = outputs(m)
+        fresh = build()
+        for t, v in zip(tensors(fresh), values):
+            t.copy_(torch.from_numpy(v).to(t.dtype))
+        L.graph_run_host(fresh, sizes, **kw)
+        want = outputs(fresh)
+        assert (got[0] == want[0]).all() and (got[1] == want[1]).all()
+        assert np.abs(got[0].reshape(-1, got[0].shape[-1]).sum(axis=1) - 1).max() < 1e-4
+        if previous is not None:
+            assert not (got[0] == previous).all()
+        previous = got[0]
