@@ -564,8 +564,12 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(const GemmArgs g) {
         for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
             for (int t = 0; t < 4; ++t) {
-                va[st][ks][t] = st * STAGE_BYTES + lds_offset(wm * 128 + 16 * t + fi, 4 * ks + fq);
-                vb[st][ks][t] = st * STAGE_BYTES + BM * ROW_BYTES + lds_offset(wn * 128 + 16 * t + fi, 4 * ks + fq);
+                // Which 16-byte chunk of the K-tile lane group fq multiplies in k-step ks is free as long as A and B
+                // agree.  With 4 * ks + fq (lanes l and l + 32 two chunks apart) half of the LDS cycles of these reads
+                // were bank conflicts (SQ_LDS_BANK_CONFLICT 8.5 M per 4096^3 launch); with 2 * fq + ks there are none.
+                const int kc = 2 * fq + ks;
+                va[st][ks][t] = st * STAGE_BYTES + lds_offset(wm * 128 + 16 * t + fi, kc);
+                vb[st][ks][t] = st * STAGE_BYTES + BM * ROW_BYTES + lds_offset(wn * 128 + 16 * t + fi, kc);
                 // opaque to the compiler, or it keeps one of them and re-derives the others inside the loop
                 asm volatile("" : "+v"(va[st][ks][t]), "+v"(vb[st][ks][t]));
             }
