@@ -380,11 +380,31 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 
         float p[C][4];
         float s = 0.f;
+        if (a.op == SP_ROW_MASKED_SOFTMAX) {
+            // columns past the mask enter as -inf (their exponential is an exact 0) and the shift is the max of
+            // the columns inside the mask, as in row_kernel
+            float m = NEG_INF;
 #pragma unroll
-        for (int c = 0; c < C; ++c) {
+            for (int c = 0; c < C; ++c)
 #pragma unroll
-            for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(v[c][k] - bv);
-            s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+                for (int k = 0; k < 4; ++k) {
+                    p[c][k] = (c * 4 * T + 4 * l + k < a.mask_size) ? v[c][k] : NEG_INF;
+                    m = vmax(m, p[c][k]);
+                }
+            m = group_max<T>(m);
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(p[c][k] - m);
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
+        } else {
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(v[c][k] - bv);
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
         }
         s = group_reduce<T>(s, [](float x, float y) { return x + y; });
         const float inv = 1.f / s;
@@ -849,8 +869,9 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
         rc = set_philox(a, philox, rows, cols, __func__);
         if (rc != SP_OK) return rc;
     }
-    // Plain softmax sampling is what the fused pipeline does (same operations, same order, same bits).
-    if (op == SP_ROW_SOFTMAX && prob_out == nullptr) return launch_row<true>(a, (hipStream_t)stream, __func__);
+    // Softmax sampling, masked or not, is what the fused pipeline does (same operations, same order, same bits).
+    if ((op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX) && prob_out == nullptr)
+        return launch_row<true>(a, (hipStream_t)stream, __func__);
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 

@@ -113,10 +113,17 @@ def test_fused_and_general_kernels_agree(P, rows, cols):
     for kw in (dict(u=u), dict(rng=P.philox())):
         if "rng" in kw and (256 % (cols // 4) != 0):
             continue   # the reference's generator needs threads_per_block to be a multiple of cols/4
+        # asking for the sampled column's probability keeps a call on the general kernel
         a = P.softmax_and_discrete_sampling(x, want_cdf=True, want_u=True, **kw)
-        b = P.masked_softmax_and_discrete_sampling(x, cols, want_cdf=True, want_u=True, **kw)
-        for fa, fb in zip(a, b):
+        b = P.masked_softmax_and_discrete_sampling(x, cols, want_cdf=True, want_u=True, want_prob=True, **kw)
+        for fa, fb in zip(a, b[:4]):
             assert torch.equal(fa, fb)
+        for size in sorted({1, 3, cols // 2 + 1, cols - 1} - {0}):
+            a = P.masked_softmax_and_discrete_sampling(x, size, want_cdf=True, want_u=True, **kw)
+            b = P.masked_softmax_and_discrete_sampling(x, size, want_cdf=True, want_u=True, want_prob=True, **kw)
+            for fa, fb in zip(a, b[:4]):
+                assert torch.equal(fa, fb)
+            assert (a[1] < size).all() and (a[0][:, size:] == 0).all()
     assert torch.equal(P.softmax(x), P.masked_softmax(x, cols))     # the map alone: fused kernel vs general kernel
 
 
