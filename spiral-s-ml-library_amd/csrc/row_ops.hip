@@ -398,6 +398,23 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(p[c][k] - m);
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
+        } else if (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING) {
+            // local_regret_matching (ml/primitives.spi:718-722, masked :761-780), operation for operation as in
+            // row_kernel: positive parts over their sum, the uniform distribution over the mask when that sum is 0
+            const int limit = a.mask_size;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = (c * 4 * T + 4 * l + k < limit) ? fmaxf(v[c][k], 0.f) : 0.f;
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
+            const float inv_len = 1.f / (float)limit;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    p[c][k] = (c * 4 * T + 4 * l + k < limit) ? (s != 0.f ? p[c][k] / s : inv_len) : 0.f;
         } else {
 #pragma unroll
             for (int c = 0; c < C; ++c) {
@@ -406,12 +423,14 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
         }
-        s = group_reduce<T>(s, [](float x, float y) { return x + y; });
-        const float inv = 1.f / s;
+        if (!(a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING)) {
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
+            const float inv = 1.f / s;
 #pragma unroll
-        for (int c = 0; c < C; ++c)
+            for (int c = 0; c < C; ++c)
 #pragma unroll
-            for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
+                for (int k = 0; k < 4; ++k) p[c][k] = p[c][k] * inv;
+        }
 
         // Results that are rows themselves leave as soon as they exist, so that neither the
         // probabilities' copy for the store nor the running sums stay in registers.
@@ -474,12 +493,23 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
             }
         }
 
+        // local_get_prob of the sampled column (ml/primitives.spi:824-830): one non-zero term, so the sum is exact
+        float got = 0.f;
+        if (a.prob_out != nullptr) {
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k)
+                    if (c * 4 * T + 4 * l + k == pick) got = p[c][k];
+            got = group_reduce<T>(got, [](float x, float y) { return x + y; });
+        }
         if (row_ok && l == 0) {
             if (a.rowmax != nullptr) a.rowmax[row] = bv;
             if (a.rowsum != nullptr) a.rowsum[row] = s;
             if (a.argmax != nullptr) a.argmax[row] = bi;
             if (a.sample != nullptr) a.sample[row] = pick;
             if (a.u_out != nullptr) a.u_out[row] = uu;
+            if (a.prob_out != nullptr) a.prob_out[row] = got;
         }
     };
 
@@ -869,9 +899,9 @@ extern "C" int sp_row_sample(int op, const float* x, const float* u, const sp_ph
         rc = set_philox(a, philox, rows, cols, __func__);
         if (rc != SP_OK) return rc;
     }
-    // Softmax sampling, masked or not, is what the fused pipeline does (same operations, same order, same bits).
-    if ((op == SP_ROW_SOFTMAX || op == SP_ROW_MASKED_SOFTMAX) && prob_out == nullptr)
-        return launch_row<true>(a, (hipStream_t)stream, __func__);
+    // Softmax and regret-matching sampling, masked or not, is what the fused pipeline does (same operations, same
+    // order, same bits as the general kernel).
+    if (op != SP_ROW_IDENTITY) return launch_row<true>(a, (hipStream_t)stream, __func__);
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 

@@ -206,7 +206,7 @@ def get_action(x, u=None, rng=None, op="identity", size=0):
     gather mapping (one row per thread).  Returns (prob, action_id)."""
     if u is None and rng is None:
         rng = philox(_lib.PHILOX_GATHER)
-    _, action, prob = _sample(_ROW_OPS[op], x, u, rng, mask_size=size, want_prob=True)
+    _, action, prob = _sample(_ROW_OPS[op], x, u, rng, mask_size=size, want_prob=True, want_probs=False)
     return prob, action
 
 

@@ -104,26 +104,37 @@ def test_transpose_shapes(P, shape):
 @pytest.mark.parametrize("rows,cols", [(1, 4), (5, 16), (130, 64), (257, 256), (33, 260), (1000, 1024), (7, 1000),
                                        (4099, 256)])
 def test_fused_and_general_kernels_agree(P, rows, cols):
-    """Plain softmax sampling runs on the fused kernel, a mask that covers every column on the general one:
-    probabilities, running sums, uniforms and samples must agree bit for bit, with given and with device uniforms."""
+    """The fused kernel (softmax and regret matching, masked or not, with sampling) against the general kernel (the
+    row map alone, then sampling from its output): probabilities, samples, running sums, uniforms and the sampled
+    column's probability must agree bit for bit, with given and with device uniforms."""
     announce("fused vs general %dx%d" % (rows, cols))
     rng = np.random.default_rng(rows * 1000 + cols)
     x = dev((rng.standard_normal((rows, cols), dtype=np.float32) * 2).astype(np.float32))
     u = dev((1 - rng.random(rows, dtype=np.float32)).astype(np.float32))
+    def general(op_map, t, size, kw):
+        """The same results from the general kernel: the row map on its own, then sampling from those probabilities."""
+        probs = op_map(t, size)
+        return (probs,) + tuple(P.discrete_sampling(probs, want_cdf=True, want_u=True, want_prob=True, **kw)[1:])
+
+    def same(got, want):
+        for fa, fb in zip(got, want):
+            assert torch.equal(fa, fb)
+
     for kw in (dict(u=u), dict(rng=P.philox())):
         if "rng" in kw and (256 % (cols // 4) != 0):
             continue   # the reference's generator needs threads_per_block to be a multiple of cols/4
-        # asking for the sampled column's probability keeps a call on the general kernel
-        a = P.softmax_and_discrete_sampling(x, want_cdf=True, want_u=True, **kw)
-        b = P.masked_softmax_and_discrete_sampling(x, cols, want_cdf=True, want_u=True, want_prob=True, **kw)
-        for fa, fb in zip(a, b[:4]):
-            assert torch.equal(fa, fb)
+        full = dict(want_cdf=True, want_u=True, want_prob=True, **kw)
+        same(P.softmax_and_discrete_sampling(x, **full), general(P.masked_softmax, x, cols, kw))
+        same(P.regret_matching_and_discrete_sampling(x, **full), general(P.masked_regret_matching, x, cols, kw))
         for size in sorted({1, 3, cols // 2 + 1, cols - 1} - {0}):
-            a = P.masked_softmax_and_discrete_sampling(x, size, want_cdf=True, want_u=True, **kw)
-            b = P.masked_softmax_and_discrete_sampling(x, size, want_cdf=True, want_u=True, want_prob=True, **kw)
-            for fa, fb in zip(a, b[:4]):
-                assert torch.equal(fa, fb)
-            assert (a[1] < size).all() and (a[0][:, size:] == 0).all()
+            got = P.masked_softmax_and_discrete_sampling(x, size, **full)
+            same(got, general(P.masked_softmax, x, size, kw))
+            assert (got[1] < size).all() and (got[0][:, size:] == 0).all()
+            same(P.masked_regret_matching_and_discrete_sampling(x, size, **full),
+                 general(P.masked_regret_matching, x, size, kw))
+        neg = x.clone()
+        neg[::3] = -neg[::3].abs()       # rows without a positive entry: the uniform branch of regret matching
+        same(P.regret_matching_and_discrete_sampling(neg, **full), general(P.masked_regret_matching, neg, cols, kw))
     assert torch.equal(P.softmax(x), P.masked_softmax(x, cols))     # the map alone: fused kernel vs general kernel
 
 
