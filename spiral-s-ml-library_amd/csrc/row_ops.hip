@@ -343,7 +343,9 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 // are computed by the same operations in the same order); what differs is the instruction count:
 // padding lanes hold -inf, whose exponential is 0, so no per-element validity tests remain, full
 // waves load and store without predicates, and the max reductions are single DPP instructions.
-template <int T, int C, bool MAT>
+// ANYOP = false: plain softmax only (sp_row_ops and the plain softmax ops), the code every other variant is measured
+// against; true: the op is read from the arguments (masked softmax, regret matching), at the price of a larger kernel.
+template <int T, int C, bool MAT, bool ANYOP>
 __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -380,7 +382,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 
         float p[C][4];
         float s = 0.f;
-        if (a.op == SP_ROW_MASKED_SOFTMAX) {
+        if (ANYOP && a.op == SP_ROW_MASKED_SOFTMAX) {
             // columns past the mask enter as -inf (their exponential is an exact 0) and the shift is the max of
             // the columns inside the mask, as in row_kernel
             float m = NEG_INF;
@@ -398,7 +400,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(p[c][k] - m);
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
-        } else if (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING) {
+        } else if (ANYOP && (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING)) {
             // local_regret_matching (ml/primitives.spi:718-722, masked :761-780), operation for operation as in
             // row_kernel: positive parts over their sum, the uniform distribution over the mask when that sum is 0
             const int limit = a.mask_size;
@@ -423,7 +425,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
         }
-        if (!(a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING)) {
+        if (!(ANYOP && (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING))) {
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
             const float inv = 1.f / s;
 #pragma unroll
@@ -554,16 +556,15 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 }
 
 // MAT = true: probabilities and/or running sums are written out.
-template <int T, int C>
-__global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(
-    const RowArgs a) {
-    row_softmax_body<T, C, true>(a);
+template <int T, int C, bool ANYOP = false>
+__global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const RowArgs a) {
+    row_softmax_body<T, C, true, ANYOP>(a);
 }
 
 // MAT = false: per-row results only; nothing of the row is written back.
-template <int T, int C>
+template <int T, int C, bool ANYOP = false>
 __global__ __launch_bounds__(ROW_THREADS) void row_softmax_scalars_kernel(const RowArgs a) {
-    row_softmax_body<T, C, false>(a);
+    row_softmax_body<T, C, false, ANYOP>(a);
 }
 
 // Integer rows: identity and exact scans (two's complement wrap-around).
@@ -772,11 +773,18 @@ static int launch_row(const RowArgs& args, hipStream_t stream, const char* fn) {
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
-        if (FUSED && (a.out != nullptr || a.cdf != nullptr))
-            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid),
+        const bool rows_out = a.out != nullptr || a.cdf != nullptr, any_op = a.op != SP_ROW_SOFTMAX;
+        if (FUSED && rows_out && !any_op)
+            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value, false>), dim3(grid),
                                dim3(ROW_THREADS), 0, stream, a);
-        else if (FUSED)   // per-row results only: nothing of the row itself is written back
-            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid),
+        else if (FUSED && rows_out)
+            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value, true>), dim3(grid),
+                               dim3(ROW_THREADS), 0, stream, a);
+        else if (FUSED && !any_op)   // per-row results only: nothing of the row itself is written back
+            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value, false>), dim3(grid),
+                               dim3(ROW_THREADS), 0, stream, a);
+        else if (FUSED)
+            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value, true>), dim3(grid),
                                dim3(ROW_THREADS), 0, stream, a);
         else
             hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
