@@ -224,13 +224,13 @@ def test_replayed_runs_see_new_inputs_and_weights(L, kind):
 
     m = build()
     previous = None
-    for round_ in range(3):
-        rng = np.random.default_rng(100 + round_)
+    for pass_ in range(3):
+        rng = np.random.default_rng(100 + pass_)
         values = [(rng.standard_normal(tuple(t.shape)) * (1.0 if i == 0 else 0.1)).astype(np.float32)
                   for i, t in enumerate(tensors(m))]
         for t, v in zip(tensors(m), values):
             t.copy_(torch.from_numpy(v).to(t.dtype))
-        L.graph_run_host(m, sizes, **kw)          # round 0 records, rounds 1 and 2 replay
+        L.graph_run_host(m, sizes, **kw)          # the first pass records, the second and third replay
         got = outputs(m)
         fresh = build()
         for t, v in zip(tensors(fresh), values):
