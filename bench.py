@@ -151,9 +151,19 @@ def main():
     cpu = None
     if not args.no_cpu and not args.only:
         t = best_of(lambda: np.matmul(a, b.T), 3)
-        cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s", "cores": len(os.sched_getaffinity(0)),
+        blas = {"vendor": None, "version": None, "threads": None}
+        try:   # which BLAS np.matmul ran on and with how many threads
+            from threadpoolctl import threadpool_info
+            pools = [p for p in threadpool_info() if p.get("user_api") == "blas"]
+            if pools:
+                blas = {"vendor": pools[0].get("internal_api"), "version": pools[0].get("version"),
+                        "threads": pools[0].get("num_threads")}
+        except Exception:   # informational only
+            pass
+        cpu = {"value": round(flops / t / 1e12, 4), "unit": "TFLOP/s",
+               "cores": blas["threads"] or len(os.sched_getaffinity(0)),
                "kind": "port", "sample": "full 4096^3 problem, np.matmul(A32, B32.T) in f32 on the bf16-rounded "
-               "inputs (all BLAS threads), 1 warm-up + best of 3",
+               "inputs, 1 warm-up + best of 3", "blas": blas, "cpus_allowed": len(os.sched_getaffinity(0)),
                "os_cpu_count": os.cpu_count()}
     del a, b
 
@@ -241,7 +251,7 @@ def main():
                 nbytes = 2 * x.nbytes
             elif kind == "reduce_sum":
                 from ml._lib import check, lib, ptr, stream_ptr
-                ws = torch.empty(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device="cuda")
+                ws = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device="cuda")
                 out = torch.empty(4, dtype=torch.float32, device="cuda")
                 fn = lambda: check(lib.sp_reduce_sum(0, ptr(xd), ptr(out), xd.numel(), ptr(ws), ws.numel(), stream_ptr()))
                 nbytes = x.nbytes + 4
@@ -300,16 +310,22 @@ def main():
             measured = json.load(f)
         if head["roofline"] is not None:
             head["roofline"]["traffic"] = measured["headline"]["traffic_bytes"]
+            head["roofline"]["traffic_measured_at"] = measured.get("measured_at")
         for name, res in extra.items():
             if name in measured and res.get("roofline") is not None:
                 res["roofline"]["traffic"] = measured[name]["traffic_bytes"]
     except (OSError, KeyError, ValueError):
         pass
 
+    # `value` and `ms_per_step` come from the same clock (wall time between two device syncs around the K
+    # launches): value = 2 * 4096^3 / ms_per_step.  `roofline.achieved` is the kernel's own rate, from HIP events
+    # on the launch stream (`event_ms_per_step`); the two differ by the host's share of a launch.
     line = {
         "metric": "GEMM TFLOP/s (% MFMA peak) at 4096^3 bf16; fused MLP fwd rows/sec",
-        "value": head["tflops"], "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
-        "ms_per_step": head["wall_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "value": None if head["wall_ms"] is None else round(flops / (head["wall_ms"] * 1e-3) / 1e12, 2),
+        "unit": "TFLOP/s", "n_gpus": 1, "steps": K, "warmup": W,
+        "ms_per_step": head["wall_ms"], "event_ms_per_step": head.get("ms"),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "C = A.B^T, M=N=K=4096, A/B bf16 row-major N(0,1)/sqrt(K) (seed 2), f32 accumulate, "
                                "f32 output", "tile": head["tile"]},

@@ -248,13 +248,14 @@ def get_prob(p, action):
 
 
 def binarize(x, modulo):
-    """`local_binarize` (ml/primitives.spi:817-821): bit j set iff x_j > 0, OR-ed, mod `modulo`.
+    """`local_binarize` (ml/primitives.spi:817-821): bit j set iff not (x_j <= 0) (so a NaN sets its bit), OR-ed,
+    mod `modulo`.
     The shift is the device's 32-bit shift, which gives 0 for a shift count of 32 or more (the
     source's own comment points at that difference from the CPU), so columns j >= 32 drop out.
     PARITY UNPINNED: the reference holds no output of this function."""
     x = _f32(x)
     j = np.arange(x.shape[-1], dtype=np.uint64)
-    bits = np.where((x > 0) & (j < 32), np.uint64(1) << (j % np.uint64(32)), np.uint64(0))
+    bits = np.where(~(x <= 0) & (j < 32), np.uint64(1) << (j % np.uint64(32)), np.uint64(0))
     return (np.bitwise_or.reduce(bits, axis=-1) & np.uint64(0xFFFFFFFF)) % np.uint64(modulo)
 
 

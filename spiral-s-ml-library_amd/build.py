@@ -19,7 +19,9 @@ LIB = os.path.join(HERE, "libspiral_mi355.so")
 SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"),
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
-         "-Wno-unknown-warning-option"]
+         "-Wno-unknown-warning-option",
+         # the DMA blocks name M0 as clobbered; the compiler notes that M0 is a reserved register, once per use
+         "-Wno-inline-asm"]
 
 
 def hipcc():

@@ -63,6 +63,23 @@ int device_cu_count() {
     return c->cus;
 }
 
+// The opt-in to more than 64 KiB of dynamic LDS is per kernel and device.  Each host thread remembers the
+// (kernel, device) pairs it has opted in (thread-local, so nothing is shared between threads; the HIP call
+// itself is thread safe and idempotent, a second thread merely repeats it once).
+int ensure_dynamic_lds(const void* kernel, int lds_bytes) {
+    struct Seen { const void* kernel; int device; };
+    static thread_local Seen seen[64];
+    static thread_local int n_seen = 0;
+    int dev = 0;
+    (void)hipGetDevice(&dev);
+    for (int i = 0; i < n_seen; ++i)
+        if (seen[i].kernel == kernel && seen[i].device == dev) return SP_OK;
+    hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes, hipGetErrorString(e));
+    if (n_seen < 64) seen[n_seen++] = Seen{kernel, dev};
+    return SP_OK;
+}
+
 struct KernelEntry {
     std::string name;
     const void* fn;

@@ -45,6 +45,8 @@ inline int check_launch(const char* what) {
 // The kernels are built for gfx950 only; refuse to launch on anything else instead of faulting.
 int require_gfx950(const char* what);
 int device_cu_count();
+// Opt `kernel` in to `lds_bytes` of dynamic LDS on the current device (once per host thread, kernel and device).
+int ensure_dynamic_lds(const void* kernel, int lds_bytes);
 // Name -> kernel registry behind sp_kernel_info().
 void register_kernel(const char* name, const void* fn, int threads);
 

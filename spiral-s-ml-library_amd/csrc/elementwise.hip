@@ -47,41 +47,65 @@ __device__ __forceinline__ T block_sum(T v, T* slots) {
     return r;  // valid in wave 0
 }
 
-// Per-block partial sums: 16-byte loads, four of them in flight per lane and four independent
-// running sums; the order of the additions depends only on n and the grid, so the result is the
-// same from run to run.
-template <typename T>
-__global__ __launch_bounds__(EW_THREADS) void reduce_partial_kernel(const T* __restrict__ x, T* __restrict__ partial, long n) {
+// Full-tensor sum in ONE launch.  Every block adds up its share (16-byte loads, U of them in flight per lane and U
+// independent running sums), writes its partial sum to `partial[blockIdx.x]` and takes a ticket from `counter`;
+// the block that draws the last ticket adds the partials in index order and writes the result.  Which block that
+// is changes from run to run, the order of the additions does not: the result depends on n and the grid only.
+// `counter` must be zero when the kernel starts; the last block leaves it at zero for the next launch.
+// The partials cross between the private L2 caches of the XCDs: the writer's device-scope fence writes them back
+// before its ticket is taken, and the last block's fence discards stale lines before it reads them.
+template <typename T, int U>
+__global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restrict__ x, T* __restrict__ out, long n,
+                                                                T* partial, unsigned* counter) {
     __shared__ T slots[EW_THREADS / WAVE];
+    __shared__ unsigned ticket;
     constexpr int V = 16 / sizeof(T);
     typedef T VT __attribute__((ext_vector_type(V)));
     const VT* xv = reinterpret_cast<const VT*>(x);
     const long nv = n / V;
     const long stride = (long)gridDim.x * EW_THREADS;
     const long tid = (long)blockIdx.x * EW_THREADS + threadIdx.x;
-    VT a0 = VT(0), a1 = VT(0), a2 = VT(0), a3 = VT(0);
-    long i = tid;
-    for (; i + 3 * stride < nv; i += 4 * stride) {
-        const VT v0 = xv[i], v1 = xv[i + stride], v2 = xv[i + 2 * stride], v3 = xv[i + 3 * stride];
-        a0 += v0; a1 += v1; a2 += v2; a3 += v3;
-    }
-    for (; i < nv; i += stride) a0 += xv[i];
-    const VT a = (a0 + a1) + (a2 + a3);
-    T acc = a[0];
+    VT a[U];
 #pragma unroll
-    for (int k = 1; k < V; ++k) acc += a[k];
+    for (int k = 0; k < U; ++k) a[k] = VT(0);
+    long i = tid;
+    for (; i + (U - 1) * stride < nv; i += U * stride) {
+        VT v[U];
+#pragma unroll
+        for (int k = 0; k < U; ++k) v[k] = xv[i + k * stride];
+#pragma unroll
+        for (int k = 0; k < U; ++k) a[k] += v[k];
+    }
+    for (; i < nv; i += stride) a[0] += xv[i];
+#pragma unroll
+    for (int d = 1; d < U; d <<= 1)
+#pragma unroll
+        for (int k = 0; k + d < U; k += 2 * d) a[k] += a[k + d];
+    T acc = a[0][0];
+#pragma unroll
+    for (int k = 1; k < V; ++k) acc += a[0][k];
     for (long j = nv * V + tid; j < n; j += stride) acc += x[j];   // the last n % V elements
     acc = block_sum(acc, slots);
-    if (threadIdx.x == 0) partial[blockIdx.x] = acc;
+    if (threadIdx.x == 0) {
+        partial[blockIdx.x] = acc;
+        __threadfence();
+        ticket = atomicAdd(counter, 1u);
+    }
+    __syncthreads();
+    if (ticket != gridDim.x - 1) return;
+    __threadfence();
+    T total = T(0);
+    for (unsigned b = threadIdx.x; b < gridDim.x; b += EW_THREADS) total += partial[b];
+    total = block_sum(total, slots);
+    if (threadIdx.x == 0) {
+        out[0] = total;
+        *counter = 0u;
+    }
 }
 
-template <typename T>
-__global__ __launch_bounds__(EW_THREADS) void reduce_final_kernel(const T* __restrict__ partial, T* __restrict__ out, int count) {
-    __shared__ T slots[EW_THREADS / WAVE];
-    T acc = T(0);
-    for (int i = threadIdx.x; i < count; i += EW_THREADS) acc += partial[i];
-    acc = block_sum(acc, slots);
-    if (threadIdx.x == 0) out[0] = acc;
+// Sets `count` 32-bit words to zero (a kernel rather than a memset so that callers may record it into a graph).
+__global__ __launch_bounds__(WAVE) void clear_words_kernel(unsigned* p, int count) {
+    for (int i = threadIdx.x; i < count; i += WAVE) p[i] = 0u;
 }
 
 // to[a][c][b] = from[a][b][c]; 64x64 tiles through LDS, padded by one word per row so that the
@@ -141,16 +165,28 @@ __global__ __launch_bounds__(EW_THREADS) void transpose_vec4_kernel(const unsign
     }
 }
 
+// Layout of a reduction's scratch memory: REDUCE_MAX_BLOCKS partial sums of 8 bytes, then the ticket counter.
+constexpr long REDUCE_COUNTER_OFFSET = (long)REDUCE_MAX_BLOCKS * 8;
+constexpr long REDUCE_SCRATCH_BYTES = REDUCE_COUNTER_OFFSET + 256;
+
 template <typename T>
-static int run_reduce(const void* x, void* out, int64_t n, void* workspace, hipStream_t stream) {
+static int run_reduce(const void* x, void* out, int64_t n, void* scratch_mem, hipStream_t stream) {
     long blocks = (n + EW_THREADS * 16 - 1) / (EW_THREADS * 16);   // >= 4 vectors of 16 bytes per lane
     if (blocks > REDUCE_MAX_BLOCKS) blocks = REDUCE_MAX_BLOCKS;
     if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL(reduce_partial_kernel<T>, dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x,
-                       (T*)workspace, (long)n);
-    hipLaunchKernelGGL(reduce_final_kernel<T>, dim3(1), dim3(EW_THREADS), 0, stream, (const T*)workspace, (T*)out,
-                       (int)blocks);
+    unsigned* counter = reinterpret_cast<unsigned*>((unsigned char*)scratch_mem + REDUCE_COUNTER_OFFSET);
+    hipLaunchKernelGGL((reduce_sum_kernel<T, 4>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x, (T*)out,
+                       (long)n, (T*)scratch_mem, counter);
     return check_launch("sp_reduce_sum");
+}
+
+static int run_reduce_dtype(int dtype, const void* x, void* out, int64_t n, void* scratch_mem, hipStream_t s) {
+    switch (dtype) {
+        case 0: return run_reduce<float>(x, out, n, scratch_mem, s);
+        case 1: return run_reduce<int>(x, out, n, scratch_mem, s);
+        case 2: return run_reduce<unsigned long long>(x, out, n, scratch_mem, s);
+    }
+    return fail(SP_ERR_DTYPE, "sp_reduce_sum: dtype must be 0 (f32), 1 (i32) or 2 (u64), got %d", dtype);
 }
 
 }  // namespace sp
@@ -180,7 +216,7 @@ extern "C" int sp_map_f32(int op, const float* x, float* out, int64_t n, void* s
     return check_launch(__func__);
 }
 
-extern "C" int64_t sp_reduce_workspace_bytes(void) { return (int64_t)REDUCE_MAX_BLOCKS * 8; }
+extern "C" int64_t sp_reduce_workspace_bytes(void) { return (int64_t)REDUCE_SCRATCH_BYTES; }
 
 extern "C" int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes,
                              void* stream) {
@@ -188,18 +224,13 @@ extern "C" int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, voi
     SP_REQUIRE_PTR(out);
     SP_REQUIRE_PTR(workspace);
     if (n <= 0) return fail(SP_ERR_SHAPE, "sp_reduce_sum: n must be positive");
+    if (dtype < 0 || dtype > 2) return fail(SP_ERR_DTYPE, "sp_reduce_sum: dtype must be 0 (f32), 1 (i32) or 2 (u64), got %d", dtype);
     if (workspace_bytes < sp_reduce_workspace_bytes())
         return fail(SP_ERR_ARG, "sp_reduce_sum: workspace must hold %lld bytes, got %lld",
                     (long long)sp_reduce_workspace_bytes(), (long long)workspace_bytes);
     int rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
-    hipStream_t s = (hipStream_t)stream;
-    switch (dtype) {
-        case 0: return run_reduce<float>(x, out, n, workspace, s);
-        case 1: return run_reduce<int>(x, out, n, workspace, s);
-        case 2: return run_reduce<unsigned long long>(x, out, n, workspace, s);
-    }
-    return fail(SP_ERR_DTYPE, "sp_reduce_sum: dtype must be 0 (f32), 1 (i32) or 2 (u64), got %d", dtype);
+    return run_reduce_dtype(dtype, x, out, n, workspace, (hipStream_t)stream);
 }
 
 extern "C" int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int64_t c, void* stream) {

@@ -104,13 +104,13 @@ __device__ __forceinline__ void dma_to_lds(const unsigned char* base, unsigned l
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(lane_offset), "s"(base), "s"(lds_addr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // The same with a full address per lane (the last, partial K-tile of a ragged K: chunks past the end of a row
 // are fetched from a block of zeros instead).
 __device__ __forceinline__ void dma_to_lds_addr(const unsigned char* addr, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(addr), "s"(lds_addr) : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(addr), "s"(lds_addr) : "memory", "m0");
 }
 __device__ __attribute__((aligned(16))) const unsigned kZeroChunk[4] = {0u, 0u, 0u, 0u};
 
@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(const GemmArgs g) {
                      "global_load_lds_dwordx4 %10, %11"                                                                  \
                      : "+a"(c4), "+a"(c5), "+a"(c6), "+a"(c7)                                                            \
                      : "v"(b4), "v"(b5), "v"(b6), "v"(b7), "v"(a), "v"(vo0), "v"(vo1), "s"(base), "s"(dw), "n"(D0), "n"(D1) \
-                     : "memory", "scc")
+                     : "memory", "scc", "m0")
         if constexpr (DT == SP_BF16) SP_W4_BLOCK("bf16");
         else SP_W4_BLOCK("f16");
 #undef SP_W4_BLOCK
@@ -783,12 +783,14 @@ template <int DT>
 __global__ __launch_bounds__(256) void gemm_abt_generic_kernel(const GemmArgs g) {
     constexpr int ES = (DT == SP_F32) ? 4 : 2;
     constexpr int PER = 16 / ES;
-    const long n = (long)blockIdx.x * 16 + (threadIdx.x & 15);
-    const long m = (long)blockIdx.y * 16 + (threadIdx.x >> 4);
+    // blocks of 16 x 16 outputs, numbered row by row in blockIdx.x (a grid's y extent stops at 65535)
+    const long nb_n = (g.N + 15) / 16;
+    const long n = ((long)blockIdx.x % nb_n) * 16 + (threadIdx.x & 15);
+    const long m = ((long)blockIdx.x / nb_n) * 16 + (threadIdx.x >> 4);
     if (m >= g.M || n >= g.N) return;
-    const unsigned char* a = (const unsigned char*)g.A + (long)blockIdx.z * g.stride_a + m * g.K * ES;
-    const unsigned char* b = (const unsigned char*)g.B + (long)blockIdx.z * g.stride_b + n * g.K * ES;
-    unsigned char* const Cb = (unsigned char*)g.C + (long)blockIdx.z * g.stride_c;
+    const unsigned char* a = (const unsigned char*)g.A + (long)blockIdx.y * g.stride_a + m * g.K * ES;
+    const unsigned char* b = (const unsigned char*)g.B + (long)blockIdx.y * g.stride_b + n * g.K * ES;
+    unsigned char* const Cb = (unsigned char*)g.C + (long)blockIdx.y * g.stride_c;
     float s = 0.f;
     for (long k = 0; k < g.K; k += PER) {
         const u32x4 va = *reinterpret_cast<const u32x4*>(a + k * ES);
@@ -889,15 +891,8 @@ template <int DT, int OT, int BM, int BN, int WM, int WN, int NS, int NSA = NS, 
 static int launch_tiled_stages(const GemmArgs& g, hipStream_t stream) {
     auto kernel = gemm_abt_kernel<DT, OT, BM, BN, WM, WN, NS, NSA, RAGGED>;
     const int lds_bytes = (NSA * BM + NS * BN) * ROW_BYTES;
-    static bool attr_set[64] = {false};
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    if (!attr_set[dev & 63]) {
-        hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes,
-                                         hipGetErrorString(e));
-        attr_set[dev & 63] = true;
-    }
+    const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
+    if (rc != SP_OK) return rc;
     const long tiles = (long)g.tiles_m * g.tiles_n;
     hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(WM * WN * 64), lds_bytes, stream, g);
     return check_launch("sp_gemm_abt");
@@ -935,15 +930,8 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
     } else {
         auto kernel = gemm_abt_w4_kernel<DT, OT>;
         const int lds_bytes = 2 * (256 + 256) * ROW_BYTES;
-        static bool attr_set[64] = {false};
-        int dev = 0;
-        (void)hipGetDevice(&dev);
-        if (!attr_set[dev & 63]) {
-            hipError_t e = hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-            if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute(%d B LDS) failed: %s", lds_bytes,
-                                             hipGetErrorString(e));
-            attr_set[dev & 63] = true;
-        }
+        const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
+        if (rc != SP_OK) return rc;
         const long tiles = (long)g.tiles_m * g.tiles_n;
         hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(256), lds_bytes, stream, g);
         return check_launch("sp_gemm_abt");
@@ -959,7 +947,7 @@ static int launch_dtype(int cfg, const GemmArgs& g, hipStream_t stream) {
         case 1: return launch_tiled<DT, OT, 128, 128, 2, 2>(g, stream);
         case 2: return launch_tiled<DT, OT, 64, 64, 2, 2>(g, stream);
     }
-    dim3 grid((unsigned)((g.N + 15) / 16), (unsigned)((g.M + 15) / 16), (unsigned)g.batch);
+    dim3 grid((unsigned)(((g.N + 15) / 16) * ((g.M + 15) / 16)), (unsigned)g.batch);
     hipLaunchKernelGGL(gemm_abt_generic_kernel<DT>, grid, dim3(256), 0, stream, g);
     return check_launch("sp_gemm_abt(generic)");
 }
@@ -976,7 +964,13 @@ static int validate_gemm(int dtype_in, int dtype_out, int64_t M, int64_t N, int6
     const int per = dtype_in == SP_F32 ? 4 : 8;
     if (K % per != 0)
         return fail(SP_ERR_SHAPE, "sp_gemm_abt: K must be a multiple of %d (16-byte rows), got %lld", per, (long long)K);
-    if (M > (1ll << 31) || N > (1ll << 31) || K > (1ll << 31)) return fail(SP_ERR_SHAPE, "sp_gemm_abt: dimension too large");
+    // What the kernels can address: the loaders keep per-lane byte offsets of up to 7 rows (231 in the four-wave
+    // kernel, which has a K limit of its own) in 32 bits, and a launch numbers its workgroups with an int.
+    const int es = dtype_in == SP_F32 ? 4 : 2;
+    if (M > (1ll << 31) || N > (1ll << 31) || K * es > (1ll << 29))
+        return fail(SP_ERR_SHAPE, "sp_gemm_abt: dimension too large (M, N <= 2^31, rows of A and B <= 512 MiB)");
+    if (((M + 15) / 16) * ((N + 15) / 16) > 2147483647ll)
+        return fail(SP_ERR_SHAPE, "sp_gemm_abt: M x N too large (more than 2^31 - 1 blocks of 16 x 16 outputs)");
     return SP_OK;
 }
 

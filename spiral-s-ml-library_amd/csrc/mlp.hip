@@ -84,7 +84,7 @@ __device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
                  :
                  : "v"(lane_offset), "s"(base), "s"(lds_addr)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // Head of one batch row: optional softmax and/or regret matching over the columns j < limit, then
@@ -1204,29 +1204,11 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     } else {
         kernel = wide ? (const void*)mlp_forward_kernel<SP_BF16, 8> : (const void*)mlp_forward_kernel<SP_BF16, 4>;
     }
-    // the LDS opt-in is per kernel and device; remember which (kernel, device) pairs have it (a lost
-    // race only repeats an idempotent call)
-    static const void* opted_kernel[64];
-    static int opted_device[64];
-    static int n_opted = 0;
-    int dev = 0;
-    (void)hipGetDevice(&dev);
-    bool opted = false;
-    const int n_seen = n_opted < 64 ? n_opted : 64;
-    for (int i = 0; i < n_seen; ++i) opted = opted || (opted_kernel[i] == kernel && opted_device[i] == dev);
-    hipError_t e = hipSuccess;
-    if (!opted) {
-        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
-        if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(e));
-        if (n_seen < 64) {
-            opted_kernel[n_seen] = kernel;
-            opted_device[n_seen] = dev;
-            n_opted = n_seen + 1;
-        }
-    }
+    rc = ensure_dynamic_lds(kernel, lds_bytes);
+    if (rc != SP_OK) return rc;
     const long blocks = (batch + rows_per_block - 1) / rows_per_block;
     void* args[] = {(void*)&a};
-    e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
+    hipError_t e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward: launch failed: %s", hipGetErrorString(e));
     return check_launch(__func__);
 }

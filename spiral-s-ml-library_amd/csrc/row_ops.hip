@@ -305,7 +305,7 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int j = c * 4 * T + 4 * l + k;
-                    if (ok[c] && j < 32 && v[c][k] > 0.f) bits |= 1u << j;
+                    if (ok[c] && j < 32 && !(v[c][k] <= 0.f)) bits |= 1u << j;   // the reference's test: a NaN sets its bit
                 }
             bits = group_reduce<T>(bits, [](unsigned x, unsigned y) { return x | y; });
         }
@@ -520,7 +520,8 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
         const long r = r0 + sub;
         const long b = r * (long)cols + 4 * l;
         // first: whoever waits for a piece of the row then has the uniform too
-        uu = a.philox_mode >= 0 ? reference_row_uniform(a, r) : a.u[r];
+        // (no uniform tensor and no generator: nothing samples, and no load is issued for it)
+        uu = a.philox_mode >= 0 ? reference_row_uniform(a, r) : (a.u != nullptr ? a.u[r] : 1.f);
 #pragma unroll
         for (int c = 0; c < C; ++c) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
     };
@@ -533,7 +534,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
             w[c] = f32x4{NEG_INF, NEG_INF, NEG_INF, NEG_INF};
             if (r < a.rows && c * 4 * T + 4 * l < cols) w[c] = *reinterpret_cast<const f32x4*>(a.x + b + c * 4 * T);
         }
-        uu = r < a.rows ? (a.philox_mode >= 0 ? reference_row_uniform(a, r) : a.u[r]) : 1.f;
+        uu = r < a.rows ? (a.philox_mode >= 0 ? reference_row_uniform(a, r) : (a.u != nullptr ? a.u[r] : 1.f)) : 1.f;
     };
 
     // The uniform is requested together with the row: the counter of outstanding loads runs in
@@ -765,10 +766,7 @@ template <bool FUSED>
 static int launch_row(const RowArgs& args, hipStream_t stream, const char* fn) {
     int rc = require_gfx950(fn);
     if (rc != SP_OK) return rc;
-    RowArgs a = args;
-    // The fused kernels read one uniform per row whether a sample is wanted or not; without one
-    // they read the first `rows` inputs instead, which exist because a row has at least 4 columns.
-    if (FUSED && a.u == nullptr) a.u = a.x;
+    const RowArgs& a = args;
     const int t = lanes_per_row(a.cols);
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
@@ -851,7 +849,7 @@ extern "C" int sp_philox_uniforms(const sp_philox_t* philox, float* u_out, int64
 
 extern "C" int sp_row_ops(const float* logits, const float* u, float* rowmax, float* rowsum, float* probs, float* cdf,
                           int32_t* argmax, int32_t* sample, int64_t rows, int64_t cols, uint32_t flags, void* stream) {
-    (void)flags;
+    if (flags != 0) return fail(SP_ERR_ARG, "sp_row_ops: flags is reserved and must be 0, got %u", flags);
     SP_REQUIRE_PTR(logits);
     SP_OPTIONAL_PTR(rowmax); SP_OPTIONAL_PTR(rowsum); SP_OPTIONAL_PTR(probs); SP_OPTIONAL_PTR(cdf);
     SP_OPTIONAL_PTR(argmax); SP_OPTIONAL_PTR(sample); SP_OPTIONAL_PTR(u);

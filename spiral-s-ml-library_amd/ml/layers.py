@@ -676,7 +676,8 @@ def _fused_plan(model):
     weights.reverse()
     dims = [node.spec.dim[-1]] + [w.spec.dim[0] for w in weights]
     ok = node.spec.dtype in (torch.float16, torch.bfloat16) and all(w.spec.dtype == node.spec.dtype for w in weights)
-    ok = ok and builtins.max(dims) <= 256   # `max` is a node constructor in this module and dims[0] % 16 == 0 and all(d % 32 == 0 for d in dims[1:-1]) and dims[-1] <= 64
+    # the shapes sp_mlp_forward takes (`max` is a node constructor in this module, hence builtins.max)
+    ok = ok and builtins.max(dims) <= 256 and dims[0] % 16 == 0 and all(d % 32 == 0 for d in dims[1:-1]) and dims[-1] <= 64
     return (node, weights, top, head_ops[top.f]) if ok else None
 
 

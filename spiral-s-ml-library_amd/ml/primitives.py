@@ -274,7 +274,8 @@ def reduce_sum(x):
     code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
     key = x.device.index
     if key not in _workspace:
-        _workspace[key] = torch.empty(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=x.device)
+        # zero-filled once: the kernel keeps a ticket counter in it and leaves it at zero after every call
+        _workspace[key] = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=x.device)
     ws = _workspace[key]
     out = torch.empty(4, dtype=x.dtype, device=x.device)  # 16-byte aligned scalar slot
     check(lib.sp_reduce_sum(code, ptr(x, name="x"), ptr(out), x.numel(), ptr(ws), ws.numel(), stream_ptr()))
@@ -339,6 +340,26 @@ def test2(m, n, head_dir, root="test_text_outputs/primitives/"):
     _row_test(root, m, n, head_dir, grid=False)
 
 
+def test3(n, head_dir, root="test_text_outputs/primitives/"):
+    """ml/primitives.spi test3 (:851-902): the `row_gather_*` ops, one row of width n per thread of the grid
+    (threads_per_block * blocks_per_grid rows).  Row indices, the identity map, masked (j < 3) regret matching
+    and a masked-softmax sample drawn from each thread's own Philox subsequence."""
+    m = THREADS_PER_BLOCK * BLOCKS_PER_GRID
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(CONSTANT_SEED)
+    input_identity = torch.arange(m * n, dtype=torch.float32, device="cuda").reshape(m, n)
+    x = torch.randn((m, n), generator=gen, device="cuda", dtype=torch.float32)
+    ii = torch.arange(m, dtype=torch.int32, device="cuda")[:, None].expand(m, n)
+    jj = torch.arange(n, dtype=torch.int32, device="cuda")[None, :].expand(m, n)
+    _, sample = masked_softmax_and_discrete_sampling(x, 3, rng=philox(_lib.PHILOX_GATHER), want_probs=False)
+    _dump(root, head_dir, "input_identity.txt", 1024, input_identity)
+    _dump(root, head_dir, "output_sample_reduce.txt", 1024, sample)
+    _dump(root, head_dir, "output_indices_map.txt", 1024, ii, jj)
+    _dump(root, head_dir, "output_indices_reduce.txt", 1024, ii[:, 0])
+    _dump(root, head_dir, "output_op_map.txt", 1024, masked_regret_matching(x, 3))
+    _dump(root, head_dir, "zip_input_output_identity_map.txt", 1024, x, identity(x))
+
+
 def test4(m, n, head_dir, root="test_text_outputs/primitives/"):
     _row_test(root, m, n, head_dir, grid=True)
 
@@ -364,9 +385,11 @@ def test6(m, n, head_dir, root="test_text_outputs/primitives/"):
 
 
 def main_body(root="test_text_outputs/primitives/"):
-    """ml/primitives.spi main (:1112-1137).  test3 (row_gather_*) is not part of this build."""
+    """ml/primitives.spi main (:1112-1137): tests 2 to 6 in the reference's order."""
     test2(1 << 6, 1 << 7, "test2/a/", root)
     test2(1 << 7, 1 << 6, "test2/b/", root)
+    test3(1 << 4, "test3/a", root)
+    test3(1 << 8, "test3/b", root)
     test4(1 << 7, 1 << 6, "test4/b/", root)
     test4(1 << 6, 1 << 7, "test4/a/", root)
     test5(2, 4, 8, "test5/a", root)

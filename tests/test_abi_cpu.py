@@ -54,6 +54,12 @@ def test_gemm_argument_errors(L):
     assert lib.sp_gemm_abt(*args(din=7)) == -4
     assert lib.sp_gemm_abt(*args(din=1, dout=2)) == -4
     assert lib.sp_gemm_abt(*args(alpha=0.0)) == -5 and "alpha must not be zero" in _err(L)
+    # what the kernels cannot address is refused on the host: rows longer than 512 MiB (32-bit lane offsets),
+    # more blocks than a launch can number
+    assert lib.sp_gemm_abt(*args(K=(1 << 28) + 8)) == -2 and "too large" in _err(L)
+    assert lib.sp_gemm_abt(*args(din=0, K=(1 << 27) + 4)) == -2 and "too large" in _err(L)
+    assert lib.sp_gemm_abt(*args(M=1 << 20, N=1 << 20)) == -2 and "too large" in _err(L)
+    assert lib.sp_gemm_abt(*args(M=(1 << 31) + 1)) == -2
 
 
 def test_batched_gemm_argument_errors(L):
@@ -75,6 +81,7 @@ def test_row_argument_errors(L):
     assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 8, 6, 0, None) == -2
     assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 8, 2048, 0, None) == -2
     assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 0, 8, 0, None) == -2
+    assert lib.sp_row_ops(p, None, None, None, None, None, None, None, 8, 8, 1, None) == -5 and "flags" in _err(L)
     assert lib.sp_row_ops(p, None, None, None, None, None, None, p, 8, 8, 0, None) == -1  # sample without u
     assert lib.sp_row_ops(p, None, None, None, C.c_void_p(0x2008), None, None, None, 8, 8, 0, None) == -3
     assert lib.sp_row_map_f32(99, p, p, 8, 8, 0, None) == -5

@@ -269,18 +269,26 @@ def test_four_wave_kernel_is_exact_on_integers(MM, dtype):
     assert (many.reshape(m, n) == want).all()
 
 
-def test_config2_8192_sampled_rows(MM):
-    """8192^3 in bf16: the oracle is evaluated on 192 sampled rows of C (a full CPU product is
-    ~1.1 TFLOP); linearity is checked on the whole output: (2A).B^T == 2 (A.B^T) exactly."""
-    announce("gemm config 2: 8192^3 bf16 (sampled rows)")
+@pytest.mark.parametrize("dtype,out16", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
+def test_config2_8192_sampled_rows(MM, dtype, out16):
+    """8192^3, both 16-bit input types, f32 and 16-bit output: the oracle is evaluated on 192 sampled rows of C
+    (a full CPU product is ~1.1 TFLOP); linearity is checked on the whole output: (2A).B^T == 2 (A.B^T) exactly
+    (a factor of two commutes with every rounding involved)."""
+    announce("gemm config 2: 8192^3 %s -> %s (sampled rows)" % (dtype, dtype if out16 else "f32"))
     rng = np.random.default_rng(3)
     n = 8192
-    a, b = make(rng, n, n, n, "bf16")
-    ad, bd = dev(a, torch.bfloat16), dev(b, torch.bfloat16)
-    c = MM.matmul_abt(ad, bd)
+    t = TORCH[dtype]
+    a, b = make(rng, n, n, n, dtype)
+    ad, bd = dev(a, t), dev(b, t)
+    kw = dict(out_dtype=t) if out16 else {}
+    c = MM.matmul_abt(ad, bd, **kw)
+    assert c.dtype == (t if out16 else torch.float32)
     rows = rng.choice(n, 192, replace=False)
-    assert ogemm.rel_frobenius(host(c[torch.from_numpy(rows).cuda()]), ogemm.gemm_abt(a[rows], b)) < TOL["bf16"]
-    c2 = MM.matmul_abt(ad * 2, bd)
+    want = ogemm.gemm_abt(a[rows], b)
+    if out16:
+        want = ogemm.round_to(want, dtype)
+    assert ogemm.rel_frobenius(host(c[torch.from_numpy(rows).cuda()].float()), want) < TOL[dtype]
+    c2 = MM.matmul_abt(ad * 2, bd, **kw)
     assert torch.equal(c2, c * 2)
 
 

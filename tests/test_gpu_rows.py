@@ -354,3 +354,46 @@ def test_row_ops_full_size(P):
     # scalar-outputs-only mode gives the same indices
     lean = P.row_ops(dev(x), dev(u), want=("argmax", "sample", "rowmax", "rowsum"))
     assert (host(lean["sample"]) == out["sample"]).all() and (host(lean["argmax"]) == out["argmax"]).all()
+
+
+def test_main_body_writes_the_reference_files(P, golden, tmp_path):
+    """`primitives.main_body` (ml/primitives.spi main, :1112-1137) writes every file of the reference's
+    test_text_outputs/primitives tree; the files that do not depend on the random input are parsed back with the
+    fixture parser and must equal the reference's own prints exactly (same leaves, same truncation)."""
+    import os
+    import sys
+    from conftest import GOLDEN
+    if GOLDEN not in sys.path:
+        sys.path.insert(0, GOLDEN)
+    import make_fixtures as mf
+
+    announce("primitives.main_body")
+    root = str(tmp_path) + "/"
+    P.main_body(root)
+    torch.cuda.synchronize()
+    fixed = {"test2": ["input_identity", "output_identity", "output_indices_map", "output_indices_reduction",
+                       "output_sum_exclusive"],
+             "test3": ["input_identity", "output_indices_map", "output_indices_reduce"],
+             "test6": ["input_identity", "output_reduce_block", "output_reduce_grid"]}
+    fixed["test4"] = fixed["test2"]
+    every = {"test2": mf.ROW_NAMES, "test4": mf.ROW_NAMES, "test3": mf.GATHER_NAMES, "test6": mf.REDUCE_NAMES}
+    for test, sub in [("test2", "a"), ("test2", "b"), ("test3", "a"), ("test3", "b"), ("test4", "a"), ("test4", "b"),
+                      ("test6", "a")]:
+        want = golden("primitives_%s_%s" % (test, sub))
+        got = mf.convert_case(os.path.join(root, test, sub), every[test])
+        assert set(got) == set(want), (test, sub, sorted(set(want) ^ set(got)))   # the same files exist
+        for key in fixed[test]:
+            assert got[key].shape == want[key].shape and (got[key] == want[key]).all(), (test, sub, key)
+            assert bool(got[key + "__truncated"]) == bool(want[key + "__truncated"]), (test, sub, key)
+        for key in want:                                      # input-dependent files: same extent of the print
+            assert got[key].shape == want[key].shape, (test, sub, key)
+    for sub in ("a", "b"):
+        want = golden("primitives_test5_" + sub)
+        with open(os.path.join(root, "test5", sub, "transpose.txt")) as f:
+            parts = [ln for ln in f.read().splitlines() if ln.startswith("[")]
+        assert len(parts) == 2
+        assert (mf.to_array(*mf.parse_tensor_text(parts[0])) == want["input"]).all()
+        assert (mf.to_array(*mf.parse_tensor_text(parts[1])) == want["output"]).all()
+    # the sampled indices of test3 obey the mask (j < 3)
+    s3 = mf.convert_case(os.path.join(root, "test3", "b"), ["output_sample_reduce"])["output_sample_reduce"]
+    assert s3.shape == (1024,) and (s3 >= 0).all() and (s3 < 3).all()

@@ -111,3 +111,23 @@ def test_printing_uses_the_golden_text_format():
     # the first three lines of the reference's layers/test1/layers.txt after "---"
     row = "[0.000000; 0.000000; 0.000000; 0.000000]"
     assert lines == ["[" + "; ".join([row] * 4) + "]"] * 2 + ["[" + "; ".join([row] * 2) + "]"]
+
+
+def test_fused_plan_takes_only_the_shapes_the_fused_kernel_runs():
+    """A 16-bit relu stack with a sampling head is planned as one fused launch only for the widths the fused
+    kernel accepts (input a multiple of 16, hidden widths multiples of 32, nothing above 256, head <= 64)."""
+    def stack(dims, dtype="f16"):
+        x = L.input("input", (24, 16, dims[0]), dtype)
+        for i, (k, n) in enumerate(zip(dims[:-1], dims[1:])):
+            x = L.matmul((k, n), x)
+            if i + 2 < len(dims):
+                x = L.relu(x)
+        return L.create_model(L.masked_softmax_and_discrete_sample(3, x), device="cpu")
+
+    assert L._fused_plan(stack([32, 256, 256, 64])) is not None
+    assert L._fused_plan(stack([32, 64, 3 * 32, 16])) is not None
+    assert L._fused_plan(stack([32, 48, 16])) is None          # hidden width not a multiple of 32
+    assert L._fused_plan(stack([32, 256, 128])) is None        # head wider than 64
+    assert L._fused_plan(stack([24, 256, 64])) is None         # input width not a multiple of 16
+    assert L._fused_plan(stack([32, 512, 64])) is None         # wider than 256
+    assert L._fused_plan(stack([32, 256, 64], "float")) is None   # f32 graphs run node by node

@@ -168,8 +168,27 @@ def test_binarize_and_get_prob_by_hand():
     wide = np.ones((1, 40), dtype=np.float32)          # columns 32.. are shifted out
     assert row_ops.binarize(wide, 2 ** 32 - 1).tolist() == [0]   # 0xFFFFFFFF mod 0xFFFFFFFF
     assert row_ops.binarize(wide, 2 ** 31).tolist() == [2 ** 31 - 1]
+    # the reference's bit test is `not (x <= 0)`: a NaN sets its bit, -0.0 and -inf do not
+    odd = np.array([[np.nan, -0.0, np.inf, -np.inf]], dtype=np.float32)
+    assert row_ops.binarize(odd, 100).tolist() == [0b0101]
     p = np.array([[0.1, 0.2, 0.7], [0.3, 0.3, 0.4]], dtype=np.float32)
     assert row_ops.get_prob(p, [2, 0]).tolist() == [np.float32(0.7), np.float32(0.3)]
+
+
+def test_chosen_edge_semantics_of_argmax_and_softmax():
+    """Where this build fixes what the reference leaves open (or does differently), the choice is pinned here:
+    argmax ties go to the LOWEST index (the reference's `if a > b then a else b` keeps the later operand inside a
+    thread and is order-dependent across threads), a row of NaNs gives index 0, and softmax shifts by the row max,
+    so it stays finite where the reference's shift by the mean overflows."""
+    x = np.array([[1, 3, 3, 2], [5, 5, 5, 5], [-1, -7, -1, -1]], dtype=np.float32)
+    assert row_ops.argmax(x).tolist() == [1, 0, 0]
+    assert row_ops.argmax(np.full((1, 8), np.nan, dtype=np.float32)).tolist() == [0]
+    big = np.array([[0, 0, 0, 200.0]], dtype=np.float32)      # exp(200 - mean 50) overflows f32, exp(200 - 200) does not
+    with np.errstate(over="ignore", invalid="ignore"):
+        assert not np.isfinite(row_ops.softmax(big, shift="mean")).all()
+    assert np.isfinite(row_ops.softmax(big)).all() and row_ops.softmax(big)[0, 3] == 1.0
+    small = np.array([[0.5, -1.0, 2.0, 0.0]], dtype=np.float32)
+    assert np.allclose(row_ops.softmax(small), row_ops.softmax(small, shift="mean"), rtol=1e-6)
 
 
 def test_layer_stream_reduces_to_block_stream_and_shifts_by_offset():
