@@ -273,7 +273,7 @@ def test_four_wave_kernel_is_exact_on_integers(MM, dtype):
 def test_config2_8192_sampled_rows(MM, dtype, out16):
     """8192^3, both 16-bit input types, f32 and 16-bit output: the oracle is evaluated on 192 sampled rows of C
     (a full CPU product is ~1.1 TFLOP); linearity is checked on the whole output: (2A).B^T == 2 (A.B^T) exactly
-    (a factor of two commutes with every rounding involved)."""
+    (a factor of two commutes with every rounding involved, f16 subnormals aside)."""
     announce("gemm config 2: 8192^3 %s -> %s (sampled rows)" % (dtype, dtype if out16 else "f32"))
     rng = np.random.default_rng(3)
     n = 8192
@@ -289,7 +289,14 @@ def test_config2_8192_sampled_rows(MM, dtype, out16):
         want = ogemm.round_to(want, dtype)
     assert ogemm.rel_frobenius(host(c[torch.from_numpy(rows).cuda()].float()), want) < TOL[dtype]
     c2 = MM.matmul_abt(ad * 2, bd, **kw)
-    assert torch.equal(c2, c * 2)
+    if out16 and dtype == "f16":
+        # f16 results below 2^-14 are subnormal: their spacing is fixed at 2^-24, so the doubled sum is rounded
+        # on a grid that 2 * (rounded sum) does not share.  Exact in the normal range, one step of 2^-24 below it.
+        normal = c.abs() >= 2.0 ** -13
+        assert torch.equal(c2[normal], (c * 2)[normal])
+        assert float((c2.float() - 2 * c.float()).abs().max()) <= 2.0 ** -24
+    else:
+        assert torch.equal(c2, c * 2)
 
 
 @pytest.mark.parametrize("k,n", [(256, 256), (512, 1024), (2048, 256)])
