@@ -181,7 +181,7 @@ def main():
             ("gemm_bf16_65536x256x256_bias_relu", lambda: gemm_case(4, 65536, 256, 256, "bf16", bias_relu=True)[0]),
         ]
 
-        def mlp_case():
+        def mlp_case(packed=True):
             rng = np.random.default_rng(7)
             dims = [32, 256, 256, 256, 3]
             batch = 16384
@@ -195,16 +195,27 @@ def main():
             from ml import _lib
             wp = (C.c_void_p * 4)(*[w.data_ptr() for w in wd])
             dp = (C.c_int32 * 5)(*dims)
-            call = (_lib.SP_F16, _lib.ptr(xd), 4, wp, None, dp, _lib.ptr(ud), _lib.ptr(policy), _lib.ptr(action), None,
-                    batch, _lib.HEAD_SOFTMAX_RM, 0)
-            fn = lambda: _lib.check(_lib.lib.sp_mlp_forward(*call, _lib.stream_ptr()))
+            if packed:
+                # the weights are packed into MFMA operand order ONCE, outside the timed region (a change of layout
+                # made when the weights are set, like a transpose at model load); every timed step is one
+                # sp_mlp_forward_packed launch that reads nothing but the packed buffer, x and u
+                pk = layers.pack_weights(wd)
+                call = (_lib.SP_F16, _lib.ptr(xd), 4, _lib.ptr(pk.buffer), None, dp, _lib.ptr(ud), _lib.ptr(policy),
+                        _lib.ptr(action), None, batch, _lib.HEAD_SOFTMAX_RM, 0)
+                fn = lambda: _lib.check(_lib.lib.sp_mlp_forward_packed(*call, _lib.stream_ptr()))
+            else:
+                call = (_lib.SP_F16, _lib.ptr(xd), 4, wp, None, dp, _lib.ptr(ud), _lib.ptr(policy), _lib.ptr(action), None,
+                        batch, _lib.HEAD_SOFTMAX_RM, 0)
+                fn = lambda: _lib.check(_lib.lib.sp_mlp_forward(*call, _lib.stream_ptr()))
             wall, ev = time_launches(fn, max(K, 200), W)
             want_p, want_a, _ = olayers.mlp_forward(x, ws, u=u)
             assert ogemm.rel_frobenius(policy.cpu().numpy(), want_p) < 3e-3, "bench MLP output drifted from the oracle"
             fl = 2.0 * batch * sum(i * o for i, o in zip(dims[:-1], dims[1:]))
             res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
                    "roofline": roofline_mfma(fl, ev, "f16"), "seed": 7,
-                   "timing": "mean over back-to-back launches between two HIP events"}
+                   "timing": "mean over back-to-back launches between two HIP events" +
+                             ("; weights packed once before the timed region (sp_mlp_pack_weights)" if packed else
+                              "; row-major weights (sp_mlp_forward)")}
             if not args.no_cpu:
                 t = best_of(lambda: olayers.mlp_forward(x, ws, u=u), 3)
                 res["cpu_rows_per_s"] = round(batch / t, 1)
@@ -285,7 +296,8 @@ def main():
                     "timing": "mean over back-to-back graph_run_host calls (one fused-MLP launch each; the run's Philox "
                               "uniforms depend on (model, seed) only and are drawn when the plan is built)"}
 
-        cases += [("mlp_leduc_16384", mlp_case), ("layers_graph_leduc_16384", graph_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
+        cases += [("mlp_leduc_16384", mlp_case), ("mlp_leduc_16384_rowmajor", lambda: mlp_case(False)),
+                  ("layers_graph_leduc_16384", graph_case), ("row_ops_65536x256_scalars", lambda: rows_case(False)),
                   ("row_ops_65536x256_materialised", lambda: rows_case(True)),
                   ("map_relu_65536x256", lambda: elementwise_case("map_relu")),
                   ("reduce_sum_f32_65536x256", lambda: elementwise_case("reduce_sum")),

@@ -248,7 +248,7 @@ typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID
 int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream);
 
 /* Sum of all n elements into out[0], one launch.  dtype: 0 = f32, 1 = i32, 2 = u64.  `workspace` must hold
- * at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial sums and a ticket counter;
+ * at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial sums and ticket counters;
  * no allocation here).  It must be ZERO-FILLED once before its first use; every call leaves it ready for the
  * next one.  Calls that may run at the same time need a workspace each.  The order of the additions depends
  * on n only, so the f32 result is the same from run to run.
@@ -303,6 +303,31 @@ typedef enum {
 int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights, const float* const* biases,
                    const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,
                    int64_t batch, int32_t head, int32_t mask_size, void* stream);
+
+/*
+ * The same forward pass over weights that were packed once into MFMA operand order: the weights then stream
+ * from global memory straight into registers, every load of a launch in flight from its first cycle, instead of
+ * through an LDS ring (config 3: 8.5 us -> see the bench).  Build extension; the reference keeps its weights
+ * row-major in the weights arena (ml/layers.spi:127-179) and has no counterpart.
+ *
+ *   sp_mlp_packed_bytes   size of the packed buffer for a stack, 0 when the packed kernel does not take it:
+ *                         3 to 5 layers, every hidden width 256, dims[0] a multiple of 16 and <= 256,
+ *                         dims[n_layers] <= 64
+ *   sp_mlp_pack_weights   writes `packed` (caller memory, 16-byte aligned, at least sp_mlp_packed_bytes) from
+ *                         the row-major `weights` of sp_mlp_forward; one small launch, nothing is allocated.
+ *                         Has to be repeated whenever the weights change; the packed buffer holds no pointers.
+ *                         Of an output layer wider than 16 only the first 16 rows are packed.
+ *   sp_mlp_forward_packed sp_mlp_forward with `packed` in place of `weights`; same results (the k-order of the
+ *                         sums is the same).  At most 16 outputs: dims[n_layers] <= 16, or a masked head of at
+ *                         most 16 columns without logits_out.  SP_ERR_UNSUPPORTED for any other stack: call
+ *                         sp_mlp_forward with the row-major weights instead.
+ */
+int64_t sp_mlp_packed_bytes(int32_t n_layers, const int32_t* dims);
+int sp_mlp_pack_weights(int dtype, int32_t n_layers, const void* const* weights, const int32_t* dims, void* packed,
+                        int64_t packed_bytes, void* stream);
+int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void* packed, const float* const* biases,
+                          const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,
+                          int64_t batch, int32_t head, int32_t mask_size, void* stream);
 
 #ifdef __cplusplus
 }

@@ -16,7 +16,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libspiral_mi355.so")
-SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip"]
+SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"),
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
          "-Wno-unknown-warning-option",
@@ -43,7 +43,7 @@ def build(force=True, verbose=False):
     """Compile every HIP source and link the shared library.  Returns the library path."""
     os.makedirs(OBJ, exist_ok=True)
     cc = hipcc()
-    headers = [os.path.join(CSRC, "common.h"), os.path.join(ROOT, "include", "spiral_mi355.h")]
+    headers = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "mlp_common.h"), os.path.join(ROOT, "include", "spiral_mi355.h")]
     newest_header = max(os.path.getmtime(h) for h in headers)
 
     def compile_one(src):

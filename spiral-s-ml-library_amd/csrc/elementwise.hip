@@ -48,17 +48,26 @@ __device__ __forceinline__ T block_sum(T v, T* slots) {
 }
 
 // Full-tensor sum in ONE launch.  Every block adds up its share (16-byte loads, U of them in flight per lane and U
-// independent running sums), writes its partial sum to `partial[blockIdx.x]` and takes a ticket from `counter`;
-// the block that draws the last ticket adds the partials in index order and writes the result.  Which block that
-// is changes from run to run, the order of the additions does not: the result depends on n and the grid only.
-// `counter` must be zero when the kernel starts; the last block leaves it at zero for the next launch.
-// The partials cross between the private L2 caches of the XCDs: the writer's device-scope fence writes them back
-// before its ticket is taken, and the last block's fence discards stale lines before it reads them.
+// independent running sums), writes its partial sum to `partial[blockIdx.x]` and takes a ticket; the block that
+// draws the last ticket adds the partials in index order and writes the result.  Which block that is changes from
+// run to run, the order of the additions does not: the result depends on n and the grid only.
+// Tickets are drawn in two levels -- a counter per group of REDUCE_GROUP blocks, then one counter that the last
+// block of every group draws from: atomic operations on ONE address take ~11 ns each on this part, whoever issues
+// them (2048 tickets from one counter: 23 us), on different addresses they overlap.
+// Partial sums and counters are device-scope atomic accesses: they go to memory past the XCD's private L2, so
+// nothing has to be written back or invalidated (a device-scope fence walks the whole L2, once per block: 60 us
+// for 2048 blocks).  A partial sum's store has completed before its block draws a ticket.
+// `counters` (REDUCE_COUNTERS of them, REDUCE_COUNTER_STRIDE bytes apart) must be zero when the kernel starts;
+// the blocks that draw last tickets leave them at zero for the next launch.
+constexpr int REDUCE_GROUP = 64;
+constexpr int REDUCE_COUNTERS = REDUCE_MAX_BLOCKS / REDUCE_GROUP + 1;     // one per group, then the top one
+constexpr int REDUCE_COUNTER_STRIDE = 256;
+
 template <typename T, int U>
 __global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restrict__ x, T* __restrict__ out, long n,
-                                                                T* partial, unsigned* counter) {
+                                                                T* partial, unsigned char* counters) {
     __shared__ T slots[EW_THREADS / WAVE];
-    __shared__ unsigned ticket;
+    __shared__ unsigned is_last;
     constexpr int V = 16 / sizeof(T);
     typedef T VT __attribute__((ext_vector_type(V)));
     const VT* xv = reinterpret_cast<const VT*>(x);
@@ -87,25 +96,29 @@ __global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restr
     for (long j = nv * V + tid; j < n; j += stride) acc += x[j];   // the last n % V elements
     acc = block_sum(acc, slots);
     if (threadIdx.x == 0) {
-        partial[blockIdx.x] = acc;
-        __threadfence();
-        ticket = atomicAdd(counter, 1u);
+        __hip_atomic_store(partial + blockIdx.x, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const unsigned group = blockIdx.x / REDUCE_GROUP, groups = (gridDim.x + REDUCE_GROUP - 1) / REDUCE_GROUP;
+        const unsigned members = group + 1 < groups ? REDUCE_GROUP : gridDim.x - group * REDUCE_GROUP;
+        unsigned* mine = reinterpret_cast<unsigned*>(counters + group * REDUCE_COUNTER_STRIDE);
+        unsigned* top = reinterpret_cast<unsigned*>(counters + (REDUCE_COUNTERS - 1) * REDUCE_COUNTER_STRIDE);
+        unsigned last = 0;
+        if (__hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
+            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (__hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
+                __hip_atomic_store(top, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = 1;
+            }
+        }
+        is_last = last;
     }
     __syncthreads();
-    if (ticket != gridDim.x - 1) return;
-    __threadfence();
+    if (is_last == 0) return;
     T total = T(0);
-    for (unsigned b = threadIdx.x; b < gridDim.x; b += EW_THREADS) total += partial[b];
+    for (unsigned b = threadIdx.x; b < gridDim.x; b += EW_THREADS)
+        total += __hip_atomic_load(partial + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     total = block_sum(total, slots);
-    if (threadIdx.x == 0) {
-        out[0] = total;
-        *counter = 0u;
-    }
-}
-
-// Sets `count` 32-bit words to zero (a kernel rather than a memset so that callers may record it into a graph).
-__global__ __launch_bounds__(WAVE) void clear_words_kernel(unsigned* p, int count) {
-    for (int i = threadIdx.x; i < count; i += WAVE) p[i] = 0u;
+    if (threadIdx.x == 0) out[0] = total;
 }
 
 // to[a][c][b] = from[a][b][c]; 64x64 tiles through LDS, padded by one word per row so that the
@@ -165,18 +178,17 @@ __global__ __launch_bounds__(EW_THREADS) void transpose_vec4_kernel(const unsign
     }
 }
 
-// Layout of a reduction's scratch memory: REDUCE_MAX_BLOCKS partial sums of 8 bytes, then the ticket counter.
+// Layout of a reduction's scratch memory: REDUCE_MAX_BLOCKS partial sums of 8 bytes, then the ticket counters.
 constexpr long REDUCE_COUNTER_OFFSET = (long)REDUCE_MAX_BLOCKS * 8;
-constexpr long REDUCE_SCRATCH_BYTES = REDUCE_COUNTER_OFFSET + 256;
+constexpr long REDUCE_SCRATCH_BYTES = REDUCE_COUNTER_OFFSET + (long)REDUCE_COUNTERS * REDUCE_COUNTER_STRIDE;
 
 template <typename T>
 static int run_reduce(const void* x, void* out, int64_t n, void* scratch_mem, hipStream_t stream) {
     long blocks = (n + EW_THREADS * 16 - 1) / (EW_THREADS * 16);   // >= 4 vectors of 16 bytes per lane
     if (blocks > REDUCE_MAX_BLOCKS) blocks = REDUCE_MAX_BLOCKS;
     if (blocks < 1) blocks = 1;
-    unsigned* counter = reinterpret_cast<unsigned*>((unsigned char*)scratch_mem + REDUCE_COUNTER_OFFSET);
     hipLaunchKernelGGL((reduce_sum_kernel<T, 4>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x, (T*)out,
-                       (long)n, (T*)scratch_mem, counter);
+                       (long)n, (T*)scratch_mem, (unsigned char*)scratch_mem + REDUCE_COUNTER_OFFSET);
     return check_launch("sp_reduce_sum");
 }
 

@@ -25,156 +25,12 @@
 //
 // Semantics follow the graph interpreter of ml/layers.spi:194-240 (BlockMatmul = x . w^T with w
 // stored (out, in), relu = max 0) and the heads of ml/primitives.spi:711-722,748-798.
-#include "common.h"
+#include "mlp_common.h"
 
 #pragma clang fp contract(off)
 
 namespace sp {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-typedef __attribute__((ext_vector_type(2))) unsigned int u32x2;
-
-constexpr int MLP_MAX_LAYERS = 8;
-constexpr int MLP_MAX_DIM = 256;       // widest layer input / hidden width
-constexpr int MLP_MAX_OUT = 64;        // widest head
-constexpr int MLP_STAGES = 4;
-constexpr int MLP_STAGE_BYTES = MLP_MAX_DIM * 128;   // 256 weight rows x 64 K-columns x 2 bytes
-constexpr int MLP_DMA_PER_CHUNK = MLP_MAX_DIM / 8;         // 1 KiB DMA instructions per full chunk
-constexpr int INT_MAX_ = 2147483647;
-
-struct MlpArgs {
-    const void* x;
-    const void* w[MLP_MAX_LAYERS];
-    const float* b[MLP_MAX_LAYERS];
-    int dims[MLP_MAX_LAYERS + 1];
-    int n_layers;
-    const float* u;
-    float* policy;
-    int* action;
-    float* logits;
-    long batch;
-    int head;
-    int mask_size;
-    int k0, nout;        // dims[0] and dims[n_layers] once more, so that a kernel needs no dependent load for them
-    int out_stride;      // floats between two rows of policy / logits (= dims[n_layers]; nout may be smaller, see sp_mlp_forward)
-};
-
-// max(x, 0) and rounding of two f32 values to the 16-bit storage type, packed into one register
-// (v_max_f32 + v_cvt_pk_{f16,bf16}_f32: round to nearest even in hardware).  The max is issued from
-// assembly because fmaxf() would first canonicalise its operand with a second v_max.
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-template <int DT>
-__device__ __forceinline__ unsigned relu_pack2(float a, float b) {
-    float ra, rb;
-    asm("v_max_f32 %0, 0, %1" : "=v"(ra) : "v"(a));
-    asm("v_max_f32 %0, 0, %1" : "=v"(rb) : "v"(b));
-    if constexpr (DT == SP_F16) return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{ra, rb}, f16x2));
-    else return __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{ra, rb}, bf16x2));
-}
-
-// One wave-wide DMA: lane i copies 16 bytes from base + lane_offset to LDS byte lds_addr + 16 * i.
-// Issued from inline assembly so the chunks in flight do not make the compiler wait before LDS
-// reads of the chunk being multiplied; completion is tracked by vmcnt.
-__device__ __forceinline__ void mlp_dma(const unsigned char* base, unsigned lane_offset, unsigned lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-                 :
-                 : "v"(lane_offset), "s"(base), "s"(lds_addr)
-                 : "memory", "m0");
-}
-
-// Head of one batch row: optional softmax and/or regret matching over the columns j < limit, then
-// local_discrete_sampling (ml/primitives.spi:782-798) with sequential prefix sums.  `src` holds the
-// row's N last-layer outputs; MAXN bounds N at compile time so that narrow heads stay in registers.
-// Columns past `limit` enter the softmax as -inf and leave it as exact zeros, columns past N are zeros
-// from the start: sums over all MAXN columns then equal the sums over the valid ones bit for bit, and
-// the loops need no per-column conditions.
-struct HeadOut {
-    float* policy;
-    int* action;
-    float* logits;
-    int head;
-    int stride;   // floats between two rows of policy / logits; columns N .. stride - 1 of policy are written as zeros
-};
-__device__ __forceinline__ HeadOut head_out(const MlpArgs& a) {
-    return HeadOut{a.policy, a.action, a.logits, a.head, a.out_stride};
-}
-
-template <int MAXN>
-__device__ __forceinline__ void head_row(const HeadOut& o, const float* src, long row, int N, int limit, float u,
-                                         int fill_end = 1 << 30) {
-    float p[MAXN];
-#pragma unroll
-    for (int n = 0; n < MAXN; ++n) p[n] = n < N ? src[n] : 0.f;
-    if (o.logits != nullptr) {
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n)
-            if (n < N) o.logits[row * o.stride + n] = p[n];
-    }
-    // exp on the hardware exp2 unit and one hardware reciprocal (1 ulp) per normalisation: a 16-lane
-    // serial head is otherwise a visible part of a forward pass that takes a few microseconds
-    if (o.head == SP_HEAD_SOFTMAX || o.head == SP_HEAD_SOFTMAX_RM) {
-        float m = -__builtin_inff();
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) {
-            p[n] = n < limit ? p[n] : -__builtin_inff();
-            m = fmaxf(m, p[n]);
-        }
-        float s = 0.f;
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) {
-            p[n] = __builtin_amdgcn_exp2f((p[n] - m) * 1.44269504088896340736f);
-            s = s + p[n];
-        }
-        const float inv = __builtin_amdgcn_rcpf(s);
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) p[n] = p[n] * inv;
-    }
-    if (o.head == SP_HEAD_REGRET_MATCHING || o.head == SP_HEAD_SOFTMAX_RM) {
-        float s = 0.f;
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) {
-            p[n] = n < limit ? fmaxf(p[n], 0.f) : 0.f;
-            s = s + p[n];
-        }
-        const float inv_len = __builtin_amdgcn_rcpf((float)limit);
-        const float inv = s != 0.f ? __builtin_amdgcn_rcpf(s) : 0.f;
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) p[n] = s != 0.f ? p[n] * inv : (n < limit ? inv_len : 0.f);
-    }
-#pragma unroll
-    for (int n = 0; n < MAXN; ++n)
-        if (n < N) o.policy[row * o.stride + n] = p[n];
-    if (o.stride > N) {   // a masked head computed for its valid columns only: the rest of the row is exact zeros
-        float* tail = o.policy + row * o.stride;   // (up to fill_end: the caller may fill the rest with whole waves)
-        const int end = o.stride < fill_end ? o.stride : fill_end;
-        int c = N;
-        for (; c < end && ((c & 3) != 0 || (o.stride & 3) != 0); ++c) tail[c] = 0.f;
-        for (; c + 4 <= end; c += 4) *reinterpret_cast<float4*>(tail + c) = make_float4(0.f, 0.f, 0.f, 0.f);
-    }
-    if (o.action != nullptr) {
-        float run = 0.f, m = -__builtin_inff();
-        float cdf[MAXN];
-#pragma unroll
-        for (int n = 0; n < MAXN; ++n) {
-            run = run + p[n];
-            cdf[n] = run;
-            if (p[n] > 0.f) m = fmaxf(m, run);
-        }
-        const float thr = u * m;
-        int pick = INT_MAX_;
-#pragma unroll
-        for (int n = MAXN - 1; n >= 0; --n)
-            if (p[n] > 0.f && cdf[n] >= thr) pick = n;
-        o.action[row] = pick;
-    }
-}
-
-__device__ __forceinline__ int mlp_swz(int row) { return (((row >> 3) & 3) << 1) | ((row >> 1) & 1); }
 
 // NW waves per workgroup, 16 batch rows per wave.
 template <int DT, int NW>
@@ -392,22 +248,6 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
 // past K0 re-read the last valid piece and meet zero activations), the last layer (at most 64
 // outputs) travels as ONE chunk holding its four 64-column slabs at 64-row spacing and always
 // computes 4 tiles (rows past the outputs are stale but finite-or-not they only reach unused columns).
-template <int N>
-struct IC { static constexpr int value = N; };
-
-// relu + rounding of four f32 to the 16-bit storage type: round first (v_cvt_pk), then clamp the two
-// packed values at zero as signed 16-bit integers -- a negative float of either format has the sign
-// bit set, so it is a negative integer, and relu commutes with the sign-symmetric rounding.
-template <int DT>
-__device__ __forceinline__ unsigned pack_relu2(float a, float b) {
-    unsigned p;
-    if constexpr (DT == SP_F16) p = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, f16x2));
-    else p = __builtin_bit_cast(unsigned, __builtin_convertvector(f32x2{a, b}, bf16x2));
-    unsigned r;
-    asm("v_pk_max_i16 %0, %1, 0" : "=v"(r) : "v"(p));
-    return r;
-}
-
 template <int DT, int NW, int C0>
 __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     constexpr int H = 256;

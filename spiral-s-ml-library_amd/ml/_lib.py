@@ -69,6 +69,10 @@ SIGNATURES = {
     "sp_transpose_inner_b32": (C.c_int, [_P, _P, _I64, _I64, _I64, _P]),
     "sp_mlp_forward": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
                                  _I64, _I32, _I32, _P]),
+    "sp_mlp_packed_bytes": (C.c_int64, [_I32, C.POINTER(C.c_int32)]),
+    "sp_mlp_pack_weights": (C.c_int, [C.c_int, _I32, C.POINTER(_P), C.POINTER(C.c_int32), _P, _I64, _P]),
+    "sp_mlp_forward_packed": (C.c_int, [C.c_int, _P, _I32, _P, C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
+                                        _I64, _I32, _I32, _P]),
 }
 
 
@@ -87,7 +91,8 @@ def load(path=LIB_PATH):
 # Entry points that launch work; their last argument is the stream.
 LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_row_map_f32", "sp_row_map_i32",
                       "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_update_mask",
-                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_transpose_inner_b32", "sp_mlp_forward"))
+                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
+                      "sp_mlp_forward_packed"))
 
 
 class Tape:

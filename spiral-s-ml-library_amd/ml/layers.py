@@ -36,21 +36,60 @@ HEADS = {None: _lib.HEAD_NONE, "none": _lib.HEAD_NONE, "softmax": _lib.HEAD_SOFT
 # fused dense stack
 # ----------------------------------------------------------------------------------------------
 
+class PackedWeights:
+    """The weights of a dense stack in the order the packed kernel multiplies them in (sp_mlp_pack_weights):
+    `buffer` is one uint8 tensor, `dims` the layer widths, `dtype` the storage type.  A snapshot: pack again after
+    the weights have changed (`pack_weights(weights, into=packed)` reuses the buffer)."""
+
+    def __init__(self, buffer, dims, dtype):
+        self.buffer, self.dims, self.dtype = buffer, list(dims), dtype
+
+
+def packed_bytes(dims):
+    """Bytes of the packed form of a stack with these widths; 0 when the packed kernel does not take the stack."""
+    return int(lib.sp_mlp_packed_bytes(len(dims) - 1, (C.c_int32 * len(dims))(*dims)))
+
+
+def pack_weights(weights, into=None):
+    """Pack the row-major weights [(out_i, in_i), ...] of a stack once, for `mlp_forward(..., packed=...)`.
+    Returns None when the packed kernel does not take the stack (then call mlp_forward with the weights)."""
+    dims = [weights[0].shape[1]] + [w.shape[0] for w in weights]
+    need = packed_bytes(dims)
+    if need == 0:
+        return None
+    n = len(weights)
+    if into is None:
+        into = PackedWeights(torch.empty(need, dtype=torch.uint8, device=weights[0].device), dims, weights[0].dtype)
+    elif into.dims != dims or into.dtype != weights[0].dtype:
+        raise ValueError("the packed buffer was made for another stack")
+    wp = (C.c_void_p * n)(*[ptr(w, weights[0].dtype, "weights[%d]" % i) for i, w in enumerate(weights)])
+    check(lib.sp_mlp_pack_weights(_lib.DTYPES[weights[0].dtype], n, wp, (C.c_int32 * (n + 1))(*dims), ptr(into.buffer),
+                                  into.buffer.numel(), stream_ptr()))
+    return into
+
+
 def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None, mask_size=0, want_logits=False,
-                policy_out=None, action_out=None):
+                policy_out=None, action_out=None, packed=None):
     """policy, action[, logits] = fused forward of relu-MLP + head + discrete sampling.
 
     x: (batch, in) f16/bf16; weights[i]: (out_i, in_i) of the same dtype (the B operand of A.B^T,
     ml/layers.spi:227-240,467); biases: optional list of f32 (out_i,) or None entries (build
     extension, the reference has no bias); u: (batch,) f32 uniforms in (0, 1] or None (no action).
     head: None | "softmax" | "regret_matching" | "softmax_regret_matching"; mask_size > 0 restricts
-    the head to columns j < mask_size (masked_* layers, ml/layers.spi:408-432)."""
-    n = len(weights)
-    dims = [x.shape[1]] + [w.shape[0] for w in weights]
-    for i, w in enumerate(weights):
-        if w.dtype != x.dtype:
-            raise TypeError("weights[%d] must have the dtype of x" % i)
-        assert w.shape[1] == dims[i], "The K dimension of the A and B tensors must match."
+    the head to columns j < mask_size (masked_* layers, ml/layers.spi:408-432).  packed: the result of
+    pack_weights(weights) -- the stack then runs on the packed kernel and `weights` is not read."""
+    if packed is not None:
+        n, dims = len(packed.dims) - 1, packed.dims
+        if packed.dtype != x.dtype:
+            raise TypeError("the packed weights must have the dtype of x")
+        assert x.shape[1] == dims[0], "The K dimension of the A and B tensors must match."
+    else:
+        n = len(weights)
+        dims = [x.shape[1]] + [w.shape[0] for w in weights]
+        for i, w in enumerate(weights):
+            if w.dtype != x.dtype:
+                raise TypeError("weights[%d] must have the dtype of x" % i)
+            assert w.shape[1] == dims[i], "The K dimension of the A and B tensors must match."
     batch = x.shape[0]
     policy = policy_out if policy_out is not None else \
         torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device)
@@ -58,15 +97,21 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
     if action is None and u is not None:
         action = torch.empty((batch,), dtype=torch.int32, device=x.device)
     logits = torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device) if want_logits else None
-    wp = (C.c_void_p * n)(*[ptr(w, name="weights[%d]" % i) for i, w in enumerate(weights)])
     bp = None
     if biases is not None:
         bp = (C.c_void_p * n)(*[ptr(b, torch.float32, "biases[%d]" % i) if b is not None else None
                                 for i, b in enumerate(biases)])
     dp = (C.c_int32 * (n + 1))(*dims)
-    check(lib.sp_mlp_forward(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, bp, dp, ptr(u, torch.float32, "u"),
-                             ptr(policy, torch.float32, "policy_out"), ptr(action, torch.int32, "action_out"),
-                             ptr(logits), batch, HEADS[head], mask_size, stream_ptr()))
+    if packed is not None:
+        check(lib.sp_mlp_forward_packed(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, ptr(packed.buffer), bp, dp,
+                                        ptr(u, torch.float32, "u"), ptr(policy, torch.float32, "policy_out"),
+                                        ptr(action, torch.int32, "action_out"), ptr(logits), batch, HEADS[head],
+                                        mask_size, stream_ptr()))
+    else:
+        wp = (C.c_void_p * n)(*[ptr(w, name="weights[%d]" % i) for i, w in enumerate(weights)])
+        check(lib.sp_mlp_forward(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, bp, dp, ptr(u, torch.float32, "u"),
+                                 ptr(policy, torch.float32, "policy_out"), ptr(action, torch.int32, "action_out"),
+                                 ptr(logits), batch, HEADS[head], mask_size, stream_ptr()))
     out = (policy, action)
     return out + (logits,) if want_logits else out
 

@@ -140,3 +140,32 @@ def test_mlp_argument_errors(L):
     assert call(mask=4) == -5
     assert call(act=p) == -1  # action without u
     assert call(ws=(C.c_void_p * 2)(p, None)) == -1
+
+
+def test_packed_mlp_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x6000)
+    dims = lambda *d: (C.c_int32 * len(d))(*d)
+    assert lib.sp_mlp_packed_bytes(4, dims(32, 256, 256, 256, 3)) == 4 * 4096 + 2 * 131072 + 8192
+    assert lib.sp_mlp_packed_bytes(3, dims(128, 256, 256, 64)) == 4 * 8 * 4096 + 131072 + 8192
+    assert lib.sp_mlp_packed_bytes(3, dims(32, 128, 256, 3)) == 0
+    assert lib.sp_mlp_packed_bytes(2, dims(32, 256, 3)) == 0
+    assert lib.sp_mlp_packed_bytes(6, dims(32, 256, 256, 256, 256, 256, 3)) == 0
+    assert lib.sp_mlp_packed_bytes(4, None) == 0
+    w = (C.c_void_p * 4)(p, p, p, p)
+    d = dims(32, 256, 256, 256, 3)
+    assert lib.sp_mlp_pack_weights(1, 4, w, d, None, 1 << 20, None) == -1
+    assert lib.sp_mlp_pack_weights(0, 4, w, d, p, 1 << 20, None) == -4
+    assert lib.sp_mlp_pack_weights(1, 4, w, d, p, 1000, None) == -5 and "must hold" in _err(L)
+    assert lib.sp_mlp_pack_weights(1, 4, w, dims(32, 256, 128, 256, 3), p, 1 << 20, None) == -6
+    assert lib.sp_mlp_pack_weights(1, 4, (C.c_void_p * 4)(p, None, p, p), d, p, 1 << 20, None) == -1
+    call = lambda dtype=1, x=p, n=4, pk=p, dd=d, u=None, pol=p, act=None, logits=None, batch=8, head=1, mask=0: \
+        lib.sp_mlp_forward_packed(dtype, x, n, pk, None, dd, u, pol, act, logits, batch, head, mask, None)
+    assert call(dtype=0) == -4
+    assert call(pk=None) == -1
+    assert call(batch=0) == -2
+    assert call(act=p) == -1                                        # action without u
+    assert call(dd=dims(32, 256, 64, 256, 3)) == -6                 # a hidden width other than 256
+    assert call(dd=dims(32, 256, 256, 256, 64)) == -6 and "16 outputs" in _err(L)     # wide head, no mask
+    assert call(dd=dims(32, 256, 256, 256, 64), mask=3, logits=p) == -6               # wide masked head with logits
+    assert call(mask=4) == -5

@@ -28,10 +28,15 @@ def make_problem(rng, batch, dims, dtype):
     return x, ws, u
 
 
-def check(LY, x, ws, u, dtype, head="softmax_regret_matching", mask=0, biases=None):
+def check(LY, x, ws, u, dtype, head="softmax_regret_matching", mask=0, biases=None, packed=False):
     t = TORCH[dtype]
     bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
-    policy, action, logits = LY.mlp_forward(dev(x, t), [dev(w, t) for w in ws], bd, head, dev(u), mask, True)
+    wd = [dev(w, t) for w in ws]
+    pk = None
+    if packed:
+        pk = LY.pack_weights(wd)
+        assert pk is not None and pk.buffer.numel() == LY.packed_bytes([x.shape[1]] + [w.shape[0] for w in ws])
+    policy, action, logits = LY.mlp_forward(dev(x, t), wd, bd, head, dev(u), mask, True, packed=pk)
     policy, action, logits = host(policy), host(action), host(logits)
     want_p, _, want_l = olayers.mlp_forward(x, ws, biases, HEAD_CODE[head], u, None, mask or None)
     # hidden activations are rounded to the storage dtype before they feed the next MFMA: f16 keeps
@@ -153,3 +158,71 @@ def test_masked_head_without_logits(LY, dtype, batch, dims, head, mask):
     assert (policy[:, mask:] == 0).all() and np.abs(policy.sum(axis=1) - 1).max() < 1e-5
     assert ogemm.rel_frobenius(policy, want_p) < 2e-4 and ogemm.rel_frobenius(policy, host(full_p)) < 2e-4
     assert (action == orow.discrete_sampling(policy, u)).all() and (action < mask).all() and (action >= 0).all()
+
+
+@pytest.mark.parametrize("dims,head,mask,batch,dtype,with_bias", [
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 16384, "f16", False),     # BASELINE config 3
+    ([32, 256, 256, 256, 3], "softmax", 0, 1, "bf16", False),                        # a single row
+    ([32, 256, 256, 3], "softmax_regret_matching", 0, 100, "f16", True),             # three layers
+    ([32, 256, 256, 256, 256, 5], "softmax_regret_matching", 0, 333, "bf16", True),  # five layers: refills into both register sets
+    ([48, 256, 256, 16], "regret_matching", 0, 130, "bf16", False),                  # two first-layer k-steps, K0 not a multiple of 32
+    ([64, 256, 256, 256, 256, 9], "softmax", 7, 640, "f16", True),                   # two first-layer k-steps, five layers, masked head with logits
+    ([128, 256, 256, 256, 10], "softmax", 7, 300, "f16", True),                      # eight first-layer k-steps (zero-padded K0)
+    ([256, 256, 256, 8], "regret_matching", 5, 130, "f16", False),                   # a full-width first layer, three layers
+    ([256, 256, 256, 256, 256, 16], "softmax", 0, 64, "bf16", True),                 # full-width first layer, five layers, widest head
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 20000, "f16", False),     # more workgroups than compute units
+])
+def test_packed_weights_kernel(LY, dims, head, mask, batch, dtype, with_bias):
+    """The kernel that streams pre-packed weights straight into registers (sp_mlp_pack_weights +
+    sp_mlp_forward_packed) against the oracle, and against sp_mlp_forward on the row-major weights."""
+    announce("mlp packed %s head=%s mask=%d batch=%d %s bias=%s" % (dims, head, mask, batch, dtype, with_bias))
+    rng = np.random.default_rng(sum(dims) + batch + 1)
+    x, ws, u = make_problem(rng, batch, dims, dtype)
+    biases = None
+    if with_bias:
+        biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
+        biases[1] = None
+    policy, action = check(LY, x, ws, u, dtype, head, mask, biases, packed=True)
+    t = TORCH[dtype]
+    bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
+    plain_p, plain_a = LY.mlp_forward(dev(x, t), [dev(w, t) for w in ws], bd, head, dev(u), mask)
+    assert ogemm.rel_frobenius(policy, host(plain_p)) < 2e-4
+    assert (action != host(plain_a)).mean() < 1e-3      # same uniforms, policies equal to rounding
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_packed_masked_head_without_logits(LY, dtype):
+    """A 64-wide output layer under a 3-column mask (the reference's shape for a 3-action game) on the packed
+    kernel: only the valid columns are computed, the rest of each policy row is exact zeros inside sentinels."""
+    announce("mlp packed masked head, no logits " + dtype)
+    batch, dims, mask = 4100, [32, 256, 256, 256, 64], 3
+    rng = np.random.default_rng(77)
+    x, ws, u = make_problem(rng, batch, dims, dtype)
+    t = TORCH[dtype]
+    xd, wd, ud = dev(x, t), [dev(w, t) for w in ws], dev(u)
+    pk = LY.pack_weights(wd)
+    buf = torch.full((64 + batch * 64 + 64,), -9.0, dtype=torch.float32, device="cuda")
+    policy_t = buf[64:64 + batch * 64].view(batch, 64)
+    action_t = torch.full((batch,), -1, dtype=torch.int32, device="cuda")
+    LY.mlp_forward(xd, None, None, "softmax", ud, mask, False, policy_out=policy_t, action_out=action_t, packed=pk)
+    raw = host(buf)
+    assert (raw[:64] == -9).all() and (raw[-64:] == -9).all()
+    policy, action = raw[64:-64].reshape(batch, 64), host(action_t)
+    want_p, _, _ = olayers.mlp_forward(x, ws, None, HEAD_CODE["softmax"], u, dtype, mask)
+    assert (policy[:, mask:] == 0).all() and np.abs(policy.sum(axis=1) - 1).max() < 1e-5
+    assert ogemm.rel_frobenius(policy, want_p) < 2e-4
+    assert (action == orow.discrete_sampling(policy, u)).all() and (action < mask).all() and (action >= 0).all()
+    # the logits of a wide masked layer are more than the packed kernel computes: the call says so
+    from ml import _lib
+    with pytest.raises(_lib.SpiralError, match="UNSUPPORTED"):
+        LY.mlp_forward(xd, None, None, "softmax", ud, mask, True, packed=pk)
+
+
+def test_packing_is_refused_for_other_stacks(LY):
+    announce("mlp packed: unsupported stacks")
+    t = torch.float16
+    mk = lambda dims: [torch.zeros((o, i), dtype=t, device="cuda") for i, o in zip(dims[:-1], dims[1:])]
+    assert LY.pack_weights(mk([32, 64, 64, 3])) is None                  # hidden width other than 256
+    assert LY.pack_weights(mk([32, 256, 3])) is None                     # two layers
+    assert LY.pack_weights(mk([32] + [256] * 6 + [3])) is None           # deeper than the packed kernel goes
+    assert LY.packed_bytes([32, 256, 256, 256, 3]) == 4 * 4096 + 2 * 131072 + 8192
