@@ -256,6 +256,16 @@ int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream);
 int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes, void* stream);
 int64_t sp_reduce_workspace_bytes(void);
 
+/* sp_reduce_sum for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
+ * partial sums and the ticket counters live in a 24.25 KiB array inside the library's own device image, one copy
+ * per GPU, kept until the process ends; the call allocates nothing and uses no memset.  Same kernel, same grid and
+ * therefore bit-identical results to sp_reduce_sum.  n must not exceed sp_reduce_sum_static_max_n() (2^36
+ * elements), else SP_ERR_SHAPE.  All calls on one GPU share the array: calls that may overlap in time (different
+ * streams, different threads) race and must be serialised by the caller. */
+int sp_reduce_sum_static(int dtype, const void* x, void* out, int64_t n, void* stream);
+int64_t sp_reduce_sum_static_max_n(void);
+
 /* to[a][c][b] = from[a][b][c] for 4-byte elements.  Replaces `grid_transpose_snd`
  * (ml/primitives.spi:36-112, test5 :1078-1088). */
 int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int64_t c, void* stream);

@@ -5,6 +5,8 @@
 // grid_transpose_snd (:36-112).
 #include "common.h"
 
+#include <mutex>
+
 namespace sp {
 
 typedef __attribute__((ext_vector_type(4))) float f32x4;
@@ -119,6 +121,11 @@ __global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restr
         total += __hip_atomic_load(partial + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     total = block_sum(total, slots);
     if (threadIdx.x == 0) out[0] = total;
+}
+
+// Sets `count` 32-bit words to zero (a kernel rather than a memset so that callers may record it into a graph).
+__global__ __launch_bounds__(EW_THREADS) void clear_words_kernel(unsigned* p, int count) {
+    for (int i = threadIdx.x; i < count; i += EW_THREADS) p[i] = 0u;
 }
 
 // to[a][c][b] = from[a][b][c]; 64x64 tiles through LDS, padded by one word per row so that the
@@ -243,6 +250,59 @@ extern "C" int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, voi
     int rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
     return run_reduce_dtype(dtype, x, out, n, workspace, (hipStream_t)stream);
+}
+
+// ---- the sum for callers that cannot allocate: scratch memory inside the library's own image ----
+// One copy of this array exists on every GPU the library runs on, for the life of the process.  Host code must not
+// use the name as an address (it is a host-side stand-in for the device symbol): the per-device address comes from
+// hipGetSymbolAddress, once per device, and everything below uses that pointer.
+static __device__ __align__(256) unsigned char scratch[REDUCE_SCRATCH_BYTES];
+
+static int static_scratch(void** out) {
+    static std::mutex lock;
+    static void* address[64] = {nullptr};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(SP_ERR_DEVICE, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(SP_ERR_DEVICE, "sp_reduce_sum_static: device index %d out of range", dev);
+    std::lock_guard<std::mutex> guard(lock);
+    if (address[dev] == nullptr) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));   // with device `dev` current: its copy of the array
+        if (e != hipSuccess || p == nullptr)
+            return fail(SP_ERR_DEVICE, "sp_reduce_sum_static: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+        address[dev] = p;
+    }
+    *out = address[dev];
+    return SP_OK;
+}
+
+extern "C" int64_t sp_reduce_sum_static_max_n(void) { return (int64_t)1 << 36; }
+
+extern "C" int sp_reduce_sum_static(int dtype, const void* x, void* out, int64_t n, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    if (n <= 0) return fail(SP_ERR_SHAPE, "sp_reduce_sum_static: n must be positive");
+    if (n > sp_reduce_sum_static_max_n())
+        return fail(SP_ERR_SHAPE, "sp_reduce_sum_static: n = %lld is beyond the maximum of %lld elements", (long long)n,
+                    (long long)sp_reduce_sum_static_max_n());
+    if (dtype < 0 || dtype > 2)
+        return fail(SP_ERR_DTYPE, "sp_reduce_sum_static: dtype must be 0 (f32), 1 (i32) or 2 (u64), got %d", dtype);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    void* mem = nullptr;
+    rc = static_scratch(&mem);
+    if (rc != SP_OK) return rc;
+    // The array keeps what the last call left in it.  Only the ticket counters have to start at zero (the partial
+    // sums are written before they are read); they are cleared by a kernel, not a memset, so that the call may be
+    // recorded into a graph.
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(EW_THREADS), 0, s,
+                       reinterpret_cast<unsigned*>((unsigned char*)mem + REDUCE_COUNTER_OFFSET),
+                       (int)(REDUCE_COUNTERS * REDUCE_COUNTER_STRIDE / 4));
+    rc = check_launch(__func__);
+    if (rc != SP_OK) return rc;
+    return run_reduce_dtype(dtype, x, out, n, mem, s);
 }
 
 extern "C" int sp_transpose_inner_b32(const void* from, void* to, int64_t a, int64_t b, int64_t c, void* stream) {

@@ -66,6 +66,8 @@ SIGNATURES = {
     "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
     "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),
     "sp_reduce_workspace_bytes": (C.c_int64, []),
+    "sp_reduce_sum_static": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
+    "sp_reduce_sum_static_max_n": (C.c_int64, []),
     "sp_transpose_inner_b32": (C.c_int, [_P, _P, _I64, _I64, _I64, _P]),
     "sp_mlp_forward": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
                                  _I64, _I32, _I32, _P]),
@@ -91,7 +93,7 @@ def load(path=LIB_PATH):
 # Entry points that launch work; their last argument is the stream.
 LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_row_map_f32", "sp_row_map_i32",
                       "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_update_mask",
-                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
+                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_reduce_sum_static", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
                       "sp_mlp_forward_packed"))
 
 

@@ -282,6 +282,15 @@ def reduce_sum(x):
     return out[0]
 
 
+def reduce_sum_static(x, out):
+    """reduce_sum without any allocation: the scratch memory is an array inside the library (sp_reduce_sum_static),
+    the result goes to out[0] of a caller-owned, 16-byte aligned tensor of x's dtype.  Calls on one GPU must not
+    overlap in time."""
+    code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
+    check(lib.sp_reduce_sum_static(code, ptr(x, name="x"), ptr(out, x.dtype, "out"), x.numel(), stream_ptr()))
+    return out
+
+
 def transpose_snd(x, out=None):
     """grid_transpose_snd from to: swap the two innermost dimensions (ml/primitives.spi:107-109)."""
     if x.element_size() != 4 or x.dim() < 2:
