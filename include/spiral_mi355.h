@@ -229,17 +229,43 @@ int sp_row_binarize(const float* x, uint32_t* out, int64_t rows, int64_t cols, u
  * produces, :131-132); winners (mask[e] != 0) keep their value, every other member is redrawn as
  * (normals[r, e] * max(std, noise) + mean) * decay with mean / std taken over the winners of the
  * row (std = biased std * n / (n - 1), 0 for a single winner).  The reference draws `normals`
- * from curand_normal on the fly; here the caller supplies standard normals (rows, ensemble).
+ * from curand_normal on the fly; here the caller supplies standard normals (rows, ensemble), or calls
+ * sp_cem_resample_philox below.
  * `out` may be weights_t.  The reference uses noise 0.1, decay 1 (:76-78).
  */
 int sp_cem_resample(const float* weights_t, const int32_t* mask, const float* normals, float* out, int64_t rows,
                     int64_t ensemble, float noise, float decay, void* stream);
 
 /*
+ * sp_cem_resample with the normals drawn on the device, as the reference does (`random.normal rng`, ml/cem.spi:113,
+ * corecuda/random.spi:85: curand_normal on a Philox4_32_10 state): row r takes the sequence curand_normal yields for
+ * curand_init(seed, subsequence = r, offset), i.e. columns 4 g .. 4 g + 3 are the two Box-Muller pairs of 4-draw
+ * group offset / 4 + g.  `offset` (a multiple of 4) lets successive updates continue the stream.  Which thread
+ * draws for which weight is a property of the reference's launch geometry and its fast sincos, neither of which this
+ * build shares: the mapping above is this build's own and the values are not bit-comparable with the reference's.
+ */
+int sp_cem_resample_philox(const float* weights_t, const int32_t* mask, uint64_t seed, uint64_t offset, float* out,
+                           int64_t rows, int64_t ensemble, float noise, float decay, void* stream);
+
+/*
  * `grid_update_rewards_mask` (ml/cem.spi:92-96): rewards is (ensemble, 2) f32 pairs (reward sum,
  * count); mask[e] = (count ? reward / count : 0) >= average over the ensemble; the pairs are zeroed.
  */
 int sp_cem_update_mask(float* rewards, int32_t* mask, int64_t ensemble, void* stream);
+
+typedef enum { SP_REDUCE_SUM = 0, SP_REDUCE_PROD = 1, SP_REDUCE_MAX = 2, SP_REDUCE_MIN = 3, SP_REDUCE_AVERAGE = 4 } sp_reduce_op;
+typedef enum { SP_MAP_IN_IDENTITY = 0, SP_MAP_IN_SQUARE = 1, SP_MAP_IN_ABS = 2 } sp_map_in;
+typedef enum { SP_MAP_OUT_IDENTITY = 0, SP_MAP_OUT_SQRT = 1 } sp_map_out;
+
+/*
+ * out[r] = map_out(reduce over j of map_in(x[r, j])), x (rows, cols) f32, out (rows,) f32; cols any multiple of 4.
+ * Replaces `row_reduce` of `local_sum` / `local_prod` / `local_max` / `local_min` / `local_average`
+ * (ml/primitives.spi:330-348,523-526), `reduce_2d` and `map_reduce_map_2d map_in neutral f map_out from to`
+ * (ml/primitives.spi:593-660) for the lambdas in the enums above; `grid_map_reduce_map_2d grid sqr 0 (+) sqrt` is the
+ * per-row weight norm of the CEM update (ml/cem.spi:139).  The neutral elements are the reference's (0, 1, -inf, +inf);
+ * `local_length` is cols.  The order of a float sum depends on cols only.
+ */
+int sp_row_reduce_f32(int op, int map_in, int map_out, const float* x, float* out, int64_t rows, int64_t cols, void* stream);
 
 typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID = 3 } sp_map_op;
 

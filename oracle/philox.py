@@ -118,3 +118,24 @@ def draws_per_sampling_node(rows_per_block, cols, threads_per_block=256):
     """32-bit draws one sampling node takes from every thread's generator: 4 per row-iteration."""
     r_per_iter = threads_per_block // (cols // 4)
     return 4 * ((rows_per_block + r_per_iter - 1) // r_per_iter)
+
+
+def curand_normal_rows(rows, cols, seed=CONSTANT_SEED, offset=0):
+    """Standard normals as `curand_normal` (corecuda/random.spi:85) hands them out: row r is the sequence of
+    a Philox state initialised with curand_init(seed, subsequence = r, offset); successive draws come in
+    Box-Muller pairs from two 32-bit words x, y:
+        u = x * 2^-32 + 2^-33,  v = y * (2^-32 * 2 pi) + 2^-33 * 2 pi,  (sqrt(-2 ln u) sin v, sqrt(-2 ln u) cos v)
+    (cuRAND's `_curand_box_muller`, restated from its published header; evaluated in f32).  This is the stream
+    sp_cem_resample_philox draws from.  PARITY UNPINNED against the reference: it assigns draws to weights by its
+    launch geometry and evaluates sin/cos/log with the fast intrinsics of its platform; no output of it exists."""
+    assert cols % 2 == 0 and offset % 4 == 0
+    r = np.repeat(np.arange(rows), cols)
+    j = np.tile(np.arange(cols), rows)
+    x = curand_words(seed, r, offset + (j // 2) * 2).astype(np.float32)
+    y = curand_words(seed, r, offset + (j // 2) * 2 + 1).astype(np.float32)
+    two_pi = np.float32(2.3283064e-10) * np.float32(6.2831855)
+    u = x * np.float32(2.3283064e-10) + np.float32(1.1641532e-10)
+    v = y * two_pi + two_pi * np.float32(0.5)
+    s = np.sqrt(np.float32(-2.0) * np.log(u)).astype(np.float32)
+    out = np.where(j % 2 == 0, s * np.sin(v).astype(np.float32), s * np.cos(v).astype(np.float32))
+    return out.astype(np.float32).reshape(rows, cols)

@@ -69,6 +69,19 @@ def row_sum(x):
     return _f32(x).sum(axis=-1, dtype=np.float64).astype(np.float32)
 
 
+def row_reduce(x, op="sum", map_in="identity", map_out="identity"):
+    """`row_reduce` of `local_sum` / `local_prod` / `local_max` / `local_min` / `local_average`
+    (ml/primitives.spi:330-348) and `map_reduce_map_2d map_in neutral f map_out` (:593-660) along the innermost
+    dimension.  Sums and products accumulate in f64 and are rounded once: compare to a tolerance."""
+    x = _f32(x).astype(np.float64)
+    x = {"identity": x, "square": x * x, "abs": np.abs(x)}[map_in]
+    r = {"sum": x.sum(axis=-1), "prod": x.prod(axis=-1), "max": x.max(axis=-1), "min": x.min(axis=-1),
+         "average": x.sum(axis=-1) / x.shape[-1]}[op]
+    if map_out == "sqrt":
+        r = np.sqrt(r)
+    return r.astype(np.float32)
+
+
 def argmax(x):
     """`local_argmax` (ml/primitives.spi:705-708).  The reference keeps `a` when `a.v > b.v` in a
     butterfly whose operand order is unspecified, so ties are arbitrary there; this build fixes

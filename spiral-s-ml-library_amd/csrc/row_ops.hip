@@ -50,8 +50,8 @@ struct RowArgs {
 // Philox4x32-10 (Salmon et al., SC'11) with cuRAND's counter layout: key = seed, counter =
 // (group, 0, subsequence_lo, subsequence_hi); returns word `word` of the group, mapped to (0, 1]
 // like curand_uniform (corecuda/random.spi:22-32,84).
-__device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigned long long subsequence,
-                                                unsigned long long group, int word) {
+__device__ __forceinline__ void philox_words(unsigned long long seed, unsigned long long subsequence,
+                                             unsigned long long group, unsigned (&w)[4]) {
     unsigned c0 = (unsigned)group, c1 = (unsigned)(group >> 32), c2 = (unsigned)subsequence,
              c3 = (unsigned)(subsequence >> 32);
     unsigned k0 = (unsigned)seed, k1 = (unsigned)(seed >> 32);
@@ -66,8 +66,28 @@ __device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigne
         unsigned n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
         c0 = n0; c1 = n1; c2 = n2; c3 = n3;
     }
-    const unsigned w = word == 0 ? c0 : word == 1 ? c1 : word == 2 ? c2 : c3;
-    return (float)w * 2.3283064e-10f + 1.1641532e-10f;
+    w[0] = c0; w[1] = c1; w[2] = c2; w[3] = c3;
+}
+
+__device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigned long long subsequence,
+                                                unsigned long long group, int word) {
+    unsigned w[4];
+    philox_words(seed, subsequence, group, w);
+    const unsigned v = word == 0 ? w[0] : word == 1 ? w[1] : word == 2 ? w[2] : w[3];
+    return (float)v * 2.3283064e-10f + 1.1641532e-10f;
+}
+
+// Two standard normals from two 32-bit draws, the Box-Muller form of curand_normal (corecuda/random.spi:85):
+// u = x 2^-32 + 2^-33, v = 2 pi (y 2^-32 + 2^-33), (sqrt(-2 ln u) sin v, sqrt(-2 ln u) cos v).  The library's own
+// logf / sincosf: the low bits differ from the fast intrinsics of the reference's platform.
+__device__ __forceinline__ void box_muller(unsigned x, unsigned y, float& n0, float& n1) {
+    const float u = (float)x * 2.3283064e-10f + 1.1641532e-10f;
+    const float v = (float)y * (2.3283064e-10f * 6.2831855f) + (2.3283064e-10f * 6.2831855f * 0.5f);
+    const float s = sqrtf(-2.0f * logf(u));
+    float sn, cs;
+    sincosf(v, &sn, &cs);
+    n0 = s * sn;
+    n1 = s * cs;
 }
 
 // Which (subsequence, 4-word group) the reference's sampling op uses for row r: every thread of
@@ -616,10 +636,13 @@ __global__ __launch_bounds__(ROW_THREADS) void philox_uniforms_kernel(const RowA
 // Cross-entropy-method resampling of one weight position across the ensemble (ml/cem.spi:99-117):
 // the row holds that weight for every ensemble member; winners (mask != 0) keep their value, the
 // others are redrawn from N(mean, max(std, noise)) of the winners' values, times `decay`.
+// z == nullptr: the normals are drawn here -- row r takes the sequence curand_normal yields for (seed, subsequence r)
+// from 4-draw group `group0` on, so columns 4 g .. 4 g + 3 come from group group0 + g.
 template <int T, int C>
 __global__ __launch_bounds__(ROW_THREADS) void cem_kernel(const float* __restrict__ x, const int* __restrict__ mask,
                                                           const float* __restrict__ z, float* __restrict__ out, long rows,
-                                                          int cols, float noise, float decay) {
+                                                          int cols, float noise, float decay, unsigned long long seed,
+                                                          unsigned long long group0) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
     const int l = lane % T;
@@ -640,8 +663,17 @@ __global__ __launch_bounds__(ROW_THREADS) void cem_kernel(const float* __restric
             int4 mv = make_int4(0, 0, 0, 0);
             if (ok[c]) {
                 xv = *reinterpret_cast<const f32x4*>(x + row * (long)cols + col);
-                zv = *reinterpret_cast<const f32x4*>(z + row * (long)cols + col);
                 mv = *reinterpret_cast<const int4*>(mask + col);
+                if (z != nullptr) {
+                    zv = *reinterpret_cast<const f32x4*>(z + row * (long)cols + col);
+                } else {
+                    unsigned w[4];
+                    philox_words(seed, (unsigned long long)row, group0 + (unsigned long long)(col / 4), w);
+                    float n0, n1, n2, n3;
+                    box_muller(w[0], w[1], n0, n1);
+                    box_muller(w[2], w[3], n2, n3);
+                    zv = f32x4{n0, n1, n2, n3};
+                }
             }
             const int m4[4] = {mv.x, mv.y, mv.z, mv.w};
 #pragma unroll
@@ -978,10 +1010,117 @@ extern "C" int sp_cem_resample(const float* weights_t, const int32_t* mask, cons
     const int grid = row_grid(rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
         hipLaunchKernelGGL((cem_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
-                           (hipStream_t)stream, weights_t, mask, normals, out, (long)rows, (int)ensemble, noise, decay);
+                           (hipStream_t)stream, weights_t, mask, normals, out, (long)rows, (int)ensemble, noise, decay,
+                           0ull, 0ull);
     });
     if (rc != SP_OK) return rc;
     return check_launch(__func__);
+}
+
+extern "C" int sp_cem_resample_philox(const float* weights_t, const int32_t* mask, uint64_t seed, uint64_t offset, float* out,
+                                      int64_t rows, int64_t ensemble, float noise, float decay, void* stream) {
+    SP_REQUIRE_PTR(weights_t);
+    SP_REQUIRE_PTR(mask);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, ensemble);
+    if (rc != SP_OK) return rc;
+    if (offset % 4 != 0) return fail(SP_ERR_ARG, "sp_cem_resample_philox: offset must be a multiple of 4 draws, got %llu",
+                                     (unsigned long long)offset);
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    const int t = lanes_per_row(ensemble);
+    const int c = (int)((ensemble + 4 * t - 1) / (4 * t));
+    const int grid = row_grid(rows, t);
+    rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
+        hipLaunchKernelGGL((cem_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
+                           (hipStream_t)stream, weights_t, mask, (const float*)nullptr, out, (long)rows, (int)ensemble, noise,
+                           decay, (unsigned long long)seed, (unsigned long long)(offset / 4));
+    });
+    if (rc != SP_OK) return rc;
+    return check_launch(__func__);
+}
+
+// ---- one reduction per row: out[r] = map_out(reduce over j of map_in(x[r, j])) ----
+// T lanes share a row (any width that is a multiple of 4: a lane walks its 4-column pieces 4 T columns apart), each
+// folds its own elements in order, then the lanes' results meet in a butterfly; the order of a float sum depends on
+// the width only.
+template <int OP>
+__device__ __forceinline__ float reduce_op(float a, float b) {
+    if constexpr (OP == SP_REDUCE_SUM || OP == SP_REDUCE_AVERAGE) return a + b;
+    else if constexpr (OP == SP_REDUCE_PROD) return a * b;
+    else if constexpr (OP == SP_REDUCE_MAX) return fmaxf(a, b);
+    else return fminf(a, b);
+}
+
+template <int T, int OP>
+__global__ __launch_bounds__(ROW_THREADS) void row_reduce_kernel(const float* __restrict__ x, float* __restrict__ out, long rows,
+                                                                 long cols, int map_in, int map_out) {
+    constexpr int ROWS_PER_WAVE = WAVE / T;
+    const float neutral = OP == SP_REDUCE_PROD ? 1.f : OP == SP_REDUCE_MAX ? -__builtin_inff() : OP == SP_REDUCE_MIN ? __builtin_inff() : 0.f;
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int l = lane % T, sub = lane / T;
+    const long wave_id = (long)blockIdx.x * (ROW_THREADS / WAVE) + (threadIdx.x / WAVE);
+    const long n_waves = (long)gridDim.x * (ROW_THREADS / WAVE);
+    for (long row0 = wave_id * ROWS_PER_WAVE; row0 < rows; row0 += n_waves * ROWS_PER_WAVE) {
+        const long row = row0 + sub;
+        float acc = neutral;
+        if (row < rows) {
+            const float* xr = x + row * cols;
+            for (long col = 4 * l; col < cols; col += 4 * T) {
+                const f32x4 v = *reinterpret_cast<const f32x4*>(xr + col);
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    float e = v[k];
+                    if (map_in == SP_MAP_IN_SQUARE) e = e * e;
+                    else if (map_in == SP_MAP_IN_ABS) e = fabsf(e);
+                    acc = reduce_op<OP>(acc, e);
+                }
+            }
+        }
+        acc = group_reduce<T>(acc, [](float a, float b) { return reduce_op<OP>(a, b); });
+        if (OP == SP_REDUCE_AVERAGE) acc = acc / (float)cols;
+        if (map_out == SP_MAP_OUT_SQRT) acc = sqrtf(acc);
+        if (row < rows && l == 0) out[row] = acc;
+    }
+}
+
+template <int OP>
+static int launch_row_reduce(const float* x, float* out, int64_t rows, int64_t cols, int map_in, int map_out, hipStream_t stream) {
+    int t = 1;
+    while (t * 4 < cols && t < 64) t *= 2;
+    const int grid = row_grid(rows, t);
+#define SP_ROW_REDUCE_T(TT)                                                                                             \
+    case TT: hipLaunchKernelGGL((row_reduce_kernel<TT, OP>), dim3(grid), dim3(ROW_THREADS), 0, stream, x, out, (long)rows,  \
+                                (long)cols, map_in, map_out); break;
+    switch (t) {
+        SP_ROW_REDUCE_T(1) SP_ROW_REDUCE_T(2) SP_ROW_REDUCE_T(4) SP_ROW_REDUCE_T(8) SP_ROW_REDUCE_T(16) SP_ROW_REDUCE_T(32)
+        SP_ROW_REDUCE_T(64)
+    }
+#undef SP_ROW_REDUCE_T
+    return check_launch("sp_row_reduce_f32");
+}
+
+extern "C" int sp_row_reduce_f32(int op, int map_in, int map_out, const float* x, float* out, int64_t rows, int64_t cols,
+                                 void* stream) {
+    SP_REQUIRE_PTR(x);
+    if (out == nullptr) return fail(SP_ERR_NULL, "sp_row_reduce_f32: out is NULL");
+    if (rows <= 0 || cols <= 0 || cols % 4 != 0)
+        return fail(SP_ERR_SHAPE, "sp_row_reduce_f32: rows must be positive and cols a positive multiple of 4 (got %lld, %lld)",
+                    (long long)rows, (long long)cols);
+    if (rows > (int64_t)1 << 40 || cols > (int64_t)1 << 40) return fail(SP_ERR_SHAPE, "sp_row_reduce_f32: tensor too large");
+    if (map_in < SP_MAP_IN_IDENTITY || map_in > SP_MAP_IN_ABS) return fail(SP_ERR_ARG, "sp_row_reduce_f32: unknown map_in %d", map_in);
+    if (map_out < SP_MAP_OUT_IDENTITY || map_out > SP_MAP_OUT_SQRT) return fail(SP_ERR_ARG, "sp_row_reduce_f32: unknown map_out %d", map_out);
+    if (op < SP_REDUCE_SUM || op > SP_REDUCE_AVERAGE) return fail(SP_ERR_ARG, "sp_row_reduce_f32: unknown op %d", op);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    hipStream_t s = (hipStream_t)stream;
+    switch (op) {
+        case SP_REDUCE_SUM: return launch_row_reduce<SP_REDUCE_SUM>(x, out, rows, cols, map_in, map_out, s);
+        case SP_REDUCE_PROD: return launch_row_reduce<SP_REDUCE_PROD>(x, out, rows, cols, map_in, map_out, s);
+        case SP_REDUCE_MAX: return launch_row_reduce<SP_REDUCE_MAX>(x, out, rows, cols, map_in, map_out, s);
+        case SP_REDUCE_MIN: return launch_row_reduce<SP_REDUCE_MIN>(x, out, rows, cols, map_in, map_out, s);
+        default: return launch_row_reduce<SP_REDUCE_AVERAGE>(x, out, rows, cols, map_in, map_out, s);
+    }
 }
 
 extern "C" int sp_cem_update_mask(float* rewards, int32_t* mask, int64_t ensemble, void* stream) {

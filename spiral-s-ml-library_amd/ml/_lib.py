@@ -13,6 +13,9 @@ GEMM_RELU, GEMM_FORCE_GENERIC = 0x1, 0x100
  ROW_INCLUSIVE_SCAN, ROW_EXCLUSIVE_SCAN) = range(8)
 PHILOX_BLOCK, PHILOX_GRID, PHILOX_GATHER, PHILOX_LAYER = 0, 1, 2, 3
 MAP_COPY, MAP_RELU, MAP_TANH, MAP_SIGMOID = 0, 1, 2, 3
+REDUCE_SUM, REDUCE_PROD, REDUCE_MAX, REDUCE_MIN, REDUCE_AVERAGE = 0, 1, 2, 3, 4
+MAP_IN_IDENTITY, MAP_IN_SQUARE, MAP_IN_ABS = 0, 1, 2
+MAP_OUT_IDENTITY, MAP_OUT_SQRT = 0, 1
 HEAD_NONE, HEAD_SOFTMAX, HEAD_REGRET_MATCHING, HEAD_SOFTMAX_RM = 0, 1, 2, 3
 
 ERROR_NAMES = {0: "SP_OK", -1: "SP_ERR_NULL", -2: "SP_ERR_SHAPE", -3: "SP_ERR_ALIGN", -4: "SP_ERR_DTYPE",
@@ -61,7 +64,9 @@ SIGNATURES = {
     "sp_philox_uniforms": (C.c_int, [C.POINTER(PhiloxConfig), _P, _I64, _I64, _P]),
     "sp_row_get_prob": (C.c_int, [C.c_int, _P, _P, _P, _I64, _I64, _I32, _P]),
     "sp_cem_resample": (C.c_int, [_P, _P, _P, _P, _I64, _I64, C.c_float, C.c_float, _P]),
+    "sp_cem_resample_philox": (C.c_int, [_P, _P, C.c_uint64, C.c_uint64, _P, _I64, _I64, C.c_float, C.c_float, _P]),
     "sp_cem_update_mask": (C.c_int, [_P, _P, _I64, _P]),
+    "sp_row_reduce_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, _P, _P, _I64, _I64, _P]),
     "sp_row_binarize": (C.c_int, [_P, _P, _I64, _I64, C.c_uint32, _P]),
     "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
     "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),
@@ -92,7 +97,8 @@ def load(path=LIB_PATH):
 
 # Entry points that launch work; their last argument is the stream.
 LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_row_map_f32", "sp_row_map_i32",
-                      "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_update_mask",
+                      "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_resample_philox",
+                      "sp_row_reduce_f32", "sp_cem_update_mask",
                       "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_reduce_sum_static", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
                       "sp_mlp_forward_packed"))
 

@@ -1146,6 +1146,20 @@ def matmul_ensemble(cba, x):
     return BlockMatmul(x, apply("ensemble", weights))
 
 
+@_curried
+def matmul_ensemble_with_adjoint(cba, x):
+    """`matmul_ensemble_with_adjoint (c, b, a) x` (ml/layers.spi:472-479): the E weight matrices (E, out, in) in the
+    weights arena under the key "weights" AND their transposed dual ((out, in), E) in the weight-adjoint arena, the
+    pair under the key "cem_weight_layer_dual" -- the two tensors the CEM update transposes between
+    (`grid_transpose weights transposed_weights`, ml/cem.spi:131-146).  The product reads the first of the pair."""
+    c, b, a = cba
+    dtype = _input_dtype(x)
+    dual = key_graph("cem_weight_layer_dual",
+                     pair(key_graph("weights", Layer(weight_id(), (c, a, b), weight_init, dtype)),
+                          Layer(weight_adjoint_id(), (a, b, c), None, dtype)))
+    return BlockMatmul(x, apply("ensemble", fst_(dual)))
+
+
 def _input_dtype(x):
     return get_dim({}, x).dtype
 

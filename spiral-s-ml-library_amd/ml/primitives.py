@@ -232,22 +232,108 @@ def cem_update_rewards_mask(rewards, mask=None):
     return mask
 
 
-def cem(transposed_weights, mask, normals=None, noise=0.1, decay=1.0, out=None, generator=None):
+def cem(transposed_weights, mask, normals=None, noise=0.1, decay=1.0, out=None, generator=None, rng=None):
     """`cem rng transposed_weights model` (ml/cem.spi:99-117), in place by default like the reference:
     every row holds one weight position across the ensemble; the members outside `mask` are redrawn from the
-    winners' mean and spread.  `normals` (same shape) defaults to fresh standard normals."""
+    winners' mean and spread.  `rng=(seed, offset)` draws the normals on the device like the reference does
+    (curand_normal on Philox4_32_10, row r = subsequence r, `offset` draws in; sp_cem_resample_philox); otherwise
+    `normals` (same shape) is used, which defaults to fresh standard normals from torch."""
     rows, cols = _rows_cols(transposed_weights)
     if mask.shape != (cols,):
         raise ValueError("one mask entry per ensemble member expected")
+    if out is None:
+        out = transposed_weights
+    if rng is not None:
+        if normals is not None:
+            raise ValueError("give normals or rng, not both")
+        seed, offset = rng
+        check(lib.sp_cem_resample_philox(ptr(transposed_weights, torch.float32, "transposed_weights"),
+                                         ptr(mask, torch.int32, "mask"), seed, offset, ptr(out, torch.float32, "out"),
+                                         rows, cols, noise, decay, stream_ptr()))
+        return out
     if normals is None:
         normals = torch.randn(transposed_weights.shape, generator=generator, device=transposed_weights.device,
                               dtype=torch.float32)
-    if out is None:
-        out = transposed_weights
     check(lib.sp_cem_resample(ptr(transposed_weights, torch.float32, "transposed_weights"), ptr(mask, torch.int32, "mask"),
                               ptr(normals, torch.float32, "normals"), ptr(out, torch.float32, "out"), rows, cols, noise,
                               decay, stream_ptr()))
     return out
+
+
+_REDUCE_OPS = {"sum": _lib.REDUCE_SUM, "+": _lib.REDUCE_SUM, "prod": _lib.REDUCE_PROD, "*": _lib.REDUCE_PROD,
+               "max": _lib.REDUCE_MAX, "min": _lib.REDUCE_MIN, "average": _lib.REDUCE_AVERAGE}
+_MAP_IN = {"identity": _lib.MAP_IN_IDENTITY, "id": _lib.MAP_IN_IDENTITY, "square": _lib.MAP_IN_SQUARE,
+           "sqr": _lib.MAP_IN_SQUARE, "abs": _lib.MAP_IN_ABS}
+_MAP_OUT = {"identity": _lib.MAP_OUT_IDENTITY, "id": _lib.MAP_OUT_IDENTITY, "sqrt": _lib.MAP_OUT_SQRT}
+
+
+def row_reduce(x, op="sum", map_in="identity", map_out="identity", out=None):
+    """One reduction along the innermost dimension: out[...] = map_out(reduce_j map_in(x[..., j])) (sp_row_reduce_f32).
+    `row_reduce` of the `local_*` reductions (ml/primitives.spi:330-348,523-526) and `reduce_2d` /
+    `map_reduce_map_2d` (:593-660); the inner dimension may be any multiple of 4."""
+    rows, cols = _rows_cols(x) if x.dim() >= 2 else (1, x.numel())
+    if out is None:
+        out = torch.empty(x.shape[:-1] if x.dim() >= 2 else (1,), dtype=torch.float32, device=x.device)
+    if out.numel() != rows:
+        raise ValueError("The first dimension of the input has to equal the dimension of the output in the reduce_2d kernel.")
+    check(lib.sp_row_reduce_f32(_REDUCE_OPS[op], _MAP_IN[map_in], _MAP_OUT[map_out], ptr(x, torch.float32, "x"),
+                                ptr(out, torch.float32, "out"), rows, cols, stream_ptr()))
+    return out
+
+
+def local_sum(x):
+    """row_reduce local_sum (ml/primitives.spi:338)."""
+    return row_reduce(x, "sum")
+
+
+def local_prod(x):
+    """row_reduce local_prod (ml/primitives.spi:344)."""
+    return row_reduce(x, "prod")
+
+
+def local_max(x):
+    """row_reduce local_max (ml/primitives.spi:346)."""
+    return row_reduce(x, "max")
+
+
+def local_min(x):
+    """row_reduce local_min (ml/primitives.spi:348)."""
+    return row_reduce(x, "min")
+
+
+def local_average(x):
+    """row_reduce local_average (ml/primitives.spi:342): local_sum / local_length."""
+    return row_reduce(x, "average")
+
+
+def local_length(x):
+    """local_length (ml/primitives.spi:340): the extent of the innermost dimension."""
+    return x.shape[-1]
+
+
+def map_reduce_map_2d(map_in, neutral_element, f, map_out, from_, to=None):
+    """`map_reduce_map_2d map_in neutral_element f map_out from to` (ml/primitives.spi:647-651) for the named
+    lambdas: map_in in {"id", "sqr", "abs"}, f in {"+", "*", "max", "min"} with its own neutral element (the
+    argument is checked against it), map_out in {"id", "sqrt"}.  `map_reduce_map_2d("sqr", 0, "+", "sqrt", w_t)`
+    is the per-row weight norm of the CEM update (ml/cem.spi:139)."""
+    neutral = {"+": 0.0, "sum": 0.0, "*": 1.0, "prod": 1.0, "max": float("-inf"), "min": float("inf")}[f]
+    if float(neutral_element) != neutral and not (f == "max" and float(neutral_element) == 0.0 and map_in in ("sqr", "square", "abs")):
+        raise ValueError("the neutral element of %r is %r" % (f, neutral))
+    return row_reduce(from_, f, map_in, map_out, out=to)
+
+
+grid_map_reduce_map_2d = map_reduce_map_2d
+
+
+def reduce_2d(neutral_element, f, from_, to=None):
+    """`reduce_2d neutral_element f from to` (ml/primitives.spi:617-618)."""
+    return map_reduce_map_2d("id", neutral_element, f, "id", from_, to)
+
+
+def reduce_max(x):
+    """`grid_reduce grid 0 max norms` of the CEM update's weight-norm print (ml/cem.spi:140): the largest element of a
+    tensor whose element count is a multiple of 4, as a 0-d tensor (all elements treated as one row)."""
+    return row_reduce(x.reshape(1, -1), "max")[0]
 
 
 def grid_transpose(x, out=None):

@@ -105,6 +105,14 @@ def test_row_argument_errors(L):
     assert lib.sp_row_binarize(p, None, 8, 8, 7, None) == -1
     assert lib.sp_cem_resample(p, p, None, p, 8, 8, 0.1, 1.0, None) == -1
     assert lib.sp_cem_resample(p, p, p, p, 8, 6, 0.1, 1.0, None) == -2
+    assert lib.sp_cem_resample_philox(p, p, 1, 0, None, 8, 8, 0.1, 1.0, None) == -1
+    assert lib.sp_cem_resample_philox(p, p, 1, 6, p, 8, 8, 0.1, 1.0, None) == -5 and "multiple of 4" in _err(L)
+    assert lib.sp_cem_resample_philox(p, p, 1, 0, p, 8, 6, 0.1, 1.0, None) == -2
+    assert lib.sp_row_reduce_f32(0, 0, 0, p, None, 8, 8, None) == -1
+    assert lib.sp_row_reduce_f32(0, 0, 0, p, p, 8, 6, None) == -2
+    assert lib.sp_row_reduce_f32(9, 0, 0, p, p, 8, 8, None) == -5
+    assert lib.sp_row_reduce_f32(0, 5, 0, p, p, 8, 8, None) == -5
+    assert lib.sp_row_reduce_f32(0, 0, 2, p, p, 8, 8, None) == -5
     assert lib.sp_cem_update_mask(p, p, 0, None) == -2
     assert lib.sp_cem_update_mask(None, p, 4, None) == -1
 

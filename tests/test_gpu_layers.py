@@ -120,6 +120,49 @@ def test_batched_ensemble_pass_equals_member_by_member_loop(L):
     assert (want_i < 17).all() and len(np.unique(want_i)) > 5
 
 
+def test_ensemble_with_adjoint_and_the_cem_update(L):
+    """`matmul_ensemble_with_adjoint` keeps every ensemble layer as the pair (weights, transposed dual in the adjoint
+    arena); the product is the one `matmul_ensemble` computes, and the reference's CEM update walks the pair:
+    transpose into the dual, resample the losers there, weight norms, transpose back (ml/cem.spi:120-146)."""
+    from ml import primitives as P
+    announce("layers ensemble with adjoint + CEM update")
+    ensemble = 8
+    def graph(ctor):
+        out = L.pair(L.apply("ensemble", L.input("output_probs", (ensemble, Q, 16, 64))),
+                     L.apply("ensemble", L.input("output_indices", (ensemble, Q, 16), "int")))
+        return L.softmax_and_discrete_sample_(out, L.pipe(L.input("input", (Q, 16, 32)), ctor((ensemble, 32, 64))))
+    m = L.create_model(graph(L.matmul_ensemble_with_adjoint))
+    ref = L.create_model(graph(L.matmul_ensemble))
+    sizes = [x["array"].numel() for x in m.data]
+    assert sizes[L.weight_adjoint_id()] == 64 * 32 * ensemble * 4 and sizes[:2] == [x["array"].numel() for x in ref.data][:2]
+    L.pass_init(m)
+    w, wt = L.key_extract(m, "cem_weight_layer_dual")
+    assert tuple(w.shape) == (ensemble, 64, 32) and tuple(wt.shape) == (64, 32, ensemble)
+    assert w.data_ptr() == L.key_extract(m, "weights").data_ptr()
+    L.key_extract(ref, "weights").copy_(w)
+    xin = fill(L.key_extract(m, "input"), np.random.default_rng(5))
+    L.key_extract(ref, "input").copy_(L.key_extract(m, "input"))
+    L.graph_run_host(m, {"ensemble": ensemble})
+    L.graph_run_host(ref, {"ensemble": ensemble})
+    assert (host(L.key_extract(m, "output_probs")) == host(L.key_extract(ref, "output_probs"))).all()
+    assert (host(L.key_extract(m, "output_indices")) == host(L.key_extract(ref, "output_indices"))).all()
+    # apply_updates (ml/cem.spi:120-146) on the pair
+    w0 = host(w).reshape(ensemble, -1).copy()
+    rewards = dev(np.stack([np.arange(ensemble, dtype=np.float32), np.ones(ensemble, dtype=np.float32)], axis=1))
+    mask = P.cem_update_rewards_mask(rewards)
+    assert host(mask).tolist() == [0, 0, 0, 0, 1, 1, 1, 1] and (host(rewards) == 0).all()
+    w2, wt2 = w.reshape(ensemble, -1), wt.reshape(-1, ensemble)
+    P.grid_transpose(w2, wt2)
+    assert (host(wt2) == w0.T).all()
+    P.cem(wt2, mask, rng=(L._prim.CONSTANT_SEED, 0))
+    norms = P.grid_map_reduce_map_2d("sqr", 0, "+", "sqrt", wt2)
+    max_norm = float(P.reduce_max(norms))
+    P.grid_transpose(wt2, w2)
+    want_t = orow.cem_resample(w0.T.copy(), host(mask), ophilox.curand_normal_rows(64 * 32, ensemble), 0.1, 1.0)
+    assert np.abs(host(w2) - want_t.T).max() < 2e-5 and (host(w2)[4:] == w0[4:]).all()
+    assert abs(max_norm - np.sqrt((want_t.astype(np.float64) ** 2).sum(axis=1)).max()) < 1e-4
+
+
 def test_other_heads_and_maps(L):
     announce("layers heads and maps")
     x = L.input("input", (Q, 8, 32))

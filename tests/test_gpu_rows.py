@@ -320,6 +320,61 @@ def test_cem_update(P, dim, ensemble):
     assert np.abs(got - want1).max() < 1e-6
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 4), (5, 16), (130, 64), (257, 256), (33, 260), (7, 1000), (1, 4096), (3, 5000),
+                                       (70000, 8)])
+def test_row_reduce(P, rows, cols):
+    """`row_reduce` of local_sum / prod / max / min / average and `map_reduce_map_2d` (square -> sum -> sqrt: the
+    weight norms of the CEM update) at widths from one lane per row to rows longer than a wave's chunk."""
+    announce("row reduce %dx%d" % (rows, cols))
+    rng = np.random.default_rng(rows * 7 + cols)
+    x = rng.standard_normal((rows, cols), dtype=np.float32)
+    xd = dev(x)
+    assert (host(P.local_max(xd)) == x.max(axis=1)).all() and (host(P.local_min(xd)) == x.min(axis=1)).all()
+    scale = np.abs(x).sum(axis=1) + 1e-30
+    assert (np.abs(host(P.local_sum(xd)) - orow.row_reduce(x, "sum")) <= 2e-6 * scale).all()
+    assert (np.abs(host(P.local_average(xd)) - orow.row_reduce(x, "average")) <= 2e-6 * scale / cols).all()
+    assert P.local_length(xd) == cols
+    near_one = (1 + 0.01 * x).astype(np.float32)
+    got = host(P.local_prod(dev(near_one)))
+    assert np.allclose(got, orow.row_reduce(near_one, "prod"), rtol=1e-4 + 2e-7 * cols)
+    norms = host(P.map_reduce_map_2d("sqr", 0, "+", "sqrt", xd))
+    assert np.allclose(norms, orow.row_reduce(x, "sum", "square", "sqrt"), rtol=1e-5)
+    assert np.allclose(host(P.row_reduce(xd, "max", "abs")), np.abs(x).max(axis=1), rtol=0, atol=0)
+    assert float(P.reduce_max(dev(norms.copy())) if rows % 4 == 0 else P.reduce_max(xd)) == \
+        (norms.max() if rows % 4 == 0 else x.max())
+    into = torch.full((rows,), -5.0, dtype=torch.float32, device="cuda")
+    assert P.reduce_2d(0, "+", xd, into) is into and (host(into) == host(P.local_sum(xd))).all()
+    with pytest.raises(ValueError, match="neutral element"):
+        P.map_reduce_map_2d("id", 1, "+", "id", xd)
+
+
+@pytest.mark.parametrize("rows,cols", [(64, 16), (1000, 64), (513, 256), (40, 1024)])
+def test_cem_with_device_normals(P, rows, cols):
+    """sp_cem_resample_philox: the normals are curand_normal's Box-Muller pairs of the Philox stream (seed,
+    subsequence = row), restated in oracle.philox.curand_normal_rows; `offset` continues the stream."""
+    announce("cem device normals %dx%d" % (rows, cols))
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols), dtype=np.float32)
+    mask = (rng.random(cols) < 0.4).astype(np.int32)
+    mask[1] = 1
+    z = ophilox.curand_normal_rows(rows, cols, 777, 0)
+    got = host(P.cem(dev(x), dev(mask), rng=(777, 0), noise=0.1, decay=0.5, out=torch.empty((rows, cols), device="cuda")))
+    want = orow.cem_resample(x, mask, z, 0.1, 0.5)
+    assert (got[:, mask != 0] == x[:, mask != 0]).all()
+    assert np.abs(got - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+    # one winner of value 0, noise 1: the redrawn members ARE the normals
+    one = np.zeros(cols, dtype=np.int32); one[0] = 1
+    x0 = x.copy(); x0[:, 0] = 0
+    n0 = host(P.cem(dev(x0), dev(one), rng=(777, 0), noise=1.0, out=torch.empty((rows, cols), device="cuda")))[:, 1:]
+    assert np.abs(n0 - z[:, 1:]).max() < 2e-5
+    assert abs(n0.mean()) < 5 / np.sqrt(n0.size) and abs(n0.std() - 1) < 0.05
+    n8 = host(P.cem(dev(x0), dev(one), rng=(777, 8), noise=1.0, out=torch.empty((rows, cols), device="cuda")))
+    assert (n8[:, 1:cols - 8] == n0[:, 8:cols - 1]).all()     # eight draws in: the same sequence, shifted by eight
+    from ml import _lib
+    with pytest.raises(_lib.SpiralError, match="multiple of 4"):
+        P.cem(dev(x0), dev(one), rng=(777, 6))
+
+
 def test_sampling_edge_cases(P):
     announce("sampling edge cases")
     p = np.zeros((4, 8), dtype=np.float32)

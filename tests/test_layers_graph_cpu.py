@@ -131,3 +131,19 @@ def test_fused_plan_takes_only_the_shapes_the_fused_kernel_runs():
     assert L._fused_plan(stack([24, 256, 64])) is None         # input width not a multiple of 16
     assert L._fused_plan(stack([32, 512, 64])) is None         # wider than 256
     assert L._fused_plan(stack([32, 256, 64], "float")) is None   # f32 graphs run node by node
+
+
+def test_ensemble_with_adjoint_places_the_dual_in_the_adjoint_arena():
+    """`matmul_ensemble_with_adjoint` (ml/layers.spi:472-479): weights (E, out, in) in the weights arena, their dual
+    ((out, in), E) in the third arena, both reachable under "cem_weight_layer_dual", the product as matmul_ensemble's."""
+    e, k, n = 4, 32, 64
+    x = L.pipe(L.input("input", (24, 64, k)), L.matmul_ensemble_with_adjoint((e, k, n)))
+    g = L.softmax_and_discrete_sample(x)
+    plain = L.softmax_and_discrete_sample(L.pipe(L.input("input", (24, 64, k)), L.matmul_ensemble((e, k, n))))
+    assert sizes(g) == sizes(plain)[:2] + [n * k * e * 4]
+    m = L.create_model(g, device="cpu")
+    w, wt = L.key_extract(m, "cem_weight_layer_dual")
+    assert tuple(w.shape) == (e, n, k) and tuple(wt.shape) == (n, k, e)
+    assert w.data_ptr() == L.key_extract(m, "weights").data_ptr()
+    assert wt.data_ptr() == L.model_to_model_ptrs(m)[L.weight_adjoint_id()].data_ptr()
+    assert L.get_dim({}, x).dim == (24, 64, n)

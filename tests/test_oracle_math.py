@@ -228,3 +228,35 @@ def test_cem_resample_closed_forms():
 def test_cem_rewards_mask_by_hand():
     rewards = np.array([[2.0, 1.0], [0.0, 0.0], [9.0, 3.0], [1.0, 2.0]], dtype=np.float32)   # averages 2, 0, 3, 0.5
     assert row_ops.cem_update_rewards_mask(rewards).tolist() == [1, 0, 1, 0]                 # mean 1.375
+
+
+def test_curand_normal_rows_is_box_muller_on_the_pinned_words():
+    """The normals are a fixed function of Philox words that the known-answer vectors pin: for every pair,
+    n0^2 + n1^2 = -2 ln u and atan2(n0, n1) = v (mod 2 pi) with u, v from words 2 i, 2 i + 1 of the row's stream;
+    the sample moments are a standard normal's; `offset` shifts the sequence."""
+    rows, cols = 300, 64
+    z = philox.curand_normal_rows(rows, cols, 99, 0).astype(np.float64)
+    r = np.repeat(np.arange(rows), cols // 2)
+    i = np.tile(np.arange(cols // 2), rows)
+    x = philox.curand_words(99, r, 2 * i).astype(np.float64)
+    y = philox.curand_words(99, r, 2 * i + 1).astype(np.float64)
+    u = x * 2.0 ** -32 + 2.0 ** -33
+    v = 2 * np.pi * (y * 2.0 ** -32 + 2.0 ** -33)
+    n0, n1 = z[:, 0::2].reshape(-1), z[:, 1::2].reshape(-1)
+    assert np.allclose(n0 * n0 + n1 * n1, -2 * np.log(u), rtol=1e-5, atol=1e-6)
+    assert np.allclose(n0, np.sqrt(-2 * np.log(u)) * np.sin(v), atol=3e-6)
+    assert np.allclose(n1, np.sqrt(-2 * np.log(u)) * np.cos(v), atol=3e-6)
+    assert abs(z.mean()) < 5 / np.sqrt(z.size) and abs(z.std() - 1) < 0.02
+    assert abs((np.abs(z) < 1).mean() - 0.6827) < 0.01
+    shifted = philox.curand_normal_rows(rows, cols, 99, 8)
+    assert (shifted[:, :cols - 8] == philox.curand_normal_rows(rows, cols, 99, 0)[:, 8:]).all()
+
+
+def test_row_reduce_by_hand():
+    x = np.array([[1, -2, 3, 0.5], [2, 2, 2, 2]], dtype=np.float32)
+    assert row_ops.row_reduce(x, "sum").tolist() == [2.5, 8.0]
+    assert row_ops.row_reduce(x, "prod").tolist() == [-3.0, 16.0]
+    assert row_ops.row_reduce(x, "max").tolist() == [3.0, 2.0] and row_ops.row_reduce(x, "min").tolist() == [-2.0, 2.0]
+    assert row_ops.row_reduce(x, "average").tolist() == [0.625, 2.0]
+    assert row_ops.row_reduce(x, "sum", "square", "sqrt").tolist() == [np.float32(np.sqrt(14.25)), 4.0]
+    assert row_ops.row_reduce(x, "max", "abs").tolist() == [3.0, 2.0]
