@@ -749,10 +749,13 @@ static int lanes_per_row(long cols) {
     return t;
 }
 
+#ifndef SP_ROW_BLOCKS_PER_CU
+#define SP_ROW_BLOCKS_PER_CU 32     // workgroups per compute unit of the row kernels (a build may override it)
+#endif
 static int row_grid(long rows, int t) {
     const long rows_per_block = (long)(WAVE / t) * (ROW_THREADS / WAVE);
     long blocks = (rows + rows_per_block - 1) / rows_per_block;
-    const long cap = (long)device_cu_count() * 32;  // several rounds of short workgroups: the dispatcher evens out the tail
+    const long cap = (long)device_cu_count() * SP_ROW_BLOCKS_PER_CU;  // several rounds of short workgroups: the dispatcher evens out the tail
     if (blocks > cap) blocks = cap;
     return (int)(blocks < 1 ? 1 : blocks);
 }

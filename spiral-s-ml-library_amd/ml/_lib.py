@@ -5,7 +5,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "libspiral_mi355.so")
+# (SPIRAL_MI355_LIB names another build of the same library, e.g. one with different tuning constants)
+LIB_PATH = os.environ.get("SPIRAL_MI355_LIB") or os.path.join(os.path.dirname(_HERE), "libspiral_mi355.so")
 
 SP_F32, SP_F16, SP_BF16 = 0, 1, 2
 GEMM_RELU, GEMM_FORCE_GENERIC = 0x1, 0x100

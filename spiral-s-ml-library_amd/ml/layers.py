@@ -661,8 +661,10 @@ def graph_run_device(model, ls, indices):
     graph_run(model, ls, indices)
 
 
-def _build_fused_run(model, plan, ls):
-    """The closure graph_run_host calls for a graph that sp_mlp_forward can run: every argument is prepared here."""
+def _build_fused_run(model, plan, ls, static_weights=False):
+    """The closure graph_run_host calls for a graph that sp_mlp_forward can run: every argument is prepared here.
+    static_weights: the caller vouches that the weights stay as they are now; they are then packed once, here, and the
+    runs go to the packed kernel (sp_mlp_forward_packed) when it takes the stack."""
     x_node, w_nodes, top, head = plan
     x = _flat(graph_extract(Model(x_node, model.dims, model.data)))
     ws = [graph_extract(Model(w, model.dims, model.data)) for w in w_nodes]
@@ -687,6 +689,17 @@ def _build_fused_run(model, plan, ls):
     # A run restarts the generator from the same seed (ml/layers.spi:339-344), so the uniforms of a (model, seed)
     # pair are the same in every run: they are drawn once, here.
     check(lib.sp_philox_uniforms(C.byref(rng), args[6], rows, cols, stream_ptr()))
+
+    packed = pack_weights(ws) if static_weights else None
+    if packed is not None and builtins.min(dims[-1], top.size or dims[-1]) <= 16:
+        pargs = args[:3] + (ptr(packed.buffer),) + args[4:]
+        keep = keep + (packed,)
+
+        def run_packed():
+            check(lib.sp_mlp_forward_packed(*pargs, stream_ptr()))
+            return keep
+
+        return run_packed
 
     def run():
         check(lib.sp_mlp_forward(*args, stream_ptr()))
@@ -879,11 +892,19 @@ def _graph_run_batched(model, key, count, ls):
     return loop(model.graph)
 
 
-def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batched=True):
+def weights_changed(model):
+    """Forget what was prepared from the current weights (the packed copy behind `static_weights=True`): call it
+    after writing new values into the weights arena."""
+    model.__dict__.pop("_fused_runs", None)
+
+
+def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batched=True, static_weights=False):
     """Runs the graph for every combination of the key indices in `sizes`, e.g. {"ensemble": 16}
     (ml/layers.spi:336-344).  Uniforms come from the reference's per-thread Philox streams.  A loop over
     one key that only indexes leading dimensions runs as a single batched pass with the same results
-    (`batched=False` keeps the member-by-member loop)."""
+    (`batched=False` keeps the member-by-member loop).  `static_weights=True` says that the weights have not
+    changed since the previous such run (or since `weights_changed(model)`): a fused relu-MLP then keeps a copy
+    of them packed for the faster kernel instead of reading the arena on every run."""
     if fuse and not sizes:
         # The plan of a model does not change between runs: the tensors are views of its arenas and the
         # generator restarts with every run.  It is built once per (model, seed); a call then costs one
@@ -891,7 +912,7 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
         cache = model.__dict__.get("_fused_runs")
         if cache is None:
             cache = model.__dict__["_fused_runs"] = {}
-        entry = cache.get(seed)
+        entry = cache.get((seed, static_weights))
         if entry is not None:
             arenas, run = entry
             data = model.data
@@ -903,8 +924,8 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
                 entry = None    # the model was given other arenas: plan again
         if entry is None:
             plan = _fused_plan(model)
-            run = _build_fused_run(model, plan, create_layer_state(seed)) if plan is not None else False
-            cache[seed] = (tuple(d["array"] for d in model.data), run)
+            run = _build_fused_run(model, plan, create_layer_state(seed), static_weights) if plan is not None else False
+            cache[(seed, static_weights)] = (tuple(d["array"] for d in model.data), run)
             if run:
                 run()
                 return

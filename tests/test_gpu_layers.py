@@ -217,6 +217,21 @@ def test_relu_mlp_graph_runs_fused(L, dtype):
     assert ogemm.rel_frobenius(probs.reshape(-1, 64), want) < 3e-3
     assert (idx.reshape(-1) == orow.discrete_sampling(probs.reshape(-1, 64), u)).all() and (idx < 3).all()
     assert (host(first_hidden.float()) == 7).all() and workspace.numel() > 0     # intermediates were never written
+    # static weights: the same run on the packed kernel; new weights only count after weights_changed()
+    for t in L.graph_extract(m):
+        t.zero_()
+    L.graph_run_host(m, static_weights=True)
+    probs_s, idx_s = (host(t) for t in L.graph_extract(m))
+    assert ogemm.rel_frobenius(probs_s, probs) < 2e-4 and (idx_s != idx).mean() < 1e-3
+    first_w = [t for _, t, _ in L.extract_layers_(m, L.weight_id())][0]
+    first_w.zero_()
+    L.graph_run_host(m, static_weights=True)
+    assert (host(L.graph_extract(m)[0]) == probs_s).all()                        # still the packed copy
+    L.weights_changed(m)
+    L.graph_run_host(m, static_weights=True)
+    assert not (host(L.graph_extract(m)[0]) == probs_s).all()
+    first_w.copy_(torch.from_numpy(ws[0]).to(first_w.dtype))
+    L.weights_changed(m)
     with pytest.raises(Exception):
         L.graph_run_host(m, fuse=False)    # node by node the maps and row ops are f32-only
 
