@@ -6,6 +6,7 @@
 hipcc cross-compiles for gfx950 without a GPU.  The shared library is written next to this file;
 the Python host modules under ml/ load it with ctypes and fail loudly when it is missing.
 """
+import glob
 import os
 import subprocess
 import sys
@@ -17,6 +18,8 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libspiral_mi355.so")
 SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip"]
+# sources whose MFMAs are inline asm: their device assembly is kept and scanned (isa_check.py)
+ASM_MFMA_SOURCES = ["gemm.hip", "mlp.hip", "mlp_packed.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"),
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
          "-Wno-unknown-warning-option",
@@ -39,6 +42,28 @@ def _run(cmd):
     return out
 
 
+def device_asm(src):
+    return os.path.join(OBJ, src.replace(".hip", "") + "-hip-amdgcn-amd-amdhsa-gfx950.s")
+
+
+def check_isa():
+    """Scan the kept device assembly; raises on a vector-ALU write right in front of an MFMA that reads it."""
+    sys.path.insert(0, HERE)
+    try:
+        import isa_check
+    finally:
+        sys.path.pop(0)
+    for src in ASM_MFMA_SOURCES:
+        path = device_asm(src)
+        if not os.path.exists(path):
+            continue
+        hits = isa_check.scan_file(path)
+        if hits:
+            ln, kernel, writer, mfma = hits[0]
+            raise RuntimeError("%s: %d MFMA operand hazards, first at line %d in %s: '%s' then '%s'"
+                               % (path, len(hits), ln, kernel, writer, mfma))
+
+
 def build(force=True, verbose=False):
     """Compile every HIP source and link the shared library.  Returns the library path."""
     os.makedirs(OBJ, exist_ok=True)
@@ -51,13 +76,20 @@ def build(force=True, verbose=False):
         o = os.path.join(OBJ, src.replace(".hip", ".o"))
         if not force and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_header):
             return o
-        out = _run([cc] + FLAGS + ["-c", s, "-o", o])
+        keep = ["-save-temps=obj"] if src in ASM_MFMA_SOURCES else []
+        out = _run([cc] + FLAGS + keep + ["-c", s, "-o", o])
         if verbose and out.strip():
             print(out)
+        if keep:        # of the intermediate files only the device assembly stays
+            stem = os.path.join(OBJ, src.replace(".hip", ""))
+            for tmp in glob.glob(stem + "-hip-*") + glob.glob(stem + "-host-*") + glob.glob(stem + ".hip-hip-*"):
+                if tmp != device_asm(src):
+                    os.remove(tmp)
         return o
 
     with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as ex:
         objs = list(ex.map(compile_one, SOURCES))
+    check_isa()
     _run([cc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs)
     return LIB
 

@@ -110,12 +110,13 @@ __device__ __forceinline__ void static_for(F&& f) {
 //   program order: G = KS0 + 1 + S per-thread loads (inputs, uniform, biases), layer 0's 4 KS0 blocks, then the
 //   queue q = 0 .. QN - 1: layers 1 .. S - 1 (32 blocks each, k-step by k-step), the output layer's 8 blocks;
 //   issue slots:   phase 0 (start-up, while the first data is on its way): PK_SLOTS_START; phase 2 L + 1 (the MFMAs
-//   of layer L): one behind every fourth MFMA; phase 2 L + 2 (layer L's outputs are converted and written):
-//   PK_SLOTS_CONVERT.  (Measured: a load among MFMAs costs the wave ~6 cycles, among the conversions ~40.)
+//   of layer L): one behind every fourth MFMA and PK_SLOTS_TAIL more at its end; phase 2 L + 2 (the last of layer
+//   L's outputs are converted and written): none.  (Measured: a load among MFMAs costs the wave ~6 cycles, among
+//   the conversions ~40.)
 // A block of layer l lands in the registers layer l - 2 multiplied from, so it may go out from phase 2 l - 2 on.
 // Every wait names the exact number of loads issued after the one it needs (the counter runs in order).
 constexpr int PK_SLOTS_START = 8;
-constexpr int PK_SLOTS_CONVERT = 4;
+constexpr int PK_SLOTS_TAIL = 4;      // extra slots in the batch-tile-major end of a layer
 
 template <int KS0, int NL>
 struct PkSched {
@@ -123,7 +124,7 @@ struct PkSched {
     static constexpr int G = KS0 + 1 + S;
     static constexpr int QN = 32 * (S - 1) + 8;
     static constexpr int PHASES = 2 * S + 1;
-    static constexpr int slots(int p) { return p == 0 ? PK_SLOTS_START : (p & 1) ? 4 * (p == 1 ? KS0 : 8) : PK_SLOTS_CONVERT; }
+    static constexpr int slots(int p) { return p == 0 ? PK_SLOTS_START : (p & 1) ? 4 * (p == 1 ? KS0 : 8) + PK_SLOTS_TAIL : 0; }
     static constexpr int allowed(int p) {               // queue entries that may have gone out by the end of phase p
         const int lmax = (p + 2) / 2 < S - 1 ? (p + 2) / 2 : S - 1;
         return lmax == S - 1 ? QN : 32 * lmax;
@@ -136,9 +137,9 @@ struct PkSched {
     static constexpr int issued_at(int p, int s) {      // ... before slot s of phase p
         return first_q(p) + s < first_q(p + 1) ? first_q(p) + s : first_q(p + 1);
     }
-    // loads younger than the blocks of k-step ks of layer L when that k-step starts
-    static constexpr int younger(int L, int ks) {
-        const int issued = G + 4 * KS0 + issued_at(2 * L + 1, 4 * ks);
+    // loads younger than the blocks of k-step ks of layer L at the wait in front of slot `at` of that layer's phase
+    static constexpr int younger(int L, int ks, int at) {
+        const int issued = G + 4 * KS0 + issued_at(2 * L + 1, at);
         const int pos_end = L == 0 ? G + 4 * (ks + 1) : G + 4 * KS0 + 32 * (L - 1) + 4 * ks + 4;
         return issued - pos_end;
     }
@@ -147,7 +148,10 @@ struct PkSched {
     static constexpr bool all_issued = first_q(PHASES) == QN;
 };
 
-template <int DT, int KS0, int NL>
+// PLAIN: the commonest call -- a dense policy of at most 4 columns and an action, no logits, no bias on the output
+// layer -- gets an instantiation that ends in nothing but that head: what follows the last MFMA is fetched cold,
+// once per launch, and every jump over code that does not run is another round trip to the instruction cache.
+template <int DT, int KS0, int NL, bool PLAIN>
 __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) {
     typedef PkSched<KS0, NL> SCH;
     constexpr int S = SCH::S;
@@ -277,68 +281,123 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
     f32x4 acc[4][4];                                         // [batch tile][feature tile]
-    auto mfma_acc = [&](f32x4& c, const u32x4& w, const u32x4& x, bool first) {
+    // The MFMAs are asm (their weight operand is filled by asm loads the compiler must not move or copy), so the
+    // compiler cannot see the wait states one needs after a vector-ALU write of a register it reads: where the
+    // register allocator moves an accumulator with v_mov right in front of the MFMA, the matrix pipe reads the old
+    // value.  WAIT puts two wait states in front (used where the compiler's own vector-ALU work is interleaved; the
+    // build scans the generated code for the pattern everywhere else).
+    auto mfma_acc = [&](f32x4& c, const u32x4& w, const u32x4& x, bool first, auto WAIT_) {
+        constexpr bool wait = decltype(WAIT_)::value != 0;   // (the s_nop has to sit in the MFMA's own asm statement:
+                                                             //  the moves are placed right in front of the statement)
+#define SP_PK_MFMA(PRE, T, C, CONSTRAINT) asm volatile(PRE "v_mfma_f32_16x16x32_" T " %0, %1, %2, " C : CONSTRAINT(c) : "a"(w), "v"(x))
         if (first) {
-            if constexpr (DT == SP_F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=v"(c) : "a"(w), "v"(x));
-            else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=v"(c) : "a"(w), "v"(x));
+            if constexpr (DT == SP_F16 && wait) SP_PK_MFMA("s_nop 1\n\t", "f16", "0", "=v");
+            else if constexpr (DT == SP_F16) SP_PK_MFMA("", "f16", "0", "=v");
+            else if constexpr (wait) SP_PK_MFMA("s_nop 1\n\t", "bf16", "0", "=v");
+            else SP_PK_MFMA("", "bf16", "0", "=v");
         } else {
-            if constexpr (DT == SP_F16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(c) : "a"(w), "v"(x));
-            else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(c) : "a"(w), "v"(x));
+            if constexpr (DT == SP_F16 && wait) SP_PK_MFMA("s_nop 1\n\t", "f16", "%0", "+v");
+            else if constexpr (DT == SP_F16) SP_PK_MFMA("", "f16", "%0", "+v");
+            else if constexpr (wait) SP_PK_MFMA("s_nop 1\n\t", "bf16", "%0", "+v");
+            else SP_PK_MFMA("", "bf16", "%0", "+v");
         }
+#undef SP_PK_MFMA
     };
 
-    // One feature-split layer L: K-steps in order; the activation fragments of the next k-step are read one at a
-    // time behind the first MFMAs; behind every fourth MFMA one weight block of the queue is requested.
+    // One feature-split layer L.  K-steps in order, the activation fragments of the next k-step read one at a time
+    // behind the first MFMAs, a weight block of the queue requested behind every fourth MFMA.  The LAST two k-steps
+    // (the last one, of a layer that has only one) are walked batch tile by batch tile instead: tile bt's sums are
+    // then complete while tiles bt + 1 .. 3 are still being multiplied, and its outputs (bias, relu, rounding) are
+    // converted and written to the other activation buffer one packed word per MFMA, in the matrix pipe's shadow;
+    // only the last tile's conversion stands alone.  The barrier makes the outputs everyone's inputs.
     auto layer = [&](auto L_) {
         constexpr int L = decltype(L_)::value;
         constexpr int KS = L == 0 ? KS0 : 8;
+        constexpr int TAILK = KS >= 2 ? 2 : 1;                // k-steps walked batch tile by batch tile
+        constexpr int HEADK = KS - TAILK;
         constexpr int in_buf = L & 1;
+        constexpr int PHASE = 2 * L + 1;
+        const bool with_bias = (has_bias & (1u << L)) != 0;   // uniform
         u32x4 bf[2][4];
 #pragma unroll
         for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_a(in_buf, bt, 0);
-        static_for<0, KS>([&](auto KS_) {
+        static_for<0, HEADK>([&](auto KS_) {
             constexpr int ks = decltype(KS_)::value;
-            static_assert(SCH::younger(L, ks) >= 0, "a block is requested before the k-step that multiplies it");
-            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SCH::clamp63(SCH::younger(L, ks))) : "memory");
+            static_assert(SCH::younger(L, ks, 4 * ks) >= 0, "a block is requested before the k-step that multiplies it");
+            asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SCH::clamp63(SCH::younger(L, ks, 4 * ks))) : "memory");
             static_for<0, 4>([&](auto T_) {
                 constexpr int t = decltype(T_)::value;
 #pragma unroll
                 for (int bt = 0; bt < 4; ++bt) {
-                    mfma_acc(acc[bt][t], wreg(IC<(L & 1)>{}, ks, t), bf[ks & 1][bt], ks == 0);
-                    if (t == 0 && ks + 1 < KS) bf[(ks + 1) & 1][bt] = read_a(in_buf, bt, ks + 1);
+                    mfma_acc(acc[bt][t], wreg(IC<(L & 1)>{}, ks, t), bf[ks & 1][bt], ks == 0, IC<0>{});
+                    if (t == 0) bf[(ks + 1) & 1][bt] = read_a(in_buf, bt, ks + 1);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                slot(IC<2 * L + 1>{}, IC<4 * ks + t>{});
+                slot(IC<PHASE>{}, IC<4 * ks + t>{});
                 __builtin_amdgcn_sched_barrier(0);
             });
         });
-        // the layer's outputs (bias, relu, rounding) go to the other activation buffer, 16 bytes per (batch tile,
-        // tile pair), a weight block of the queue requested behind every other one; the barrier makes them everyone's inputs.
-        // The s_nops are the wait states between the last MFMA and the first read of its result, which the compiler
-        // does not know about.
-        asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
-        auto convert = [&](auto HAS_BIAS_) {
-            f32x4 bias_r[4];
-            if constexpr (decltype(HAS_BIAS_)::value != 0) {
+        // ---- the end of the layer, batch tile by batch tile ----
+        if constexpr (TAILK == 2) {
+            // fragments of k-step KS - 1 (those of KS - 2 were read behind the MFMAs of the k-step before it, or above)
+            if constexpr (HEADK == 0) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)   // [2 p + h]: features 64 w + 32 p + 8 q + 4 h .. + 3
+                for (int bt = 0; bt < 4; ++bt) bf[1][bt] = read_a(in_buf, bt, 1);
+            } else {
+#pragma unroll
+                for (int bt = 0; bt < 4; ++bt) bf[(KS - 1) & 1][bt] = read_a(in_buf, bt, KS - 1);
+            }
+        }
+        static_assert(SCH::younger(L, KS - 1, 4 * HEADK) >= 0, "a block is requested before the k-step that multiplies it");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(SCH::clamp63(SCH::younger(L, KS - 1, 4 * HEADK))) : "memory");
+        // (two copies, with and without a bias: the test is uniform and made once per layer)
+        auto end_of_layer = [&](auto HAS_BIAS_) {
+            constexpr bool has_b = decltype(HAS_BIAS_)::value != 0;
+            f32x4 bias_r[4];                                  // [2 p + h]: features 64 w + 32 p + 8 q + 4 h .. + 3
+            if constexpr (has_b) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
                     bias_r[i] = *reinterpret_cast<const f32x4*>(lds + PK_BIAS_OFF + L * 1024 + (64 * wave + 32 * (i >> 1) + 8 * q + 4 * (i & 1)) * 4);
             }
-            static_for<0, 8>([&](auto G_) {
-                constexpr int bt = decltype(G_)::value >> 1, p = decltype(G_)::value & 1;
-                f32x4 lo = acc[bt][2 * p], hi = acc[bt][2 * p + 1];
-                if constexpr (decltype(HAS_BIAS_)::value != 0) {
-                    lo += bias_r[2 * p];
-                    hi += bias_r[2 * p + 1];
+            // word E (0..7) of batch tile BT's outputs: group p = E / 4 is the tile pair (2 p, 2 p + 1), one 16-byte write
+            u32x4 cv;
+            auto convert_word = [&](auto BT_, auto E_) {
+                constexpr int bt = decltype(BT_)::value, e = decltype(E_)::value;
+                constexpr int p = e >> 2, tile = 2 * p + ((e >> 1) & 1), r = 2 * (e & 1);
+                float a0 = acc[bt][tile][r], a1 = acc[bt][tile][r + 1];
+                if constexpr (has_b) {
+                    a0 += bias_r[tile][r];
+                    a1 += bias_r[tile][r + 1];
                 }
-                const u32x4 v = {pack_relu2<DT>(lo[0], lo[1]), pack_relu2<DT>(lo[2], lo[3]), pack_relu2<DT>(hi[0], hi[1]),
-                                 pack_relu2<DT>(hi[2], hi[3])};
-                *reinterpret_cast<u32x4*>(lds + (in_buf ^ 1) * PK_ACT_BYTES + pw[p] + bt * 8192) = v;
-                if constexpr ((decltype(G_)::value & 1) != 0) slot(IC<2 * L + 2>{}, IC<(decltype(G_)::value >> 1)>{});
+                cv[e & 3] = pack_relu2<DT>(a0, a1);
+                if constexpr ((e & 3) == 3) *reinterpret_cast<u32x4*>(lds + (in_buf ^ 1) * PK_ACT_BYTES + pw[p] + bt * 8192) = cv;
+            };
+            static_for<0, 4>([&](auto BT_) {
+                constexpr int bt = decltype(BT_)::value;
+                static_for<0, 4 * TAILK>([&](auto M_) {
+                    constexpr int m = decltype(M_)::value;
+                    constexpr int ks = HEADK + m / 4, t = m % 4;
+                    mfma_acc(acc[bt][t], wreg(IC<(L & 1)>{}, ks, t), bf[ks & 1][bt], ks == 0, IC<1>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (bt > 0) {                   // the tile before this one is complete: 8 words over these MFMAs
+                        constexpr int per = 8 / (4 * TAILK);
+                        static_for<0, per>([&](auto I_) { convert_word(IC<bt - 1>{}, IC<per * m + decltype(I_)::value>{}); });
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                    // TAILK + 1 slots per batch tile, numbered in program order (the waits count on it): behind the
+                    // second MFMA, then behind every fourth
+                    if constexpr (m == 1) slot(IC<PHASE>{}, IC<4 * HEADK + bt * (TAILK + 1)>{});
+                    if constexpr (m % 4 == 3) slot(IC<PHASE>{}, IC<4 * HEADK + bt * (TAILK + 1) + 1 + m / 4>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             });
+            // the last tile: the s_nops are the wait states between the last MFMA and the first read of its result,
+            // which the compiler does not know about
+            asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
+            static_for<0, 8>([&](auto E_) { convert_word(IC<3>{}, E_); });
         };
-        if (has_bias & (1u << L)) convert(IC<1>{});           // uniform, once per layer
-        else convert(IC<0>{});
+        if (with_bias) end_of_layer(IC<1>{});
+        else end_of_layer(IC<0>{});
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
     layer(IC<0>{});
@@ -371,8 +430,7 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
     }
     const float* bias = last_bias;
     const int limit = mask_size > 0 ? mask_size : NOUT;
-    // the commonest call first, on the shortest path: a dense policy of at most 4 columns and an action, nothing else
-    if (__builtin_expect(NOUT <= 4 && out.stride == NOUT && out.logits == nullptr && out.action != nullptr && bias == nullptr, 1)) {
+    if constexpr (PLAIN) {
         const float p[4] = {d[0], d[1], d[2], d[3]};
         if (head_ok) head_row4_plain_any(out.head, out.policy, out.action, p, head_row_idx, NOUT, limit, u_row);
     } else {
@@ -414,21 +472,26 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
     }   // (the general tail)
 }
 
-template <int DT, int KS0>
+template <int DT, int KS0, bool PLAIN>
 static const void* pick_packed_kernel_nl(int n_layers) {
     switch (n_layers) {
-        case 3: return (const void*)mlp_packed_kernel<DT, KS0, 3>;
-        case 4: return (const void*)mlp_packed_kernel<DT, KS0, 4>;
-        case 5: return (const void*)mlp_packed_kernel<DT, KS0, 5>;
+        case 3: return (const void*)mlp_packed_kernel<DT, KS0, 3, PLAIN>;
+        case 4: return (const void*)mlp_packed_kernel<DT, KS0, 4, PLAIN>;
+        case 5: return (const void*)mlp_packed_kernel<DT, KS0, 5, PLAIN>;
     }
     return nullptr;
 }
 
+template <int DT, bool PLAIN>
+static const void* pick_packed_kernel_ks(int ks0, int n_layers) {
+    if (ks0 == 1) return pick_packed_kernel_nl<DT, 1, PLAIN>(n_layers);
+    if (ks0 == 2) return pick_packed_kernel_nl<DT, 2, PLAIN>(n_layers);
+    return pick_packed_kernel_nl<DT, 8, PLAIN>(n_layers);
+}
+
 template <int DT>
-static const void* pick_packed_kernel(int ks0, int n_layers) {
-    if (ks0 == 1) return pick_packed_kernel_nl<DT, 1>(n_layers);
-    if (ks0 == 2) return pick_packed_kernel_nl<DT, 2>(n_layers);
-    return pick_packed_kernel_nl<DT, 8>(n_layers);
+static const void* pick_packed_kernel(int ks0, int n_layers, bool plain) {
+    return plain ? pick_packed_kernel_ks<DT, true>(ks0, n_layers) : pick_packed_kernel_ks<DT, false>(ks0, n_layers);
 }
 
 constexpr int PK_MIN_LAYERS = 3, PK_MAX_LAYERS = 5;
@@ -444,7 +507,7 @@ static bool packed_shape_ok(int n_layers, const int32_t* dims) {
 
 namespace {
 struct MlpPackedKernelNames {
-    MlpPackedKernelNames() { register_kernel("mlp_forward_packed", (const void*)mlp_packed_kernel<SP_F16, 1, 4>, 256); }
+    MlpPackedKernelNames() { register_kernel("mlp_forward_packed", (const void*)mlp_packed_kernel<SP_F16, 1, 4, true>, 256); }
 } mlp_packed_kernel_names;
 }  // namespace
 
@@ -530,7 +593,8 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
     a.x = x; a.packed = packed; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.out_stride = dims[n_layers];
     const int ks0 = pk_ks0(dims[0]);
-    const void* kernel = dtype == SP_F16 ? pick_packed_kernel<SP_F16>(ks0, n_layers) : pick_packed_kernel<SP_BF16>(ks0, n_layers);
+    const bool plain = a.nout <= 4 && a.out_stride == a.nout && logits_out == nullptr && action_out != nullptr && a.b[n_layers - 1] == nullptr;
+    const void* kernel = dtype == SP_F16 ? pick_packed_kernel<SP_F16>(ks0, n_layers, plain) : pick_packed_kernel<SP_BF16>(ks0, n_layers, plain);
     rc = ensure_dynamic_lds(kernel, PK_LDS_BYTES);
     if (rc != SP_OK) return rc;
     const long blocks = (batch + PK_ROWS - 1) / PK_ROWS;

@@ -1,0 +1,50 @@
+"""The build's scan for the one hazard the compiler cannot see in the hand-scheduled kernels: a vector-ALU
+write of a register within two wait states of an asm MFMA that reads it."""
+import glob
+import importlib.util
+import os
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "spiral-s-ml-library_amd")
+
+
+def _module():
+    spec = importlib.util.spec_from_file_location("isa_check", os.path.join(PKG, "isa_check.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+LISTING = """
+kernel_a:
+\tv_mov_b64_e32 v[142:143], v[44:45]
+\tv_mov_b64_e32 v[140:141], v[42:43]
+\tv_mfma_f32_16x16x32_f16 v[140:143], a[32:35], v[82:85], v[140:143]
+\tv_add_f32_e32 v116, v110, v120
+\tv_mfma_f32_16x16x32_f16 v[160:163], a[36:39], v[82:85], v[160:163]
+kernel_b:
+\tv_mov_b64_e32 v[140:141], v[42:43]
+\ts_nop 1
+\tv_mfma_f32_16x16x32_f16 v[140:143], a[32:35], v[82:85], v[140:143]
+\tv_accvgpr_write_b32 a32, v7
+\tds_read_b128 v[90:93], v118 offset:33024
+\tv_mfma_f32_16x16x32_bf16 v[140:143], a[32:35], v[82:85], v[140:143]
+\tv_mov_b32_e32 v82, 0
+\tglobal_load_dwordx4 a[48:51], v1, s[4:5] offset:0x400
+\ts_waitcnt lgkmcnt(3)
+\tv_mfma_f32_16x16x32_bf16 v[144:147], a[36:39], v[82:85], 0
+"""
+
+
+def test_scan_finds_writes_inside_the_wait_states_and_only_those():
+    hits = _module().scan(LISTING.splitlines())
+    found = [(kernel, writer.split()[0], writer.split()[1]) for _, kernel, writer, _ in hits]
+    assert found == [("kernel_a", "v_mov_b64_e32", "v[142:143],"), ("kernel_a", "v_mov_b64_e32", "v[140:141],"),
+                     ("kernel_b", "v_accvgpr_write_b32", "a32,")]
+
+
+def test_built_kernels_are_clean():
+    """Whatever device assembly the last build kept has no such pair (the build itself refuses to link otherwise)."""
+    mod = _module()
+    for path in glob.glob(os.path.join(PKG, "build", "*-gfx950.s")):
+        assert mod.scan_file(path) == [], path
