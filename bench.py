@@ -39,6 +39,10 @@ def parse():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain copy of 1 GiB (sp_map_f32 copy: 1 GiB read, 1 GiB written) so that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command holds a kernel of known traffic")
+    ap.add_argument("--calibrate-hbm", action="store_true",
+                    help="instead of the benchmark: time the library's plain copy (sp_map_f32 copy) and its full-tensor "
+                         "sum (sp_reduce_sum, a pure read) on f32 tensors of 64 MiB, 256 MiB and 1 GiB and print one "
+                         "JSON line; what this box sustains, to read the HBM-bound roofline fractions against")
     return ap.parse_args()
 
 
@@ -90,6 +94,29 @@ def best_of(fn, reps):
     return best
 
 
+def calibrate_hbm(steps, warmup):
+    """Copy and read rates of the library's own streaming kernels (HIP-event time per launch)."""
+    import torch
+    from ml._lib import check, lib, ptr, stream_ptr
+    torch.cuda.set_device(0)
+    out = {}
+    ws = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device="cuda")
+    res = torch.empty(4, dtype=torch.float32, device="cuda")
+    for mib in (64, 256, 1024):
+        n = mib * (1 << 20) // 4
+        x = torch.rand(n, dtype=torch.float32, device="cuda")
+        y = torch.empty_like(x)
+        _, ev = time_launches(lambda: check(lib.sp_map_f32(0, ptr(x), ptr(y), n, stream_ptr())), steps, warmup)
+        out["copy_%dMiB" % mib] = {"ms": round(ev, 5), "gbs": round(2 * 4 * n / (ev * 1e-3) / 1e9, 1)}
+        _, ev = time_launches(lambda: check(lib.sp_reduce_sum(0, ptr(x), ptr(res), n, ptr(ws), ws.numel(), stream_ptr())),
+                              steps, warmup)
+        out["read_%dMiB" % mib] = {"ms": round(ev, 5), "gbs": round(4 * n / (ev * 1e-3) / 1e9, 1)}
+        del x, y
+        torch.cuda.empty_cache()
+    print(json.dumps({"hbm_calibration": out, "unit": "GB/s", "peak": PEAK_HBM_GBS, "steps": steps, "warmup": warmup,
+                      "kernels": "sp_map_f32(copy): n bytes read + n written; sp_reduce_sum(f32): n bytes read"}))
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -104,6 +131,9 @@ def main():
 
     global PREWARM_MS
     PREWARM_MS = args.prewarm_ms
+    if args.calibrate_hbm:
+        calibrate_hbm(args.steps, args.warmup)
+        return
     torch.cuda.set_device(0)
     TD = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}
     dev = lambda x, t=None: torch.from_numpy(np.ascontiguousarray(x)).cuda().to(t or torch.from_numpy(x).dtype)
