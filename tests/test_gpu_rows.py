@@ -452,3 +452,38 @@ def test_main_body_writes_the_reference_files(P, golden, tmp_path):
     # the sampled indices of test3 obey the mask (j < 3)
     s3 = mf.convert_case(os.path.join(root, "test3", "b"), ["output_sample_reduce"])["output_sample_reduce"]
     assert s3.shape == (1024,) and (s3 >= 0).all() and (s3 < 3).all()
+
+
+@pytest.mark.parametrize("cols", [8, 64, 256, 1024])
+def test_ties_and_nans_follow_the_stated_rules(P, cols):
+    """The behaviours no reference output pins, held to what the header states: argmax takes the LOWEST index among
+    equal maxima and index 0 for a row of NaNs (on every kernel that computes an argmax), binarize sets a bit for
+    every element that is not <= 0 (a NaN sets it, -0.0 and -inf do not)."""
+    announce("ties and NaNs cols=%d" % cols)
+    rng = np.random.default_rng(cols)
+    rows = 37
+    x = rng.standard_normal((rows, cols), dtype=np.float32)
+    top = x.max(axis=1) + 1
+    first = rng.integers(0, cols // 2, rows)
+    for r in range(rows):                      # the maximum appears at `first`, at the last column and once in between
+        x[r, first[r]] = top[r]
+        x[r, cols - 1] = top[r]
+        x[r, (first[r] + cols - 1) // 2] = top[r]
+    x[5, :] = 2.0                               # a constant row
+    want = first.copy()
+    want[5] = 0
+    assert (orow.argmax(x) == want).all()
+    assert (host(P.argmax(dev(x))) == want).all()
+    u = (1 - rng.random(rows, dtype=np.float32)).astype(np.float32)
+    assert (host(P.row_ops(dev(x), dev(u))["argmax"]) == want).all()
+    nan_rows = np.full((3, cols), np.nan, dtype=np.float32)
+    assert (host(P.argmax(dev(nan_rows))) == 0).all()
+    if cols <= 256:
+        odd = rng.standard_normal((rows, cols), dtype=np.float32)
+        odd[:, 0] = np.nan
+        odd[:, 1] = -0.0
+        odd[:, 2] = -np.inf
+        odd[:, 3] = np.inf
+        modulo = 8
+        got = host(P.binarize(dev(odd), modulo)).view(np.uint32)
+        assert (got == orow.binarize(odd, modulo)).all()
