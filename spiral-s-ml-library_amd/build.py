@@ -20,11 +20,16 @@ LIB = os.path.join(HERE, "libspiral_mi355.so")
 SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip"]
 # sources whose MFMAs are inline asm: their device assembly is kept and scanned (isa_check.py)
 ASM_MFMA_SOURCES = ["gemm.hip", "mlp.hip", "mlp_packed.hip"]
+# Kernel-argument preloading (gfx950): the first 14 dwords of a kernel's leading scalar parameters arrive in
+# registers with the wave instead of through a scalar load at kernel entry (a struct parameter is not preloaded;
+# the kernels that gain from it repeat the fields their first loads need as leading scalars).
+EXTRA_FLAGS = {}
 FLAGS = ["-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"),
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-value",
          "-Wno-unknown-warning-option",
          # the DMA blocks name M0 as clobbered; the compiler notes that M0 is a reserved register, once per use
-         "-Wno-inline-asm"]
+         "-Wno-inline-asm",
+         "-mllvm", "-amdgpu-kernarg-preload-count=14"]
 
 
 def hipcc():
@@ -77,7 +82,7 @@ def build(force=True, verbose=False):
         if not force and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_header):
             return o
         keep = ["-save-temps=obj"] if src in ASM_MFMA_SOURCES else []
-        out = _run([cc] + FLAGS + keep + ["-c", s, "-o", o])
+        out = _run([cc] + FLAGS + EXTRA_FLAGS.get(src, []) + keep + ["-c", s, "-o", o])
         if verbose and out.strip():
             print(out)
         if keep:        # of the intermediate files only the device assembly stays

@@ -151,8 +151,15 @@ struct PkSched {
 // PLAIN: the commonest call -- a dense policy of at most 4 columns and an action, no logits, no bias on the output
 // layer -- gets an instantiation that ends in nothing but that head: what follows the last MFMA is fetched cold,
 // once per launch, and every jump over code that does not run is another round trip to the instruction cache.
+// The leading parameters repeat fields of `a`: this file is built with kernel-argument preloading, which hands the
+// first 14 dwords of scalar parameters to a wave in registers when it starts (a struct is not preloaded), so the
+// addresses the first loads need are there without the ~900-cycle round trip of a scalar load from the argument
+// block; everything else is read from `a` while those loads are in flight.  (`k0_nout`: k0 | nout << 16; stacks with
+// more than three feature-split layers read all their bias pointers from `a` instead, up front as before.)
 template <int DT, int KS0, int NL, bool PLAIN>
-__global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) {
+__global__ __launch_bounds__(256) void mlp_packed_kernel(const void* x_first, const void* packed_first, const float* u_first,
+                                                         const float* b0_first, const float* b1_first, const float* b2_first,
+                                                         int batch_first, unsigned k0_nout, const MlpPackedArgs a) {
     typedef PkSched<KS0, NL> SCH;
     constexpr int S = SCH::S;
     static_assert(SCH::all_issued, "every weight block has an issue slot");
@@ -164,18 +171,14 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
     const int j = lane & 15, q = lane >> 4;
     const long row0 = (long)blockIdx.x * PK_ROWS;
     const u32x4 zero_u4 = {0u, 0u, 0u, 0u};
-    const int K0 = a.k0, NOUT = a.nout;
-    const unsigned char* const x_ptr = (const unsigned char*)a.x;
-    const unsigned char* const packed = (const unsigned char*)a.packed;
-    const long batch = a.batch;
+    const int K0 = (int)(k0_nout & 0xffffu), NOUT = (int)(k0_nout >> 16);
+    const unsigned char* const x_ptr = (const unsigned char*)x_first;
+    const unsigned char* const packed = (const unsigned char*)packed_first;
+    const long batch = batch_first;
     const HeadOut out = HeadOut{a.policy, a.action, a.logits, a.head, a.out_stride};
     const int mask_size = a.mask_size;
-    const float* const u_ptr = a.u;
+    const float* const u_ptr = u_first;
     const float* const last_bias = a.b[S];
-    // every scalar argument is read HERE, in one round trip: a read at the point of use costs a few hundred cycles,
-    // and the wait for it also drains the LDS reads in flight
-    asm volatile("" ::"s"(K0), "s"(NOUT), "s"(x_ptr), "s"(packed), "s"(batch), "s"(out.policy), "s"(out.action), "s"(out.logits),
-                 "s"(out.head), "s"(out.stride), "s"(mask_size), "s"(u_ptr), "s"(last_bias));
 
     // ---- per-thread loads: the workgroup's input rows (16-byte pieces, 4 KS0 per row), the uniform of the row
     //      this lane will finish, one bias value per feature-split layer (feature tid) ----
@@ -200,7 +203,7 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
     unsigned has_bias = 0;                                   // bit l: layer l has a bias (uniform)
 #pragma unroll
     for (int l = 0; l < S; ++l) {
-        const float* b = a.b[l];
+        const float* b = S > 3 ? a.b[l] : l == 0 ? b0_first : l == 1 ? b1_first : b2_first;
         if (b != nullptr) has_bias |= 1u << l;
         const unsigned char* bp = b != nullptr ? (const unsigned char*)(b + tid) : x_ptr;   // always a load: fixed count
         asm volatile("global_load_dword %0, %1, off" : "=v"(bias_in[l]) : "v"(bp) : "memory");
@@ -248,6 +251,9 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const MlpPackedArgs a) 
         if constexpr (SCH::first_q(P) + s_ < SCH::first_q(P + 1)) issue(IC<SCH::first_q(P) + s_>{});
     };
     static_for<0, PK_SLOTS_START>([&](auto S_) { slot(IC<0>{}, S_); });
+    // every other scalar argument is waited for HERE, once, behind the first loads: a read at the point of use costs
+    // a few hundred cycles, and the wait for it also drains the LDS reads in flight
+    asm volatile("" ::"s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(out.stride), "s"(mask_size), "s"(last_bias));
 
     // ---- operand addresses ----
     // activations: row r, 16-byte piece P (of 32) lives in slot (P & 16) | ((P ^ r) & 15) of the row's 512 bytes
@@ -598,7 +604,11 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
     rc = ensure_dynamic_lds(kernel, PK_LDS_BYTES);
     if (rc != SP_OK) return rc;
     const long blocks = (batch + PK_ROWS - 1) / PK_ROWS;
-    void* args[] = {(void*)&a};
+    if (batch > 0x7fffffffll) return fail(SP_ERR_SHAPE, "sp_mlp_forward_packed: batch must be below 2^31");
+    int batch32 = (int)batch;
+    unsigned k0_nout = (unsigned)a.k0 | ((unsigned)a.nout << 16);
+    void* args[] = {(void*)&a.x, (void*)&a.packed, (void*)&a.u, (void*)&a.b[0], (void*)&a.b[1], (void*)&a.b[2], (void*)&batch32,
+                    (void*)&k0_nout, (void*)&a};
     hipError_t e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(256), args, PK_LDS_BYTES, (hipStream_t)stream);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward_packed: launch failed: %s", hipGetErrorString(e));
     return check_launch(__func__);
