@@ -140,7 +140,9 @@ __global__ __launch_bounds__(EW_THREADS) void clear_words_kernel(unsigned* p, in
 }
 
 // to[a][c][b] = from[a][b][c]; 64x64 tiles through LDS, padded by one word per row so that the
-// transposed (column) reads hit 64 different banks.
+// transposed (column) reads hit 64 different banks.  (The reference sizes this tile at run time: `frame_iter`
+// doubles a 32 x 32 minimum under its shared-memory budget, ml/primitives.spi:17-33,56-66; here it is fixed at one
+// wave-width square, which is what 64 banks and 64 lanes ask for.)
 __global__ __launch_bounds__(EW_THREADS) void transpose_kernel(const unsigned* __restrict__ from, unsigned* __restrict__ to,
                                                                long B, long C, long tiles_b, long tiles_c) {
     __shared__ unsigned tile[64][65];

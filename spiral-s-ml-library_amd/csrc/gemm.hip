@@ -871,7 +871,9 @@ static bool use_four_waves(int dtype_in, long N, long K) {
     return dtype_in != SP_F32 && K % 128 == 0 && K <= (1l << 22) && N >= 512;
 }
 
-// Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.  "Fills" is 80 %
+// The counterpart of the reference's tile search (`frame` / `frame_iter`, ml/primitives.spi:17-33, as used by
+// matmul_config_tf32, ml/matmul/run.spi:8-19: tiles doubled from 16 x 16 under the shared-memory budget): a fixed menu
+// of three tiles.  Largest tile whose grid still fills the chip; otherwise the smallest tile that divides the shape.  "Fills" is 80 %
 // of the compute units, except for the four-wave kernel, which does per unit so much more than the 128 x 128 tiles
 // that 9/16 of the units are enough (3072^3 bf16: 144 tiles of 256 x 256 take 56 us, 576 tiles of 128 x 128 76 us; at
 // 128 tiles the two are level, below that the smaller tiles win).

@@ -115,8 +115,14 @@ __device__ __forceinline__ void static_for(F&& f) {
 //   the conversions ~40.)
 // A block of layer l lands in the registers layer l - 2 multiplied from, so it may go out from phase 2 l - 2 on.
 // Every wait names the exact number of loads issued after the one it needs (the counter runs in order).
-constexpr int PK_SLOTS_START = 8;
-constexpr int PK_SLOTS_TAIL = 4;      // extra slots in the batch-tile-major end of a layer
+#ifndef SP_PK_SLOTS_START
+#define SP_PK_SLOTS_START 8
+#endif
+constexpr int PK_SLOTS_START = SP_PK_SLOTS_START;
+#ifndef SP_PK_SLOTS_TAIL
+#define SP_PK_SLOTS_TAIL 4
+#endif
+constexpr int PK_SLOTS_TAIL = SP_PK_SLOTS_TAIL;      // extra slots in the batch-tile-major end of a layer
 
 template <int KS0, int NL>
 struct PkSched {
