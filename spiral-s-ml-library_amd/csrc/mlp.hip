@@ -596,7 +596,13 @@ constexpr int SPLIT_RING_BYTES = SPLIT_STAGES * SPLIT_STAGE_BYTES;
 constexpr int SPLIT_LDS_BYTES = SPLIT_ACT_BYTES + 4 * SPLIT_RING_BYTES;
 
 template <int DT, int KS0>
-__global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
+__global__ __launch_bounds__(256) void mlp_split_kernel(const void* x_first, const void* w0_first, const void* w1_first,
+                                                        const float* b0_first, const float* u_first, int batch_first,
+                                                        unsigned k0_nl_nout, const MlpArgs a) {
+    // (the leading parameters repeat fields of `a`: the library is built with kernel-argument preloading, which hands
+    //  the first dwords of scalar parameters to a wave in registers when it starts, so the first loads do not wait
+    //  for a scalar load from the argument block; k0_nl_nout = k0 | n_layers << 16 | nout << 24)
+    constexpr int ARGS_OFFSET = 48;                  // of `a` inside the kernel's argument block: 5 pointers, 2 ints
     constexpr int C0 = (KS0 + 1) / 2;                // chunks of the first layer
     constexpr bool HALF0 = KS0 == 1;                 // ... which is half a chunk when K0 <= 32
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -609,20 +615,18 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
     // every scalar argument in one round trip; the per-layer pointers in a register table (lane l holds
     // weights[l] and biases[l], picked by v_readlane)
-    const int K0 = a.k0, NL = a.n_layers, NOUT = a.nout;
-    const unsigned char* const x_ptr = (const unsigned char*)a.x;
-    const unsigned char* const w0_ptr = (const unsigned char*)a.w[0];
-    const unsigned char* const w1_ptr = (const unsigned char*)a.w[1];
-    const unsigned char* const b0_ptr = (const unsigned char*)a.b[0];
-    const float* const u_ptr = a.u;
-    const long batch = a.batch;
+    const int K0 = (int)(k0_nl_nout & 0xffffu), NL = (int)((k0_nl_nout >> 16) & 0xffu), NOUT = (int)(k0_nl_nout >> 24);
+    const unsigned char* const x_ptr = (const unsigned char*)x_first;
+    const unsigned char* const w0_ptr = (const unsigned char*)w0_first;
+    const unsigned char* const w1_ptr = (const unsigned char*)w1_first;
+    const unsigned char* const b0_ptr = (const unsigned char*)b0_first;
+    const float* const u_ptr = u_first;
+    const long batch = batch_first;
     const HeadOut out = head_out(a);
     const int mask_size = a.mask_size;
-    asm volatile("" ::"s"(K0), "s"(NL), "s"(NOUT), "s"(x_ptr), "s"(w0_ptr), "s"(w1_ptr), "s"(b0_ptr), "s"(u_ptr), "s"(batch),
-                 "s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(mask_size));
     u32x2 tab_w, tab_b;
     {
-        const unsigned char* args = (const unsigned char*)__builtin_amdgcn_kernarg_segment_ptr();
+        const unsigned char* args = (const unsigned char*)__builtin_amdgcn_kernarg_segment_ptr() + ARGS_OFFSET;
         asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_w) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, w)) : "memory");
         asm volatile("global_load_dwordx2 %0, %1, %2" : "=v"(tab_b) : "v"((lane & 7) * 8), "s"(args + __builtin_offsetof(MlpArgs, b)) : "memory");
     }
@@ -707,6 +711,9 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const MlpArgs a) {
     issue_chunk(IC<1>{});
     issue_chunk(IC<1>{});
     issue_chunk(IC<1>{});
+    // every other scalar argument is waited for HERE, once, behind the first loads (a read at the point of use costs
+    // a few hundred cycles, and the wait for it also drains the LDS reads in flight)
+    asm volatile("" ::"s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(out.stride), "s"(mask_size));
 
     // ---- operand addresses ----
     // weights: tile (p, h), MFMA row j -> stage row R = 32 p + 4 h + R0, R0 = 8 (j / 4) + j % 4; swz(R) does not
@@ -1047,8 +1054,18 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     rc = ensure_dynamic_lds(kernel, lds_bytes);
     if (rc != SP_OK) return rc;
     const long blocks = (batch + rows_per_block - 1) / rows_per_block;
-    void* args[] = {(void*)&a};
-    hipError_t e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
+    hipError_t e;
+    if (split) {
+        if (batch > 0x7fffffffll) return fail(SP_ERR_SHAPE, "sp_mlp_forward: batch must be below 2^31");
+        int batch32 = (int)batch;
+        unsigned k0_nl_nout = (unsigned)a.k0 | ((unsigned)a.n_layers << 16) | ((unsigned)a.nout << 24);
+        void* args[] = {(void*)&a.x, (void*)&a.w[0], (void*)&a.w[1], (void*)&a.b[0], (void*)&a.u, (void*)&batch32,
+                        (void*)&k0_nl_nout, (void*)&a};
+        e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
+    } else {
+        void* args[] = {(void*)&a};
+        e = hipLaunchKernel(kernel, dim3((unsigned)blocks), dim3(threads), args, lds_bytes, (hipStream_t)stream);
+    }
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward: launch failed: %s", hipGetErrorString(e));
     return check_launch(__func__);
 }
