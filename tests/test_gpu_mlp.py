@@ -171,6 +171,9 @@ def test_masked_head_without_logits(LY, dtype, batch, dims, head, mask):
     ([256, 256, 256, 8], "regret_matching", 5, 130, "f16", False),                   # a full-width first layer, three layers
     ([256, 256, 256, 256, 256, 16], "softmax", 0, 64, "bf16", True),                 # full-width first layer, five layers, widest head
     ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 20000, "f16", False),     # more workgroups than compute units
+    ([32, 256, 256, 256, 3], "softmax", 0, 200, "f16", "all"),                        # a bias on every layer
+    ([256, 256, 256, 256, 256, 12], "softmax", 0, 200, "bf16", "all"),
+    ([64, 256, 256, 256, 4], "regret_matching", 0, 77, "f16", "only1"),               # a bias on the second layer alone
 ])
 def test_packed_weights_kernel(LY, dims, head, mask, batch, dtype, with_bias):
     """The kernel that streams pre-packed weights straight into registers (sp_mlp_pack_weights +
@@ -181,7 +184,10 @@ def test_packed_weights_kernel(LY, dims, head, mask, batch, dtype, with_bias):
     biases = None
     if with_bias:
         biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
-        biases[1] = None
+        if with_bias == "only1":
+            biases = [b if l == 1 else None for l, b in enumerate(biases)]
+        elif with_bias != "all":
+            biases[1] = None
     policy, action = check(LY, x, ws, u, dtype, head, mask, biases, packed=True)
     t = TORCH[dtype]
     bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
