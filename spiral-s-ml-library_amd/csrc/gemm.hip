@@ -530,12 +530,23 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
 // every LDS read and every DMA alone between two MFMAs: 128 MFMAs + ~76 other instructions per K-tile.
 // The fragment of the B matrix is the MFMA's first operand: register r of lane l of accumulator tile
 // (tm, tn) holds C[m = 16 tm + l % 16][n = 16 tn + 4 (l / 16) + r].
-template <int DT, int OT>
+// NSA = 3: a ring of three stages for the A tiles next to the two for B -- all 160 KiB of LDS.  The A tile of K-tile
+// kt + 3 is requested in the second half of K-tile kt, so it has two K-tiles to arrive instead of one; B (re-read by
+// every tile row, served by the caches) keeps its lead of one.  For tall shapes whose A panels come straight from
+// HBM (65536 x 1024 x 512: 99.7 -> 97.5 us; most of what that main loop waits for is contention with the other
+// units' stores, which a longer lead does not cure).  The A stage of a K-tile is then a run-time offset (three
+// stages against a loop body of two K-tiles): the eight fragment addresses of A are re-based once per K-tile (8
+// vector adds; the square GEMMs, whose loop does not wait, lose 0.5-2 % to them and stay on NSA = 2).  Within a K-tile the B fetches go out before the A fetches, so that at the boundary
+// "everything but the 8 youngest fetches has landed" is exactly "tile kt + 1 is complete".
+template <int DT, int OT, int NSA = 2>
 __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, const GemmArgs g_rest) {
     SP_GEMM_TAKE_PRELOADED;
     static_assert(DT != SP_F32, "16-bit inputs only");
+    static_assert(NSA == 2 || NSA == 3, "two stages [A][B], or three A stages followed by two B stages");
     constexpr int BM = 256, BN = 256, NW = 4, ES = 2;
     constexpr int BK = ROW_BYTES / ES;
+    constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+    constexpr int B_BASE3 = 3 * A_BYTES;         // NSA = 3: where the B stages start
     constexpr int STAGE_BYTES = (BM + BN) * ROW_BYTES;
     constexpr int NI = (BM + BN) / 8 / NW;      // 16 DMA instructions per wave and K-tile
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
@@ -568,7 +579,9 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
         voff[q] = (unsigned)((q * 8 * NW + r) * K * ES) + chunk;
     }
     auto dma_plain = [&](int q, int stage) {
-        const unsigned d = dstw + (q < 8 ? 0 : BM * ROW_BYTES) + (q & 7) * NW * 8 * ROW_BYTES + stage * STAGE_BYTES;
+        unsigned d = dstw + (q & 7) * NW * 8 * ROW_BYTES;
+        if constexpr (NSA == 3) d += q < 8 ? stage * A_BYTES : B_BASE3 + stage * B_BYTES;
+        else d += (q < 8 ? 0 : BM * ROW_BYTES) + stage * STAGE_BYTES;
         dma_to_lds(q < 8 ? sA : sB, voff[q & 7], d);
     };
 
@@ -587,13 +600,27 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
                 // agree.  With 4 * ks + fq (lanes l and l + 32 two chunks apart) half of the LDS cycles of these reads
                 // were bank conflicts (SQ_LDS_BANK_CONFLICT 8.5 M per 4096^3 launch); with 2 * fq + ks there are none.
                 const int kc = 2 * fq + ks;
-                va[st][ks][t] = st * STAGE_BYTES + lds_offset(wm * 128 + 16 * t + fi, kc);
-                vb[st][ks][t] = st * STAGE_BYTES + BM * ROW_BYTES + lds_offset(wn * 128 + 16 * t + fi, kc);
+                if constexpr (NSA == 3) {       // A: relative to its stage (st is not used); B: its own two stages
+                    va[st][ks][t] = lds_offset(wm * 128 + 16 * t + fi, kc);
+                    vb[st][ks][t] = B_BASE3 + st * B_BYTES + lds_offset(wn * 128 + 16 * t + fi, kc);
+                } else {
+                    va[st][ks][t] = st * STAGE_BYTES + lds_offset(wm * 128 + 16 * t + fi, kc);
+                    vb[st][ks][t] = st * STAGE_BYTES + BM * ROW_BYTES + lds_offset(wn * 128 + 16 * t + fi, kc);
+                }
                 // opaque to the compiler, or it keeps one of them and re-derives the others inside the loop
                 asm volatile("" : "+v"(va[st][ks][t]), "+v"(vb[st][ks][t]));
             }
+    // NSA = 3: the A fragment addresses of the K-tile being read, re-based once per K-tile: [1] (k-step 1 of the
+    // K-tile being multiplied) at the start of a K-tile, [0] (k-step 0 of the next one) at its boundary
+    int vaa[2][4] = {};
+    unsigned a_cur = 0;                          // byte offset of the A stage of the K-tile being multiplied
+    auto rebase_a = [&](int ks, unsigned stage_bytes) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) vaa[ks][t] = va[0][ks][t] + (int)stage_bytes;
+    };
     auto load_a = [&](int st, int ks, int t, u32x4(&fa)[8]) {
-        fa[t] = *reinterpret_cast<const u32x4*>(lds + va[st][ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
+        if constexpr (NSA == 3) fa[t] = *reinterpret_cast<const u32x4*>(lds + vaa[ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
+        else fa[t] = *reinterpret_cast<const u32x4*>(lds + va[st][ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
     };
     auto load_b = [&](int st, int ks, int t, u32x4(&fb)[8]) {
         fb[t] = *reinterpret_cast<const u32x4*>(lds + vb[st][ks][t & 3] + (t >> 2) * 64 * ROW_BYTES);
@@ -643,14 +670,21 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     for (int i = 0; i < 8; ++i)
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[i][j] = zero4;
-    // prologue: tiles 0 and 1 into stages 0 and 1
+    // prologue: tiles 0 and 1 into stages 0 and 1 (NSA = 3: and the A tile 2 into the third A stage; sA then
+    // points at tile 2 and sB at tile 1, what the first boundary expects)
 #pragma unroll
     for (int q = 0; q < NI; ++q) dma_plain(q, 0);
     sA += ROW_BYTES;
     sB += ROW_BYTES;
 #pragma unroll
     for (int q = 0; q < NI; ++q) dma_plain(q, 1);
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NI) : "memory");   // tile 0 has landed
+    if constexpr (NSA == 3) {
+        sA += ROW_BYTES;
+#pragma unroll
+        for (int q = 0; q < 8; ++q) dma_plain(q, 2);
+        rebase_a(0, 0);
+    }
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSA == 3 ? NI + 8 : NI) : "memory");   // tile 0 has landed
     __syncthreads();
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
@@ -660,10 +694,15 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     // row I of k-step 1 of a tile in stage ST: fetches 2 I and 2 I + 1 of the tile after the next go into stage ST
     auto row1 = [&](auto ST_, auto I_) {
         constexpr int ST = decltype(ST_)::value, i = decltype(I_)::value;
-        constexpr int q0 = 2 * i, q1 = 2 * i + 1;     // 0..7: A, 8..15: B
-        constexpr unsigned D0 = (q0 < 8 ? 0 : BM * ROW_BYTES) + (q0 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
-        constexpr unsigned D1 = (q1 < 8 ? 0 : BM * ROW_BYTES) + (q1 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
-        const unsigned char* base = i < 4 ? sA : sB;
+        // 0..7: A, 8..15: B; NSA = 3 sends B first (rows 0..3), then A (rows 4..7)
+        constexpr int q0 = NSA == 3 ? (2 * i + 8) % 16 : 2 * i, q1 = q0 + 1;
+        constexpr unsigned D0 = NSA == 3 ? (q0 < 8 ? 0 : B_BASE3 + ST * B_BYTES) + (q0 & 7) * NW * 8 * ROW_BYTES
+                                         : (q0 < 8 ? 0 : BM * ROW_BYTES) + (q0 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
+        constexpr unsigned D1 = NSA == 3 ? (q1 < 8 ? 0 : B_BASE3 + ST * B_BYTES) + (q1 & 7) * NW * 8 * ROW_BYTES
+                                         : (q1 < 8 ? 0 : BM * ROW_BYTES) + (q1 & 7) * NW * 8 * ROW_BYTES + ST * STAGE_BYTES;
+        const unsigned char* base = q0 < 8 ? sA : sB;
+        // NSA = 3: the A tile of K-tile kt + 3 goes into the A stage K-tile kt has just released (a_cur)
+        const unsigned dw = NSA == 3 && q0 < 8 ? dstw + a_cur : dstw;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             mfma_acc(acc[i][j], fb[1][j], fa[1][i]);
@@ -672,7 +711,7 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
             __builtin_amdgcn_sched_barrier(0);
         }
         mfma4_dma2(acc[i][4], acc[i][5], acc[i][6], acc[i][7], fb[1][4], fb[1][5], fb[1][6], fb[1][7], fa[1][i], voff[q0 & 7],
-                   voff[q1 & 7], base, dstw, std::integral_constant<unsigned, D0>{}, std::integral_constant<unsigned, D1>{});
+                   voff[q1 & 7], base, dw, std::integral_constant<unsigned, D0>{}, std::integral_constant<unsigned, D1>{});
         __builtin_amdgcn_sched_barrier(0);
     };
     // One K-tile in stage ST.  k-step 0 multiplies fragments taken before it and takes those of k-step 1; the
@@ -683,6 +722,8 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     // the last tile repeat the last tile into a stage nobody reads any more: no branch in the loop.
     auto tile = [&](int kt, auto ST_) {
         constexpr int ST = decltype(ST_)::value;
+        const unsigned a_next = a_cur == 2 * A_BYTES ? 0 : a_cur + A_BYTES;
+        if constexpr (NSA == 3) rebase_a(1, a_cur);
         __builtin_amdgcn_s_waitcnt(0xC07F);   // lgkmcnt(0): one wait for all fragments of this k-step instead of one per row
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -694,9 +735,15 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        {
+        if constexpr (NSA == 3) {
+            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // all but the A tile of K-tile kt + 2
+            __syncthreads();
+            sA += kt + 3 < nk ? ROW_BYTES : 0;
+            sB += kt + 2 < nk ? ROW_BYTES : 0;
+            rebase_a(0, a_next);
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
             const int adv = kt + 2 < nk ? ROW_BYTES : 0;
             sA += adv;
             sB += adv;
@@ -710,6 +757,7 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
         row1(ST_, std::integral_constant<int, 5>{});
         row1(ST_, std::integral_constant<int, 6>{});
         row1(ST_, std::integral_constant<int, 7>{});
+        a_cur = a_next;
     };
     for (int kt = 0; kt < nk; kt += 2) {
         tile(kt, std::integral_constant<int, 0>{});
@@ -945,16 +993,37 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
     return launch_tiled_stages<DT, OT, BM, BN, WM, WN, 2>(g, stream);
 }
 
+// The four-wave kernel with a third A stage (see the kernel): when the A panels are not shared enough to come from
+// the caches.
+#ifndef SP_W4_NSA3_MODE
+#define SP_W4_NSA3_MODE 2      // 0: never, 1: always (for tests of the variant), 2: tall shapes
+#endif
+static bool three_a_stages(const GemmArgs& g) {
+    if (g.K / 64 < 4) return false;
+    if (SP_W4_NSA3_MODE == 0) return false;
+    if (SP_W4_NSA3_MODE == 1) return true;
+    return g.tiles_n <= 8 && g.tiles_m >= 4 * g.tiles_n;
+}
+
 template <int DT, int OT>
 static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
     if constexpr (DT == SP_F32) {
         return fail(SP_ERR_DTYPE, "sp_gemm_abt: the four-wave kernel takes 16-bit inputs");
     } else {
+        const long tiles = (long)g.tiles_m * g.tiles_n;
+        if (three_a_stages(g)) {
+            auto kernel = gemm_abt_w4_kernel<DT, OT, 3>;
+            const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
+            const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
+            if (rc != SP_OK) return rc;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(256), lds_bytes, stream,
+                               SP_GEMM_PRELOADED_ARGS(g), g);
+            return check_launch("sp_gemm_abt");
+        }
         auto kernel = gemm_abt_w4_kernel<DT, OT>;
         const int lds_bytes = 2 * (256 + 256) * ROW_BYTES;
         const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
         if (rc != SP_OK) return rc;
-        const long tiles = (long)g.tiles_m * g.tiles_n;
         hipLaunchKernelGGL(kernel, dim3((unsigned)tiles, (unsigned)g.batch), dim3(256), lds_bytes, stream,
                            SP_GEMM_PRELOADED_ARGS(g), g);
         return check_launch("sp_gemm_abt");
@@ -1006,6 +1075,7 @@ struct GemmKernelNames {
         register_kernel("gemm_f32_64x64", (const void*)gemm_abt_kernel<SP_F32, SP_F32, 64, 64, 2, 2>, 256);
         register_kernel("gemm_bf16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32>, 256);
         register_kernel("gemm_f16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_F16, SP_F32>, 256);
+        register_kernel("gemm_bf16_256x256_4w_3a", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32, 3>, 256);
     }
 } gemm_kernel_names;
 }  // namespace

@@ -269,6 +269,38 @@ def test_four_wave_kernel_is_exact_on_integers(MM, dtype):
     assert (many.reshape(m, n) == want).all()
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "f16"])
+def test_four_wave_kernel_on_tall_shapes_is_exact_on_integers(MM, dtype):
+    """Tall 16-bit shapes (at least four times as many tile rows as tile columns) take the four-wave kernel with a
+    ring of three A stages, whose A stage is a run-time offset and whose fetches are counted differently: the same
+    exact-integer checks, for K of four, five and nine K-tile pairs... and every epilogue option."""
+    announce("gemm four-wave kernel with three A stages, integer problems " + dtype)
+    m, n = 32768, 512
+    t = TORCH[dtype]
+    a = ((np.arange(m * 1152, dtype=np.int64).reshape(m, 1152) * 7 + 3) % 11 - 5).astype(np.float32)
+    b = ((np.arange(n * 1152, dtype=np.int64).reshape(n, 1152) * 5 + 1) % 13 - 6).astype(np.float32)
+    for k in (256, 512, 640, 1152):
+        assert MM.matmul_config_tf32(False, True, m, n, k, t) == dict(m_tile=256, n_tile=256, k_tile=64, threads=256)
+        ak, bk = np.ascontiguousarray(a[:, :k]), np.ascontiguousarray(b[:, :k])
+        want = ak.astype(np.float64) @ bk.astype(np.float64).T      # |sum| <= 30 * 1152: exact in f32
+        assert (run(MM, ak, bk, dtype) == want).all(), k
+    k = 640
+    ak, bk = np.ascontiguousarray(a[:, :k]), np.ascontiguousarray(b[:, :k])
+    want = ak.astype(np.float64) @ bk.astype(np.float64).T
+    c0 = ((np.arange(m * n, dtype=np.int64).reshape(m, n) * 3) % 17 - 8).astype(np.float32)
+    bias = ((np.arange(n) * 5) % 201 - 100).astype(np.float32)
+    c = dev(c0.copy())
+    MM.matmul_abt(dev(ak, t), dev(bk, t), c, 2.0, -3.0)
+    assert (host(c) == 2.0 * want - 3.0 * c0).all()
+    got = run(MM, ak, bk, dtype, bias=dev(bias), relu=True)
+    assert (got == np.maximum(want + bias, 0.0)).all()
+    got16 = run(MM, ak, bk, dtype, out_dtype=t)
+    assert (got16 == ogemm.round_to(want.astype(np.float32), dtype)).all()
+    # batch of 2 members of 16384 rows (64 x 2 tiles each), B shared
+    many = host(MM.matmul_abt_batched(dev(ak.reshape(2, 16384, k), t), dev(bk, t)))
+    assert (many.reshape(m, n) == want).all()
+
+
 @pytest.mark.parametrize("dtype,out16", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
 def test_config2_8192_sampled_rows(MM, dtype, out16):
     """8192^3, both 16-bit input types, f32 and 16-bit output: the oracle is evaluated on 192 sampled rows of C
