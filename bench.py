@@ -111,10 +111,13 @@ def calibrate_hbm(steps, warmup):
         _, ev = time_launches(lambda: check(lib.sp_reduce_sum(0, ptr(x), ptr(res), n, ptr(ws), ws.numel(), stream_ptr())),
                               steps, warmup)
         out["read_%dMiB" % mib] = {"ms": round(ev, 5), "gbs": round(4 * n / (ev * 1e-3) / 1e9, 1)}
+        _, ev = time_launches(lambda: y.fill_(1.0), steps, warmup)      # write only (torch's fill kernel)
+        out["write_%dMiB" % mib] = {"ms": round(ev, 5), "gbs": round(4 * n / (ev * 1e-3) / 1e9, 1)}
         del x, y
         torch.cuda.empty_cache()
     print(json.dumps({"hbm_calibration": out, "unit": "GB/s", "peak": PEAK_HBM_GBS, "steps": steps, "warmup": warmup,
-                      "kernels": "sp_map_f32(copy): n bytes read + n written; sp_reduce_sum(f32): n bytes read"}))
+                      "kernels": "sp_map_f32(copy): n bytes read + n written; sp_reduce_sum(f32): n bytes read; "
+                                 "torch.Tensor.fill_: n bytes written"}))
 
 
 def main():

@@ -538,11 +538,20 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
 // stages against a loop body of two K-tiles): the eight fragment addresses of A are re-based once per K-tile (8
 // vector adds; the square GEMMs, whose loop does not wait, lose 0.5-2 % to them and stay on NSA = 2).  Within a K-tile the B fetches go out before the A fetches, so that at the boundary
 // "everything but the 8 youngest fetches has landed" is exactly "tile kt + 1 is complete".
-template <int DT, int OT, int NSA = 2>
+// PERSIST (with NSA = 3; beta = 0, no bias, one batch member): one workgroup per compute unit walks tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ... (the same tile -> XCD map as one workgroup per tile), and the fetch stream runs on into
+// the NEXT tile: where the last K-tiles of a tile would re-fetch the last tile into dead stages, they fetch A tiles
+// 0-2 and B tile 0 of the next tile (the A ring keeps rotating across tiles; B tile 0 lands in B stage 0 because nk
+// is even).  The epilogue's staging strips move to the second B stage (XOR-swizzled instead of padded, so that they
+// fit), and B tile 1 follows once the strips are free.  What a tile's first fetches take to arrive -- 6-8 k cycles
+// when every unit asks at once -- and the 2-4 k cycles between a workgroup's end and its successor's start are then
+// spent multiplying and storing.
+template <int DT, int OT, int NSA = 2, bool PERSIST = false>
 __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, const GemmArgs g_rest) {
     SP_GEMM_TAKE_PRELOADED;
     static_assert(DT != SP_F32, "16-bit inputs only");
     static_assert(NSA == 2 || NSA == 3, "two stages [A][B], or three A stages followed by two B stages");
+    static_assert(!PERSIST || NSA == 3, "the persistent form uses the second B stage of the three-A-stage layout for its epilogue");
     constexpr int BM = 256, BN = 256, NW = 4, ES = 2;
     constexpr int BK = ROW_BYTES / ES;
     constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
@@ -554,9 +563,10 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
+    int vblock = blockIdx.x;                     // the tile's number in the launch order of one workgroup per tile
     int tm_, tn_;
-    tile_of_block(blockIdx.x, g.tiles_m, g.tiles_n, g.group_m, tm_, tn_);
-    const long m0 = (long)tm_ * BM, n0 = (long)tn_ * BN;
+    tile_of_block(vblock, g.tiles_m, g.tiles_n, g.group_m, tm_, tn_);
+    long m0 = (long)tm_ * BM, n0 = (long)tn_ * BN;
     const long K = g.K;
     const unsigned char* const Ab = (const unsigned char*)g.A + (long)blockIdx.y * g.stride_a;
     const unsigned char* const Bb = (const unsigned char*)g.B + (long)blockIdx.y * g.stride_b;
@@ -666,10 +676,6 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
 
     const int nk = (int)(K / BK);     // even (the launcher checks K % 128 == 0)
     u32x4 fa[2][8], fb[2][8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j) acc[i][j] = zero4;
     // prologue: tiles 0 and 1 into stages 0 and 1 (NSA = 3: and the A tile 2 into the third A stage; sA then
     // points at tile 2 and sB at tile 1, what the first boundary expects)
 #pragma unroll
@@ -686,6 +692,29 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     }
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(NSA == 3 ? NI + 8 : NI) : "memory");   // tile 0 has landed
     __syncthreads();
+    bool prefetched = false;          // PERSIST: this tile's first fetches went out during the previous tile
+    for (;;) {                        // (one pass unless PERSIST)
+    // PERSIST: where the next tile's operands start (this wave's rows), for the fetches of the last K-tiles
+    int next_block = 0;
+    long next_m0 = 0, next_n0 = 0;
+    bool has_next = false;
+    const unsigned char *next_a = nullptr, *next_b = nullptr;
+    if constexpr (PERSIST) {
+        next_block = vblock + (int)gridDim.x;
+        has_next = next_block < g.tiles_m * g.tiles_n;
+        if (has_next) {
+            int ntm, ntn;
+            tile_of_block(next_block, g.tiles_m, g.tiles_n, g.group_m, ntm, ntn);
+            next_m0 = (long)ntm * BM;
+            next_n0 = (long)ntn * BN;
+            next_a = uniform_ptr(Ab + (next_m0 + wave * 8) * K * ES);
+            next_b = uniform_ptr(Bb + (next_n0 + wave * 8) * K * ES);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[i][j] = zero4;
 #pragma unroll
     for (int t = 0; t < 8; ++t) {
         load_a(0, 0, t, fa[0]);
@@ -736,10 +765,17 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
             }
         }
         if constexpr (NSA == 3) {
-            asm volatile("s_waitcnt vmcnt(8)" ::: "memory");   // all but the A tile of K-tile kt + 2
+            // all but the A tile of K-tile kt + 2 (after a prefetch only B tile 1 is in flight at the first boundary)
+            if (PERSIST && prefetched && kt == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             __syncthreads();
-            sA += kt + 3 < nk ? ROW_BYTES : 0;
-            sB += kt + 2 < nk ? ROW_BYTES : 0;
+            if (PERSIST && has_next) {       // past this tile's last K-tile the stream goes on with the next tile's first
+                sA = kt + 3 == nk ? next_a : sA + ROW_BYTES;
+                sB = kt + 2 < nk ? sB + ROW_BYTES : kt + 2 == nk ? next_b : sB;   // (B tile 1 waits for the strips' stage)
+            } else {
+                sA += kt + 3 < nk ? ROW_BYTES : 0;
+                sB += kt + 2 < nk ? ROW_BYTES : 0;
+            }
             rebase_a(0, a_next);
         } else {
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -766,14 +802,18 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     // the fetches past the end must be done before the stages are reused; the last MFMAs must have written
     // their results before the accumulators are read (18 wait states, which the compiler cannot know about)
     asm volatile("s_waitcnt vmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
-
     // ---- epilogue: per 16-row accumulator row, the wave transposes 16 x 128 values through a private LDS strip
     //      and writes C (and, for beta != 0, reads it) 16 bytes per lane: 512-byte row segments, two rows per
     //      instruction for f32 output, 256-byte segments, four rows per instruction for 16-bit output ----
-    constexpr int EPI_STRIDE = 128 * 4 + 16;
+    // (PERSIST: rows of 512 bytes without padding in the second B stage, 16-byte chunk c of row r in slot c ^ r)
+    constexpr int EPI_STRIDE = PERSIST ? 128 * 4 : 128 * 4 + 16;
     static_assert(NW * 16 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
+    static_assert(!PERSIST || NW * 16 * EPI_STRIDE <= B_BYTES, "epilogue staging must fit one B stage");
     __syncthreads();
-    unsigned char* strip = lds + wave * (16 * EPI_STRIDE);
+    unsigned char* strip = lds + (PERSIST ? B_BASE3 + B_BYTES : 0) + wave * (16 * EPI_STRIDE);
+    auto strip_at = [&](int row, int chunk) {        // byte offset of 16-byte chunk `chunk` of strip row `row`
+        return row * EPI_STRIDE + ((PERSIST ? chunk ^ (row & 15) : chunk) << 4);
+    };
     constexpr int PER = OT == SP_F32 ? 4 : 8;                 // columns per lane
     constexpr int LPR = 128 / PER;                            // lanes per row
     constexpr int RPP = 64 / LPR;                             // rows per pass
@@ -803,19 +843,19 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
         for (int i = 0; i < 8; ++i) {
 #pragma unroll
             for (int j = 0; j < 8; ++j)
-                *reinterpret_cast<f32x4*>(strip + fi * EPI_STRIDE + (16 * j + 4 * fq) * 4) = acc[i][j];
+                *reinterpret_cast<f32x4*>(strip + strip_at(fi, 4 * j + fq)) = acc[i][j];
 #pragma unroll
             for (int p = 0; p < 16 / RPP; ++p, idx += row_step) {
                 const int rl = RPP * p + er;
                 f32x4 old0 = {0.f, 0.f, 0.f, 0.f}, old1 = {0.f, 0.f, 0.f, 0.f};
                 if constexpr (OT == SP_F32) {
-                    const f32x4 v = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4));
                     f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
                     if constexpr (HAS_BETA) old0 = *c;
                     *c = finish(v, old0, bias4[0]);
                 } else {
-                    const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4);
-                    const f32x4 v1 = *reinterpret_cast<const f32x4*>(strip + rl * EPI_STRIDE + ec * 4 + 16);
+                    const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4));
+                    const f32x4 v1 = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4 + 1));
                     u32x4* c = reinterpret_cast<u32x4*>((unsigned short*)Cb + idx);
                     if constexpr (HAS_BETA) {
                         const u32x4 o = *c;
@@ -841,6 +881,20 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     } else {
         if (g.relu) write_tile(std::false_type{}, std::true_type{});
         else write_tile(std::false_type{}, std::false_type{});
+    }
+    if (!PERSIST || !has_next) break;
+    // the stores are acknowledged (the next tile's first fetches landed before the epilogue), here and (barrier)
+    // everywhere; the strips are free: B tile 1 goes into the stage they occupied.  The A ring rotates on: a_cur is
+    // the stage of the next tile's K-tile 0, and its fragment addresses were re-based at the last boundary.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    sB += ROW_BYTES;
+#pragma unroll
+    for (int q = 8; q < NI; ++q) dma_plain(q, 1);
+    vblock = next_block;
+    m0 = next_m0;
+    n0 = next_n0;
+    prefetched = true;
     }
 }
 
@@ -995,6 +1049,9 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
 
 // The four-wave kernel with a third A stage (see the kernel): when the A panels are not shared enough to come from
 // the caches.
+#ifndef SP_W4_PERSIST
+#define SP_W4_PERSIST 1
+#endif
 #ifndef SP_W4_NSA3_MODE
 #define SP_W4_NSA3_MODE 2      // 0: never, 1: always (for tests of the variant), 2: tall shapes
 #endif
@@ -1011,6 +1068,17 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
         return fail(SP_ERR_DTYPE, "sp_gemm_abt: the four-wave kernel takes 16-bit inputs");
     } else {
         const long tiles = (long)g.tiles_m * g.tiles_n;
+        const int cus = device_cu_count();
+        if (SP_W4_PERSIST && three_a_stages(g) && g.batch == 1 && g.beta == 0.f && g.bias == nullptr && cus % 8 == 0 &&
+            tiles >= 2l * cus) {
+            // several tiles per compute unit: one workgroup per unit walks them and fetches ahead across the epilogue
+            auto kernel = gemm_abt_w4_kernel<DT, OT, 3, true>;
+            const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
+            const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
+            if (rc != SP_OK) return rc;
+            hipLaunchKernelGGL(kernel, dim3((unsigned)cus, 1), dim3(256), lds_bytes, stream, SP_GEMM_PRELOADED_ARGS(g), g);
+            return check_launch("sp_gemm_abt");
+        }
         if (three_a_stages(g)) {
             auto kernel = gemm_abt_w4_kernel<DT, OT, 3>;
             const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
@@ -1076,6 +1144,7 @@ struct GemmKernelNames {
         register_kernel("gemm_bf16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32>, 256);
         register_kernel("gemm_f16_256x256_4w", (const void*)gemm_abt_w4_kernel<SP_F16, SP_F32>, 256);
         register_kernel("gemm_bf16_256x256_4w_3a", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32, 3>, 256);
+        register_kernel("gemm_bf16_256x256_4w_3a_persistent", (const void*)gemm_abt_w4_kernel<SP_BF16, SP_F32, 3, true>, 256);
     }
 } gemm_kernel_names;
 }  // namespace
