@@ -274,7 +274,7 @@ typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID
 int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream);
 
 /* Sum of all n elements into out[0], one launch.  dtype: 0 = f32, 1 = i32, 2 = u64.  `workspace` must hold
- * at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial sums and ticket counters;
+ * at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial sums with their valid marks;
  * no allocation here).  It must be ZERO-FILLED once before its first use; every call leaves it ready for the
  * next one.  Calls that may run at the same time need a workspace each.  The order of the additions depends
  * on n only, so the f32 result is the same from run to run.
@@ -284,7 +284,7 @@ int64_t sp_reduce_workspace_bytes(void);
 
 /* sp_reduce_sum for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
- * partial sums and the ticket counters live in a 24.25 KiB array inside the library's own device image, one copy
+ * partial sums and their valid marks live in a 16 KiB array inside the library's own device image, one copy
  * per GPU, kept until the process ends; the call allocates nothing and uses no memset.  Same kernel, same grid and
  * therefore bit-identical results to sp_reduce_sum.  n must not exceed sp_reduce_sum_static_max_n() (2^36
  * elements), else SP_ERR_SHAPE.  All calls on one GPU share the array: calls that may overlap in time (different

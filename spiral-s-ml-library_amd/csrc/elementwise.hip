@@ -12,7 +12,7 @@ namespace sp {
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 
 constexpr int EW_THREADS = 256;
-constexpr int REDUCE_MAX_BLOCKS = 2048;
+constexpr int REDUCE_MAX_BLOCKS = 1024;
 // Workgroups per compute unit of the grid-stride kernels (tuning constants; a build may override them).
 #ifndef SP_MAP_BLOCKS_PER_CU
 #define SP_MAP_BLOCKS_PER_CU 4      // (map on 65536 x 256 f32: 19.3 us from 1024 workgroups, 20.4 from 2048, 24.4 from 256)
@@ -61,28 +61,33 @@ __device__ __forceinline__ T block_sum(T v, T* slots) {
 }
 
 // Full-tensor sum in ONE launch.  Every block adds up its share (16-byte loads, U of them in flight per lane and U
-// independent running sums), writes its partial sum to `partial[blockIdx.x]` and takes a ticket; the block that
-// draws the last ticket adds the partials in index order and writes the result.  Which block that is changes from
-// run to run, the order of the additions does not: the result depends on n and the grid only.
-// Tickets are drawn in two levels -- a counter per group of REDUCE_GROUP blocks, then one counter that the last
-// block of every group draws from: atomic operations on ONE address take ~11 ns each on this part, whoever issues
-// them (2048 tickets from one counter: 23 us), on different addresses they overlap.
-// Partial sums and counters are device-scope atomic accesses: they go to memory past the XCD's private L2, so
-// nothing has to be written back or invalidated (a device-scope fence walks the whole L2, once per block: 60 us
-// for 2048 blocks).  A partial sum's store has completed before its block draws a ticket.
-// `counters` (REDUCE_COUNTERS of them, REDUCE_COUNTER_STRIDE bytes apart) must be zero when the kernel starts;
-// the blocks that draw last tickets leave them at zero for the next launch.
-constexpr int REDUCE_GROUP = 64;
-constexpr int REDUCE_COUNTERS = REDUCE_MAX_BLOCKS / REDUCE_GROUP + 1;     // one per group, then the top one
-constexpr int REDUCE_COUNTER_STRIDE = 256;
+// independent running sums) and PUBLISHES its partial sum as one 64-bit word per 32 bits of value -- the value below,
+// a valid mark above -- with a single device-scope atomic store into slot blockIdx.x (an 8-byte sum takes two
+// words, REDUCE_MAX_BLOCKS apart).  Block 0 then polls the slots with device-scope atomic loads until every one
+// carries the mark, clears each slot it has read, adds the partials in index order and writes the result: the
+// order of the additions depends on n and the grid only.
+// The value and its mark travel in the same atomic word, so no fence, no counter and no acknowledgement stand
+// between a block's last addition and the moment block 0 can see it: the end of the kernel is one store on its way
+// out and one load that finds it.  (The form this replaces -- store, wait for its acknowledgement, draw a ticket
+// from a counter per 64 blocks, then from a top counter, last block loads the partials -- had four dependent round
+// trips to memory past the XCD's private L2 in that place, ~0.5 us each with every memory channel busy.)
+// Device-scope atomic accesses go to memory past the L2, so nothing has to be written back or invalidated.
+// Block 0's own partial never leaves its registers.  All blocks of the grid are resident at once (at most
+// SP_REDUCE_BLOCKS_PER_CU per compute unit), and a poller that got a unit before the others only holds one block's
+// worth of it, so the poll cannot keep a block from running.  It still has a bound -- REDUCE_POLL_LIMIT rounds with a
+// short sleep in between, tens of seconds -- after which the result is a NaN / all-ones word instead of a hang.
+// The slots must be zero when the kernel starts; block 0 leaves them at zero for the next launch.
+constexpr unsigned long long REDUCE_VALID = 1ull << 32;
+constexpr long REDUCE_POLL_LIMIT = 1l << 24;
 
 template <typename T, int U>
 __global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restrict__ x, T* __restrict__ out, long n,
-                                                                T* partial, unsigned char* counters) {
+                                                                unsigned long long* slots_mem) {
     __shared__ T slots[EW_THREADS / WAVE];
-    __shared__ unsigned is_last;
     constexpr int V = 16 / sizeof(T);
+    constexpr int W = sizeof(T) / 4;                            // 64-bit words per published partial sum
     typedef T VT __attribute__((ext_vector_type(V)));
+    typedef unsigned long long u64;
     const VT* xv = reinterpret_cast<const VT*>(x);
     const long nv = n / V;
     const long stride = (long)gridDim.x * EW_THREADS;
@@ -107,31 +112,69 @@ __global__ __launch_bounds__(EW_THREADS) void reduce_sum_kernel(const T* __restr
 #pragma unroll
     for (int k = 1; k < V; ++k) acc += a[0][k];
     for (long j = nv * V + tid; j < n; j += stride) acc += x[j];   // the last n % V elements
-    acc = block_sum(acc, slots);
-    if (threadIdx.x == 0) {
-        __hip_atomic_store(partial + blockIdx.x, acc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const unsigned group = blockIdx.x / REDUCE_GROUP, groups = (gridDim.x + REDUCE_GROUP - 1) / REDUCE_GROUP;
-        const unsigned members = group + 1 < groups ? REDUCE_GROUP : gridDim.x - group * REDUCE_GROUP;
-        unsigned* mine = reinterpret_cast<unsigned*>(counters + group * REDUCE_COUNTER_STRIDE);
-        unsigned* top = reinterpret_cast<unsigned*>(counters + (REDUCE_COUNTERS - 1) * REDUCE_COUNTER_STRIDE);
-        unsigned last = 0;
-        if (__hip_atomic_fetch_add(mine, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == members - 1) {
-            __hip_atomic_store(mine, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (__hip_atomic_fetch_add(top, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == groups - 1) {
-                __hip_atomic_store(top, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                last = 1;
+    acc = block_sum(acc, slots);                                    // valid in wave 0
+
+    unsigned bits[W];
+    __builtin_memcpy(bits, &acc, sizeof(T));
+    if (blockIdx.x != 0) {
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int j = 0; j < W; ++j)
+                __hip_atomic_store(slots_mem + (long)j * REDUCE_MAX_BLOCKS + blockIdx.x, REDUCE_VALID | bits[j],
+                                   __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        return;
+    }
+    // Block 0: thread t collects slots t, t + EW_THREADS, ...; all of a thread's loads are in flight together.
+    // (Every wave polling all slots, the waves a quarter of a poll period apart, measured 1 % slower.)
+    constexpr int S = REDUCE_MAX_BLOCKS / EW_THREADS;
+    u64 w[S][W];
+    bool pending = true;
+    for (long round = 0; pending && round < REDUCE_POLL_LIMIT; ++round) {
+        if (round) __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+        for (int k = 0; k < S; ++k) {
+            const unsigned b = threadIdx.x + k * EW_THREADS;
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                if (b == 0) w[k][j] = REDUCE_VALID | bits[j];
+                else if (b < gridDim.x)
+                    w[k][j] = __hip_atomic_load(slots_mem + (long)j * REDUCE_MAX_BLOCKS + b, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_AGENT);
+                else w[k][j] = REDUCE_VALID;
             }
         }
-        is_last = last;
+        u64 all = REDUCE_VALID;
+#pragma unroll
+        for (int k = 0; k < S; ++k)
+#pragma unroll
+            for (int j = 0; j < W; ++j) all &= w[k][j];
+        pending = (all & REDUCE_VALID) == 0;
     }
-    __syncthreads();
-    if (is_last == 0) return;
     T total = T(0);
-    for (unsigned b = threadIdx.x; b < gridDim.x; b += EW_THREADS)
-        total += __hip_atomic_load(partial + b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+    for (int k = 0; k < S; ++k) {
+        const unsigned b = threadIdx.x + k * EW_THREADS;
+        if (b < gridDim.x) {
+            unsigned part[W];
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                part[j] = (unsigned)w[k][j];
+                if (b != 0 && (w[k][j] & REDUCE_VALID))
+                    __hip_atomic_store(slots_mem + (long)j * REDUCE_MAX_BLOCKS + b, 0ull, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+            }
+            T v;
+            __builtin_memcpy(&v, part, sizeof(T));
+            total += v;
+        }
+    }
+    const int gave_up = __syncthreads_or(pending);
     total = block_sum(total, slots);
-    if (threadIdx.x == 0) out[0] = total;
+    if (threadIdx.x == 0) {
+        if (gave_up) __builtin_memset(&total, 0xff, sizeof(T));   // f32: a NaN; integers: all ones
+        out[0] = total;
+    }
 }
 
 // Sets `count` 32-bit words to zero (a kernel rather than a memset so that callers may record it into a graph).
@@ -198,9 +241,8 @@ __global__ __launch_bounds__(EW_THREADS) void transpose_vec4_kernel(const unsign
     }
 }
 
-// Layout of a reduction's scratch memory: REDUCE_MAX_BLOCKS partial sums of 8 bytes, then the ticket counters.
-constexpr long REDUCE_COUNTER_OFFSET = (long)REDUCE_MAX_BLOCKS * 8;
-constexpr long REDUCE_SCRATCH_BYTES = REDUCE_COUNTER_OFFSET + (long)REDUCE_COUNTERS * REDUCE_COUNTER_STRIDE;
+// A reduction's scratch memory: two 64-bit slots per possible block (low and high half of an 8-byte partial sum).
+constexpr long REDUCE_SCRATCH_BYTES = (long)REDUCE_MAX_BLOCKS * 2 * 8;
 
 template <typename T>
 static int run_reduce(const void* x, void* out, int64_t n, void* scratch_mem, hipStream_t stream) {
@@ -212,7 +254,7 @@ static int run_reduce(const void* x, void* out, int64_t n, void* scratch_mem, hi
     if (blocks > REDUCE_MAX_BLOCKS) blocks = REDUCE_MAX_BLOCKS;
     if (blocks < 1) blocks = 1;
     hipLaunchKernelGGL((reduce_sum_kernel<T, 4>), dim3((unsigned)blocks), dim3(EW_THREADS), 0, stream, (const T*)x, (T*)out,
-                       (long)n, (T*)scratch_mem, (unsigned char*)scratch_mem + REDUCE_COUNTER_OFFSET);
+                       (long)n, (unsigned long long*)scratch_mem);
     return check_launch("sp_reduce_sum");
 }
 
@@ -310,13 +352,12 @@ extern "C" int sp_reduce_sum_static(int dtype, const void* x, void* out, int64_t
     void* mem = nullptr;
     rc = static_scratch(&mem);
     if (rc != SP_OK) return rc;
-    // The array keeps what the last call left in it.  Only the ticket counters have to start at zero (the partial
-    // sums are written before they are read); they are cleared by a kernel, not a memset, so that the call may be
-    // recorded into a graph.
+    // The array keeps what the last call left in it, and the slots' valid marks have to start at zero.  A call that
+    // ran to its end leaves them so; they are cleared all the same (by a kernel, not a memset, so that the call may
+    // be recorded into a graph): this entry point has no caller-owned workspace whose state the caller vouches for.
     hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(EW_THREADS), 0, s,
-                       reinterpret_cast<unsigned*>((unsigned char*)mem + REDUCE_COUNTER_OFFSET),
-                       (int)(REDUCE_COUNTERS * REDUCE_COUNTER_STRIDE / 4));
+    hipLaunchKernelGGL(clear_words_kernel, dim3(1), dim3(EW_THREADS), 0, s, reinterpret_cast<unsigned*>(mem),
+                       (int)(REDUCE_SCRATCH_BYTES / 4));
     rc = check_launch(__func__);
     if (rc != SP_OK) return rc;
     return run_reduce_dtype(dtype, x, out, n, mem, s);

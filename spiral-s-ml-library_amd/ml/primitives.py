@@ -360,7 +360,7 @@ def reduce_sum(x):
     code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
     key = x.device.index
     if key not in _workspace:
-        # zero-filled once: the kernel keeps a ticket counter in it and leaves it at zero after every call
+        # zero-filled once: the kernel keeps the blocks' valid marks in it and leaves them at zero after every call
         _workspace[key] = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=x.device)
     ws = _workspace[key]
     out = torch.empty(4, dtype=x.dtype, device=x.device)  # 16-byte aligned scalar slot
