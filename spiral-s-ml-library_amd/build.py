@@ -18,7 +18,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libspiral_mi355.so")
 SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip"]
-# sources whose MFMAs are inline asm: their device assembly is kept and scanned (isa_check.py)
+# sources with MFMAs or wide stores in inline asm: their device assembly is kept and scanned (isa_check.py)
 ASM_MFMA_SOURCES = ["gemm.hip", "mlp.hip", "mlp_packed.hip"]
 # Kernel-argument preloading (gfx950): the first 14 dwords of a kernel's leading scalar parameters arrive in
 # registers with the wave instead of through a scalar load at kernel entry (a struct parameter is not preloaded;
@@ -52,7 +52,8 @@ def device_asm(src):
 
 
 def check_isa():
-    """Scan the kept device assembly; raises on a vector-ALU write right in front of an MFMA that reads it."""
+    """Scan the kept device assembly; raises on a vector-ALU write right in front of an MFMA that reads the register
+    or right behind a store of more than 8 bytes that has it as data."""
     sys.path.insert(0, HERE)
     try:
         import isa_check
@@ -64,9 +65,9 @@ def check_isa():
             continue
         hits = isa_check.scan_file(path)
         if hits:
-            ln, kernel, writer, mfma = hits[0]
-            raise RuntimeError("%s: %d MFMA operand hazards, first at line %d in %s: '%s' then '%s'"
-                               % (path, len(hits), ln, kernel, writer, mfma))
+            ln, kernel, writer, other = hits[0]
+            raise RuntimeError("%s: %d MFMA-operand / store-data hazards, first at line %d in %s: '%s' next to '%s'"
+                               % (path, len(hits), ln, kernel, writer, other))
 
 
 def build(force=True, verbose=False):

@@ -42,6 +42,7 @@ struct GemmArgs {
     int group_m;   // tile rows per group of the block -> tile walk (4: an XCD's 32 concurrent tiles form a 4 x 8 patch)
     int ragged;    // M or N is not a multiple of the tile: tiles_m / tiles_n are rounded up
     int k_rotate;  // workgroup t starts its K loop at K-tile (t * k_rotate) % nk and wraps around (0: everyone at 0)
+    int store_policy;   // ST_THROUGH or ST_STREAM for the stores of C when beta == 0 (with beta != 0 C is read here: ST_PLAIN)
 };
 
 // The tiled kernels take the fields their first fetches need (operand addresses, K, batch strides, the tile grid) once
@@ -111,6 +112,27 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
     const int in_group = t % group_size;
     tm = first_m + in_group % gsz;
     tn = in_group / gsz;
+}
+
+// A store of C with a cache policy.  ST_PLAIN: the compiler's store (write-back in the XCD's L2).  ST_THROUGH
+// (sc1): written through the L2 as it is issued, instead of leaving the L2 in bursts when lines are evicted or the
+// kernel ends -- the C of a GEMM is written once and read by nobody in this launch.  ST_STREAM (nt): streaming, for
+// outputs that should not take room in the caches from operands that are read again.  The host picks one per launch
+// (`store_policy`).  Measured (bf16, f32 C, us, plain / through / stream): 65536 x 256 x 256 20.8 / 18.0 / 20.7;
+// 131072 x 256 x 256 36.5 / 33.3 / 37.3; 65536 x 256 x 2048 76.0 / 75.2 / 65.0; 8192^3 731 / 730 / 689;
+// 16384 x 4096 x 4096 383 / 390 / 364; 65536 x 2048 x 512 178 / 177 / 158; 65536 x 1024 x 512 91 / 91 / 96;
+// 8192 x 8192 x 1024 123 / 128 / 132; 4096^3 92.6 / 91.8 / 92.2.
+// The s_nop behind the asm store: the hardware wants two wait states between a store of more than 8 bytes and a
+// vector-ALU write of its data registers, which the compiler provides for its own stores and cannot for one inside
+// an asm statement (without them the next instruction's result went to memory in place of some lanes' data).
+enum { ST_PLAIN = 0, ST_THROUGH = 1, ST_STREAM = 2 };
+template <int POLICY, typename V>
+__device__ __forceinline__ void store_c(V* p, V v) {
+    static_assert(sizeof(V) == 16 || sizeof(V) == 8, "16- or 8-byte pieces of C");
+    if constexpr (POLICY == ST_STREAM) __builtin_nontemporal_store(v, p);
+    else if constexpr (POLICY == ST_PLAIN) *p = v;
+    else if constexpr (sizeof(V) == 16) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 
 // One wave-wide DMA: every lane copies 16 bytes from global memory (uniform base + per-lane
@@ -453,8 +475,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
     const long row_step = (long)RPP * g.N;
     // The options are compile-time inside the loops: a branch per output row would split them into blocks of one
     // LDS read -> one store each, with every latency exposed.
-    auto write_tile = [&](auto BETA_, auto RELU_) {
+    auto write_tile = [&](auto BETA_, auto RELU_, auto POLICY_) {
         constexpr bool HAS_BETA = decltype(BETA_)::value, RELU = decltype(RELU_)::value;
+        constexpr int POLICY = decltype(POLICY_)::value;
         auto finish = [&](f32x4 v, const f32x4& old, const f32x4& bias) {
             v = v * alpha;
             if constexpr (HAS_BETA) v += beta * old;
@@ -489,7 +512,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
                     if constexpr (OT == SP_F32) {
                         f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
                         if constexpr (HAS_BETA) old = *c;
-                        *c = finish(v, old, bias4);
+                        store_c<POLICY>(c, finish(v, old, bias4));
                     } else {
                         u32x2* c = reinterpret_cast<u32x2*>((unsigned short*)Cb + idx);
                         if constexpr (HAS_BETA) {
@@ -501,18 +524,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
                         u32x2 o;
                         o.x = pack_halves<OT>(r.x, r.y);
                         o.y = pack_halves<OT>(r.z, r.w);
-                        *c = o;
+                        store_c<POLICY>(c, o);
                     }
                 }
             }
         }
     };
+    typedef std::integral_constant<int, ST_PLAIN> plain_t;
+    typedef std::integral_constant<int, ST_THROUGH> through_t;
+    typedef std::integral_constant<int, ST_STREAM> stream_t;
     if (beta != 0.f) {
-        if (g.relu) write_tile(std::true_type{}, std::true_type{});
-        else write_tile(std::true_type{}, std::false_type{});
+        if (g.relu) write_tile(std::true_type{}, std::true_type{}, plain_t{});
+        else write_tile(std::true_type{}, std::false_type{}, plain_t{});
+    } else if (g.store_policy == ST_STREAM) {
+        if (g.relu) write_tile(std::false_type{}, std::true_type{}, stream_t{});
+        else write_tile(std::false_type{}, std::false_type{}, stream_t{});
     } else {
-        if (g.relu) write_tile(std::false_type{}, std::true_type{});
-        else write_tile(std::false_type{}, std::false_type{});
+        if (g.relu) write_tile(std::false_type{}, std::true_type{}, through_t{});
+        else write_tile(std::false_type{}, std::false_type{}, through_t{});
     }
 }
 
@@ -828,8 +857,9 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     }
     // The options are compile-time inside the loops: a branch per output row would split them into blocks of one
     // LDS read -> one store each, with every latency exposed.
-    auto write_tile = [&](auto BETA_, auto RELU_) {
+    auto write_tile = [&](auto BETA_, auto RELU_, auto POLICY_) {
         constexpr bool HAS_BETA = decltype(BETA_)::value, RELU = decltype(RELU_)::value;
+        constexpr int POLICY = decltype(POLICY_)::value;
         auto finish = [&](f32x4 v, const f32x4& old, const f32x4& bias) {
             v = v * alpha;
             if constexpr (HAS_BETA) v += beta * old;
@@ -852,7 +882,7 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
                     const f32x4 v = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4));
                     f32x4* c = reinterpret_cast<f32x4*>((float*)Cb + idx);
                     if constexpr (HAS_BETA) old0 = *c;
-                    *c = finish(v, old0, bias4[0]);
+                    store_c<POLICY>(c, finish(v, old0, bias4[0]));
                 } else {
                     const f32x4 v0 = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4));
                     const f32x4 v1 = *reinterpret_cast<const f32x4*>(strip + strip_at(rl, ec / 4 + 1));
@@ -870,17 +900,23 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
                     o.y = pack_halves<OT>(r0.z, r0.w);
                     o.z = pack_halves<OT>(r1.x, r1.y);
                     o.w = pack_halves<OT>(r1.z, r1.w);
-                    *c = o;
+                    store_c<POLICY>(c, o);
                 }
             }
         }
     };
+    typedef std::integral_constant<int, ST_PLAIN> plain_t;
+    typedef std::integral_constant<int, ST_THROUGH> through_t;
+    typedef std::integral_constant<int, ST_STREAM> stream_t;
     if (beta != 0.f) {
-        if (g.relu) write_tile(std::true_type{}, std::true_type{});
-        else write_tile(std::true_type{}, std::false_type{});
+        if (g.relu) write_tile(std::true_type{}, std::true_type{}, plain_t{});
+        else write_tile(std::true_type{}, std::false_type{}, plain_t{});
+    } else if (g.store_policy == ST_STREAM) {
+        if (g.relu) write_tile(std::false_type{}, std::true_type{}, stream_t{});
+        else write_tile(std::false_type{}, std::false_type{}, stream_t{});
     } else {
-        if (g.relu) write_tile(std::false_type{}, std::true_type{});
-        else write_tile(std::false_type{}, std::false_type{});
+        if (g.relu) write_tile(std::false_type{}, std::true_type{}, through_t{});
+        else write_tile(std::false_type{}, std::false_type{}, through_t{});
     }
     if (!PERSIST || !has_next) break;
     // the stores are acknowledged (the next tile's first fetches landed before the epilogue), here and (barrier)
@@ -1196,6 +1232,14 @@ static int gemm_entry(const char* fn, int dtype_in, int dtype_out, const void* A
     g.group_m = 4;
     g.k_rotate = 7;   // odd: coprime with the power-of-two K-tile counts of the usual shapes (measured: 1, 3, ..., 13 all within 1 %)
     g.batch = (int)batch;
+    {
+        // Outputs that cannot stay in the 256 MiB memory-side cache anyway, or that would push operands out of it
+        // (operands of more than half its size), are streamed; everything else is written through the L2.
+        const double MiB = 1048576.0;
+        const double in_bytes = (double)es_in * K * ((double)M * (stride_a ? batch : 1) + (double)N * (stride_b ? batch : 1));
+        const double out_bytes = (double)es_out * M * N * batch;
+        g.store_policy = (in_bytes >= 140 * MiB || out_bytes >= 384 * MiB) ? ST_STREAM : ST_THROUGH;
+    }
     g.stride_a = stride_a * es_in; g.stride_b = stride_b * es_in; g.stride_c = stride_c * es_out;
     if (cfg < 0 && !(flags & SP_GEMM_FORCE_GENERIC)) {
         cfg = choose_cfg_ragged(dtype_in, M, N, K, batch);

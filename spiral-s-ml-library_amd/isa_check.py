@@ -1,16 +1,24 @@
-"""Check the generated gfx950 assembly for a hazard the compiler cannot see.
+"""Check the generated gfx950 assembly for hazards the compiler cannot see.
 
-The MFMAs of the hand-scheduled kernels are inline asm, which the compiler's hazard recogniser treats as
-opaque.  The hardware wants two wait states between a vector-ALU write of a register and an MFMA that reads
-it; when the register allocator moves an operand (v_mov, v_accvgpr_*) right in front of such an asm MFMA, the
-matrix pipe reads the old value and the kernel computes garbage without any error.  `scan` reports every
-v_mfma whose source registers were written by one of the two instructions before it; the build runs it over
-the device assembly of every source that holds asm MFMAs and fails on a hit.
+Instructions inside inline asm are opaque to the compiler's hazard recogniser.  Two of the hardware's rules
+bite the hand-scheduled kernels, both silently (wrong numbers, no error):
+
+* two wait states between a vector-ALU write of a register and an MFMA that reads it: when the register
+  allocator moves an operand (v_mov, v_accvgpr_*) right in front of an asm MFMA, the matrix pipe reads the old
+  value;
+* two wait states between a memory store of more than 8 bytes and a vector-ALU write of its data registers:
+  when the next instruction's result lands in a register an asm store has not read yet, that result goes to
+  memory instead.
+
+`scan` reports every v_mfma whose source registers were written by one of the two instructions before it and
+every wide store whose data registers are written by one of the two instructions behind it; the build runs it
+over the device assembly of every source with such asm and fails on a hit.
 """
 import re
 
 _RANGE = re.compile(r"([va])\[(\d+):(\d+)\]$")
 _ONE = re.compile(r"([va])(\d+)$")
+_WIDE_STORE = re.compile(r"(global|flat|scratch|buffer)_store_dwordx[34]$")
 WAIT_STATES = 2
 
 
@@ -26,21 +34,33 @@ def _regs(tok):
 
 
 def scan(lines):
-    """Hazards in an assembly listing: a list of (line number, kernel, writer, mfma)."""
-    hits, kernel, window = [], None, []
+    """Hazards in an assembly listing: a list of (line number, kernel, writer, mfma) and, for stores, of
+    (line number, kernel, writer, store)."""
+    hits, kernel, window, stores = [], None, [], []       # stores: [wait states since, data registers, text]
     for ln, line in enumerate(lines, 1):
         s = line.split(";")[0].strip()
         if not s:
             continue
         if s.endswith(":"):
             if not s.startswith(".L"):
-                kernel, window = s[:-1], []
+                kernel, window, stores = s[:-1], [], []
             continue
         if s.startswith("."):
             continue
         parts = s.split(None, 1)
         op = parts[0]
         args = [a.strip().split(" ")[0] for a in parts[1].split(",")] if len(parts) > 1 else []
+        is_valu = op.startswith("v_") and not op.startswith("v_cmp")
+        if is_valu and args:
+            written = _regs(args[0])
+            for st in stores:
+                if st[1] & written:
+                    hits.append((ln, kernel, s, st[2]))
+        for st in stores:
+            st[0] += int(args[0], 0) + 1 if op == "s_nop" and args else 1
+        stores = [st for st in stores if st[0] < WAIT_STATES]
+        if _WIDE_STORE.match(op) and len(args) > 1:
+            stores.append([0, _regs(args[0] if op.startswith("buffer_") else args[1]), s])
         if op.startswith("v_mfma"):
             src = set()
             for a in args[1:]:

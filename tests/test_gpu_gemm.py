@@ -301,6 +301,30 @@ def test_four_wave_kernel_on_tall_shapes_is_exact_on_integers(MM, dtype):
     assert (many.reshape(m, n) == want).all()
 
 
+@pytest.mark.parametrize("m,n,k", [(65536, 256, 1152), (65536, 2048, 512), (4096, 512, 8192)])
+def test_streamed_and_written_through_outputs_are_exact_on_integers(MM, m, n, k):
+    """The stores of C carry a cache policy chosen per launch: written through the L2, or -- operands of 140 MiB and
+    more, or an output of 384 MiB and more -- streamed past the caches.  The streamed form on the eight-wave kernel
+    (144 MiB of A), on the persistent four-wave kernel (512 MiB of C) and the written-through form on a square-ish
+    problem, each with every epilogue option, exact on small integers."""
+    announce("gemm store policies, integer problems %dx%dx%d" % (m, n, k))
+    t = TORCH["bf16"]
+    a = ((np.arange(m * k, dtype=np.int64).reshape(m, k) * 7 + 3) % 5 - 2).astype(np.float32)
+    b = ((np.arange(n * k, dtype=np.int64).reshape(n, k) * 5 + 1) % 7 - 3).astype(np.float32)
+    want = a @ b.T                                   # |sum| <= 6 * 8192: every partial sum is exact in f32, here and on the device
+    ad, bd = dev(a, t), dev(b, t)
+    assert (host(MM.matmul_abt(ad, bd)) == want).all()
+    bias = ((np.arange(n) * 5) % 201 - 100).astype(np.float32)
+    got = host(MM.matmul_abt(ad, bd, bias=dev(bias), relu=True))
+    assert (got == np.maximum(want + bias, 0.0)).all()
+    got16 = host(MM.matmul_abt(ad, bd, out_dtype=t).float())
+    assert (got16 == ogemm.round_to(want.astype(np.float32), "bf16")).all()
+    c0 = ((np.arange(m * n, dtype=np.int64).reshape(m, n) * 3) % 17 - 8).astype(np.float32)
+    c = dev(c0.copy())
+    MM.matmul_abt(ad, bd, c, 2.0, -3.0)
+    assert (host(c) == 2.0 * want - 3.0 * c0).all()
+
+
 @pytest.mark.parametrize("dtype,out16", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
 def test_config2_8192_sampled_rows(MM, dtype, out16):
     """8192^3, both 16-bit input types, f32 and 16-bit output: the oracle is evaluated on 192 sampled rows of C

@@ -1,5 +1,6 @@
-"""The build's scan for the one hazard the compiler cannot see in the hand-scheduled kernels: a vector-ALU
-write of a register within two wait states of an asm MFMA that reads it."""
+"""The build's scan for the hazards the compiler cannot see in the hand-scheduled kernels: a vector-ALU write of
+a register within two wait states of an asm MFMA that reads it, or of an asm store of more than 8 bytes that has
+it as data."""
 import glob
 import importlib.util
 import os
@@ -41,6 +42,31 @@ def test_scan_finds_writes_inside_the_wait_states_and_only_those():
     found = [(kernel, writer.split()[0], writer.split()[1]) for _, kernel, writer, _ in hits]
     assert found == [("kernel_a", "v_mov_b64_e32", "v[142:143],"), ("kernel_a", "v_mov_b64_e32", "v[140:141],"),
                      ("kernel_b", "v_accvgpr_write_b32", "a32,")]
+
+
+STORES = """
+kernel_c:
+\tglobal_store_dwordx4 v[2:3], v[10:13], off sc1
+\tv_add_f32_e32 v12, v1, v2
+\tglobal_store_dwordx4 v[2:3], v[20:23], off nt
+\ts_nop 1
+\tv_add_f32_e32 v22, v1, v2
+\tglobal_store_dwordx2 v[2:3], v[30:31], off
+\tv_add_f32_e32 v30, v1, v2
+\tglobal_store_dwordx4 v[2:3], v[40:43], off
+\tv_add_f32_e32 v50, v1, v2
+\tv_mul_f32_e32 v43, v1, v2
+\tv_mul_f32_e32 v40, v1, v2
+\tbuffer_store_dwordx4 v[60:63], v5, s[0:3], 0 offen
+\tv_mov_b32_e32 v5, 0
+\tv_mov_b32_e32 v61, 0
+"""
+
+
+def test_scan_finds_writes_of_a_wide_store_s_data_inside_the_wait_states():
+    hits = _module().scan(STORES.splitlines())
+    found = [(writer.split()[1], store.split()[0]) for _, _, writer, store in hits]
+    assert found == [("v12,", "global_store_dwordx4"), ("v43,", "global_store_dwordx4"), ("v61,", "buffer_store_dwordx4")]
 
 
 def test_built_kernels_are_clean():
