@@ -107,6 +107,19 @@ __device__ __forceinline__ V group_inclusive_scan(V v, int lane_in_group) {
     return v;
 }
 
+// A 16-byte store that is written THROUGH the XCD's L2 as it is issued (device scope, `sc1`) instead of being parked
+// there until its line is evicted or the kernel ends: for outputs that are written once and not read again in the
+// launch (measured: C of a 65536 x 256 x 256 GEMM 20.8 -> 18.0 us, probabilities + scan of the fused row kernel
+// 31.4 -> 30.5 us, transpose 20.6 -> 20.4 us).  The compiler has no builtin that sets sc1 on a 16-byte store, so it
+// is issued from asm, and the hardware's two wait states between a store of more than 8 bytes and a vector-ALU
+// write of its data registers -- which the compiler inserts for its own stores and cannot see here -- are the s_nop
+// (without it the next instruction's result reaches memory in place of some lanes' data).
+template <typename V>
+__device__ __forceinline__ void store16_through(V* p, V v) {
+    static_assert(sizeof(V) == 16, "one 16-byte piece per lane");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+}
+
 // All-reduce for one row per wave (T == 64) whose result comes back through a scalar register:
 // butterfly inside the 16-lane rows, row_bcast:15 / row_bcast:31 to fold the rows into lane 63,
 // v_readlane to broadcast.  Narrower groups use the butterfly.  Masked-out lanes of the row_bcast

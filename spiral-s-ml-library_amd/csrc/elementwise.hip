@@ -237,7 +237,7 @@ __global__ __launch_bounds__(EW_THREADS) void transpose_vec4_kernel(const unsign
         const int cl = 16 * p + r0;
         const long c = tc * 64 + cl, b = tb * 64 + 4 * q;
         const u32x4 w = {tile[4 * q][cl], tile[4 * q + 1][cl], tile[4 * q + 2][cl], tile[4 * q + 3][cl]};
-        if (b < B && c < C) *reinterpret_cast<u32x4*>(dst + c * B + b) = w;
+        if (b < B && c < C) store16_through(reinterpret_cast<u32x4*>(dst + c * B + b), w);
     }
 }
 

@@ -122,16 +122,13 @@ __device__ __forceinline__ void tile_of_block(int pid, int tiles_m, int tiles_n,
 // 131072 x 256 x 256 36.5 / 33.3 / 37.3; 65536 x 256 x 2048 76.0 / 75.2 / 65.0; 8192^3 731 / 730 / 689;
 // 16384 x 4096 x 4096 383 / 390 / 364; 65536 x 2048 x 512 178 / 177 / 158; 65536 x 1024 x 512 91 / 91 / 96;
 // 8192 x 8192 x 1024 123 / 128 / 132; 4096^3 92.6 / 91.8 / 92.2.
-// The s_nop behind the asm store: the hardware wants two wait states between a store of more than 8 bytes and a
-// vector-ALU write of its data registers, which the compiler provides for its own stores and cannot for one inside
-// an asm statement (without them the next instruction's result went to memory in place of some lanes' data).
 enum { ST_PLAIN = 0, ST_THROUGH = 1, ST_STREAM = 2 };
 template <int POLICY, typename V>
 __device__ __forceinline__ void store_c(V* p, V v) {
     static_assert(sizeof(V) == 16 || sizeof(V) == 8, "16- or 8-byte pieces of C");
     if constexpr (POLICY == ST_STREAM) __builtin_nontemporal_store(v, p);
     else if constexpr (POLICY == ST_PLAIN) *p = v;
-    else if constexpr (sizeof(V) == 16) asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(p), "v"(v) : "memory");
+    else if constexpr (sizeof(V) == 16) store16_through(p, v);
     else asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
 }
 

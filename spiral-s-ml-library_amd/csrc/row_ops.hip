@@ -460,7 +460,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 #pragma unroll
             for (int c = 0; c < C; ++c)
                 if (full || (row_ok && c * 4 * T + 4 * l < cols))
-                    *reinterpret_cast<f32x4*>(a.out + base + c * 4 * T) = f32x4{p[c][0], p[c][1], p[c][2], p[c][3]};
+                    store16_through(reinterpret_cast<f32x4*>(a.out + base + c * 4 * T), f32x4{p[c][0], p[c][1], p[c][2], p[c][3]});
         }
 
         const bool want_sample = a.sample != nullptr;
@@ -483,7 +483,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 }
                 last[c] = run;
                 if (MAT && a.cdf != nullptr && (full || (row_ok && c * 4 * T + 4 * l < cols)))
-                    *reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T) = f32x4{r[0], r[1], r[2], r[3]};
+                    store16_through(reinterpret_cast<f32x4*>(a.cdf + base + c * 4 * T), f32x4{r[0], r[1], r[2], r[3]});
                 if (C > 1) carry = carry + group_broadcast_last<T>(incl);
             }
             if (want_sample) {
