@@ -53,7 +53,7 @@ def device_asm(src):
 
 def check_isa():
     """Scan the kept device assembly; raises on a vector-ALU write right in front of an MFMA that reads the register
-    or right behind a store of more than 8 bytes that has it as data."""
+    or right behind a store of more than 8 bytes that has it as data, and on a use of an MFMA's result too early."""
     sys.path.insert(0, HERE)
     try:
         import isa_check
@@ -66,7 +66,7 @@ def check_isa():
         hits = isa_check.scan_file(path)
         if hits:
             ln, kernel, writer, other = hits[0]
-            raise RuntimeError("%s: %d MFMA-operand / store-data hazards, first at line %d in %s: '%s' next to '%s'"
+            raise RuntimeError("%s: %d hazards the hardware does not interlock, first at line %d in %s: '%s' next to '%s'"
                                % (path, len(hits), ln, kernel, writer, other))
 
 

@@ -8,10 +8,14 @@ bite the hand-scheduled kernels, both silently (wrong numbers, no error):
   value;
 * two wait states between a memory store of more than 8 bytes and a vector-ALU write of its data registers:
   when the next instruction's result lands in a register an asm store has not read yet, that result goes to
-  memory instead.
+  memory instead;
+* eight wait states (a 16x16x32 MFMA is four passes on gfx950) between an MFMA and any other kind of
+  instruction that reads or overwrites its result; an MFMA in between counts as four, since it waits for the
+  matrix pipe.
 
-`scan` reports every v_mfma whose source registers were written by one of the two instructions before it and
-every wide store whose data registers are written by one of the two instructions behind it; the build runs it
+`scan` reports every v_mfma whose source registers were written by one of the two instructions before it,
+every wide store whose data registers are written by one of the two instructions behind it, and every
+instruction that touches an MFMA's result too early; the build runs it
 over the device assembly of every source with such asm and fails on a hit.
 """
 import re
@@ -20,6 +24,7 @@ _RANGE = re.compile(r"([va])\[(\d+):(\d+)\]$")
 _ONE = re.compile(r"([va])(\d+)$")
 _WIDE_STORE = re.compile(r"(global|flat|scratch|buffer)_store_dwordx[34]$")
 WAIT_STATES = 2
+MFMA_RESULT_WAIT_STATES = 8
 
 
 def _regs(tok):
@@ -34,22 +39,35 @@ def _regs(tok):
 
 
 def scan(lines):
-    """Hazards in an assembly listing: a list of (line number, kernel, writer, mfma) and, for stores, of
-    (line number, kernel, writer, store)."""
-    hits, kernel, window, stores = [], None, [], []       # stores: [wait states since, data registers, text]
+    """Hazards in an assembly listing: a list of (line number, kernel, writer, mfma); for stores, of
+    (line number, kernel, writer, store); for early uses of an MFMA's result, of (line number, kernel, user, mfma)."""
+    hits, kernel, window, stores, results = [], None, [], [], []   # stores, results: [wait states since, registers, text]
     for ln, line in enumerate(lines, 1):
         s = line.split(";")[0].strip()
         if not s:
             continue
         if s.endswith(":"):
             if not s.startswith(".L"):
-                kernel, window, stores = s[:-1], [], []
+                kernel, window, stores, results = s[:-1], [], [], []
             continue
         if s.startswith("."):
             continue
         parts = s.split(None, 1)
         op = parts[0]
         args = [a.strip().split(" ")[0] for a in parts[1].split(",")] if len(parts) > 1 else []
+        if not op.startswith("v_mfma") and not op.startswith("s_"):
+            touched = set()
+            for a in args:
+                touched |= _regs(a)
+            for r in results:
+                if r[1] & touched:
+                    hits.append((ln, kernel, s, r[2]))
+        for r in results:
+            r[0] += int(args[0], 0) + 1 if op == "s_nop" and args else 4 if op.startswith("v_mfma") else 1
+        results = [r for r in results if r[0] < MFMA_RESULT_WAIT_STATES]
+        if op.startswith("v_mfma") and args:
+            dst = _regs(args[0])
+            results = [r for r in results if not (r[1] & dst)] + [[0, dst, s]]
         is_valu = op.startswith("v_") and not op.startswith("v_cmp")
         if is_valu and args:
             written = _regs(args[0])

@@ -69,6 +69,29 @@ def test_scan_finds_writes_of_a_wide_store_s_data_inside_the_wait_states():
     assert found == [("v12,", "global_store_dwordx4"), ("v43,", "global_store_dwordx4"), ("v61,", "buffer_store_dwordx4")]
 
 
+RESULTS = """
+kernel_d:
+\tv_mfma_f32_16x16x32_f16 a[0:3], v[30:33], v[2:5], a[0:3]
+\tv_mfma_f32_16x16x32_f16 a[4:7], v[30:33], v[6:9], a[4:7]
+\tv_accvgpr_read_b32 v40, a2
+\tv_accvgpr_read_b32 v41, a5
+\ts_nop 5
+\tv_accvgpr_read_b32 v42, a6
+\tv_mfma_f32_16x16x32_f16 v[10:13], v[30:33], v[6:9], v[10:13]
+\tv_mfma_f32_16x16x32_f16 v[10:13], v[34:37], v[6:9], v[10:13]
+\ts_nop 6
+\tds_write_b128 v50, v[10:13]
+\ts_nop 0
+\tglobal_store_dwordx4 v[52:53], v[10:13], off
+"""
+
+
+def test_scan_finds_uses_of_an_mfma_result_inside_its_wait_states():
+    hits = _module().scan(RESULTS.splitlines())
+    found = [(user.split()[0], user.split()[1]) for _, _, user, _ in hits]
+    assert found == [("v_accvgpr_read_b32", "v40,"), ("v_accvgpr_read_b32", "v41,"), ("ds_write_b128", "v50,")]
+
+
 def test_built_kernels_are_clean():
     """Whatever device assembly the last build kept has no such pair (the build itself refuses to link otherwise)."""
     mod = _module()
