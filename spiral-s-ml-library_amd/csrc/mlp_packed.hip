@@ -457,7 +457,7 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const void* x_first, co
         for (int idx = lane; idx < 16 * s4; idx += 64) {
             const int r = idx / s4, c = idx - r * s4;
             if (c >= c0 && first_row + r < batch)
-                *reinterpret_cast<float4*>(block + (long)r * out.stride + 4 * c) = make_float4(0.f, 0.f, 0.f, 0.f);
+                store16_through(reinterpret_cast<f32x4*>(block + (long)r * out.stride + 4 * c), f32x4{0.f, 0.f, 0.f, 0.f});
         }
     }
     if (NOUT <= 4) {
