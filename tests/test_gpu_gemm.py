@@ -325,6 +325,27 @@ def test_streamed_and_written_through_outputs_are_exact_on_integers(MM, m, n, k)
     assert (host(c) == 2.0 * want - 3.0 * c0).all()
 
 
+@pytest.mark.parametrize("dtype,m,n,k", [("bf16", 2048, 2048, 2048), ("bf16", 4096, 4096, 4096), ("bf16", 65536, 256, 512),
+                                         ("bf16", 65536, 1024, 512), ("bf16", 16384, 256, 256), ("f32", 2048, 2048, 512),
+                                         ("f16", 1000, 1000, 1024)])
+def test_results_do_not_change_from_run_to_run(MM, dtype, m, n, k):
+    """Three launches on the same N(0,1) operands give the same bits (every kernel family and both store policies).
+    A hazard the hardware does not interlock -- an instruction overwriting a register that a store or an MFMA has
+    not read yet -- shows up exactly here: as results that differ between launches."""
+    announce("gemm run-to-run %s %dx%dx%d" % (dtype, m, n, k))
+    rng = np.random.default_rng(17)
+    a, b = make(rng, m, n, k, dtype)
+    ad, bd = dev(a, TORCH[dtype]), dev(b, TORCH[dtype])
+    first = MM.matmul_abt(ad, bd)
+    for _ in range(2):
+        c = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda")
+        MM.matmul_abt(ad, bd, c)
+        assert torch.equal(c, first)
+    if dtype != "f32":
+        first16 = MM.matmul_abt(ad, bd, out_dtype=TORCH[dtype])
+        assert torch.equal(MM.matmul_abt(ad, bd, out_dtype=TORCH[dtype]), first16)
+
+
 @pytest.mark.parametrize("dtype,out16", [("bf16", False), ("f16", False), ("bf16", True), ("f16", True)])
 def test_config2_8192_sampled_rows(MM, dtype, out16):
     """8192^3, both 16-bit input types, f32 and 16-bit output: the oracle is evaluated on 192 sampled rows of C

@@ -232,3 +232,29 @@ def test_packing_is_refused_for_other_stacks(LY):
     assert LY.pack_weights(mk([32, 256, 3])) is None                     # two layers
     assert LY.pack_weights(mk([32] + [256] * 6 + [3])) is None           # deeper than the packed kernel goes
     assert LY.packed_bytes([32, 256, 256, 256, 3]) == 4 * 4096 + 2 * 131072 + 8192
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("dims,mask,with_bias", [([32, 256, 256, 256, 3], 0, False), ([32, 256, 256, 256, 64], 3, False),
+                                                 ([256, 256, 256, 16], 0, True), ([64, 128, 96, 8], 0, False)])
+def test_results_do_not_change_from_run_to_run(LY, dims, mask, with_bias, packed):
+    """Three launches on the same inputs give the same bits, for every fused kernel (hand-issued MFMAs and loads
+    counted by hand: a wait that is one short, or a register overwritten too early, shows up as results that
+    differ between launches)."""
+    announce("mlp run-to-run dims=%s packed=%s" % (dims, packed))
+    rng = np.random.default_rng(23)
+    x, ws, u = make_problem(rng, 16384, dims, "f16")
+    wd = [dev(w, torch.float16) for w in ws]
+    bd = [dev(rng.standard_normal(w.shape[0], dtype=np.float32)) for w in ws] if with_bias else None
+    pk = LY.pack_weights(wd) if packed else None
+    if packed and pk is None:
+        pytest.skip("this stack has no packed form")
+    xd, ud = dev(x, torch.float16), dev(u)
+    logits = not (packed and mask)        # the packed kernel computes a masked head for its valid columns only
+    first = [t.clone() for t in LY.mlp_forward(xd, wd, bd, "softmax_regret_matching", ud, mask, logits, packed=pk) if t is not None]
+    for _ in range(2):
+        again = [t for t in LY.mlp_forward(xd, wd, bd, "softmax_regret_matching", ud, mask, logits, packed=pk) if t is not None]
+        assert len(first) == len(again)
+        for a, b in zip(first, again):
+            assert torch.equal(a, b)
+

@@ -487,3 +487,21 @@ def test_ties_and_nans_follow_the_stated_rules(P, cols):
         modulo = 8
         got = host(P.binarize(dev(odd), modulo)).view(np.uint32)
         assert (got == orow.binarize(odd, modulo)).all()
+
+
+def test_results_do_not_change_from_run_to_run(P):
+    """Three launches of the fused row kernel and of the sum on the same inputs give the same bits (the row outputs
+    leave through hand-issued stores, the sum's partial results through a polled hand-off between workgroups)."""
+    announce("rows run-to-run")
+    rng = np.random.default_rng(29)
+    rows, cols = 65536, 256
+    x = dev((rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(2)).astype(np.float32))
+    u = dev((1 - rng.random(rows, dtype=np.float32)).astype(np.float32))
+    first = {k: v.clone() for k, v in P.row_ops(x, u).items()}
+    total = P.reduce_sum(x).clone()
+    for _ in range(2):
+        again = P.row_ops(x, u)
+        for k in first:
+            assert torch.equal(first[k], again[k]), k
+        assert torch.equal(P.reduce_sum(x), total)
+
