@@ -43,6 +43,8 @@ struct GemmArgs {
     int ragged;    // M or N is not a multiple of the tile: tiles_m / tiles_n are rounded up
     int k_rotate;  // workgroup t starts its K loop at K-tile (t * k_rotate) % nk and wraps around (0: everyone at 0)
     int store_policy;   // ST_THROUGH or ST_STREAM for the stores of C when beta == 0 (with beta != 0 C is read here: ST_PLAIN)
+    int phase_groups;   // persistent four-wave kernel: workgroup w starts ((w / 8) % phase_groups) * phase_skew
+    int phase_skew;     // sleeps of ~2048 cycles late (0 / 1 groups: everybody at once)
 };
 
 // The tiled kernels take the fields their first fetches need (operand addresses, K, batch strides, the tile grid) once
@@ -593,6 +595,16 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     int tm_, tn_;
     tile_of_block(vblock, g.tiles_m, g.tiles_n, g.group_m, tm_, tn_);
     long m0 = (long)tm_ * BM, n0 = (long)tn_ * BN;
+    if constexpr (PERSIST) {
+        // Phase groups: all units walking their tiles in step means every unit's 256 KiB of C leave at the same
+        // moment, with the matrix pipes idle, and then nobody stores for a whole main loop.  Half of the units of
+        // every XCD (blockIdx.x / 8 is the unit's number within its XCD) start about half a tile period late, so one
+        // half stores while the other multiplies.  This pays together with STREAMED stores only: written back or
+        // through the L2, the stores of one half queue in front of the other half's fetches (measured: 105 us
+        // against 90 without groups, 77 with streamed stores, 65536 x 1024 x 512).
+        const int late = g.phase_groups > 1 ? ((int)(blockIdx.x >> 3) % g.phase_groups) * g.phase_skew : 0;
+        for (int i = 0; i < late; ++i) __builtin_amdgcn_s_sleep(32);
+    }
     const long K = g.K;
     const unsigned char* const Ab = (const unsigned char*)g.A + (long)blockIdx.y * g.stride_a;
     const unsigned char* const Bb = (const unsigned char*)g.B + (long)blockIdx.y * g.stride_b;
@@ -1109,7 +1121,20 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
             const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
             const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
             if (rc != SP_OK) return rc;
-            hipLaunchKernelGGL(kernel, dim3((unsigned)cus, 1), dim3(256), lds_bytes, stream, SP_GEMM_PRELOADED_ARGS(g), g);
+            GemmArgs gp = g;
+            // Two phase groups half a tile period apart + streamed stores, where the epilogue is a large part of a
+            // tile (f32 output, at most 16 K-tiles) and there are enough tiles per unit to win back the late start
+            // (us, in step / in two groups: 65536 x 1024 x 256 71.9 / 60.2, x 512 90.4 / 77.3, x 1024 139 / 130,
+            // x 2048 228 / 235; 65536 x 2048 x 512 164 / 145; 131072 x 1024 x 512 167 / 151; 49152 x 1024 x 512
+            // 62.4 / 57.8; two tiles per unit 43.7 / 43.5; bf16 output 65.0 / 65.4).  A tile period is ~2800 cycles
+            // per K-tile + ~9000 for the epilogue.
+            const int nk = (int)(g.K / 64);
+            if (OT == SP_F32 && nk <= 16 && tiles >= 3l * cus) {
+                gp.phase_groups = 2;
+                gp.phase_skew = 3 + nk / 2;
+                gp.store_policy = ST_STREAM;
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)cus, 1), dim3(256), lds_bytes, stream, SP_GEMM_PRELOADED_ARGS(gp), gp);
             return check_launch("sp_gemm_abt");
         }
         if (three_a_stages(g)) {
