@@ -1114,8 +1114,11 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
     } else {
         const long tiles = (long)g.tiles_m * g.tiles_n;
         const int cus = device_cu_count();
-        if (SP_W4_PERSIST && three_a_stages(g) && g.batch == 1 && g.beta == 0.f && g.bias == nullptr && cus % 8 == 0 &&
-            tiles >= 2l * cus) {
+        // (also short-K problems of any aspect with three or more tiles per unit, for the phase groups below:
+        //  8192 x 8192 x 512 89 -> 82 us, 16384 x 16384 x 512 351 -> 324; from 16 K-tiles up it no longer pays)
+        const bool short_k = g.K / 64 >= 4 && g.K / 64 <= 8 && tiles >= 3l * cus;
+        if (SP_W4_PERSIST && (three_a_stages(g) || short_k) && g.batch == 1 && g.beta == 0.f && g.bias == nullptr &&
+            cus % 8 == 0 && tiles >= 2l * cus) {
             // several tiles per compute unit: one workgroup per unit walks them and fetches ahead across the epilogue
             auto kernel = gemm_abt_w4_kernel<DT, OT, 3, true>;
             const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
