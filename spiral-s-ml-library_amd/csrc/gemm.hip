@@ -566,7 +566,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
 // stages against a loop body of two K-tiles): the eight fragment addresses of A are re-based once per K-tile (8
 // vector adds; the square GEMMs, whose loop does not wait, lose 0.5-2 % to them and stay on NSA = 2).  Within a K-tile the B fetches go out before the A fetches, so that at the boundary
 // "everything but the 8 youngest fetches has landed" is exactly "tile kt + 1 is complete".
-// PERSIST (with NSA = 3; beta = 0, no bias, one batch member): one workgroup per compute unit walks tiles blockIdx.x,
+// PERSIST (with NSA = 3; beta = 0, one batch member): one workgroup per compute unit walks tiles blockIdx.x,
 // blockIdx.x + gridDim.x, ... (the same tile -> XCD map as one workgroup per tile), and the fetch stream runs on into
 // the NEXT tile: where the last K-tiles of a tile would re-fetch the last tile into dead stages, they fetch A tiles
 // 0-2 and B tile 0 of the next tile (the A ring keeps rotating across tiles; B tile 0 lands in B stage 0 because nk
@@ -1117,8 +1117,8 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
         // (also short-K problems of any aspect with three or more tiles per unit, for the phase groups below:
         //  8192 x 8192 x 512 89 -> 82 us, 16384 x 16384 x 512 351 -> 324; from 16 K-tiles up it no longer pays)
         const bool short_k = g.K / 64 >= 4 && g.K / 64 <= 8 && tiles >= 3l * cus;
-        if (SP_W4_PERSIST && (three_a_stages(g) || short_k) && g.batch == 1 && g.beta == 0.f && g.bias == nullptr &&
-            cus % 8 == 0 && tiles >= 2l * cus) {
+        if (SP_W4_PERSIST && (three_a_stages(g) || short_k) && g.batch == 1 && g.beta == 0.f && cus % 8 == 0 &&
+            tiles >= 2l * cus) {
             // several tiles per compute unit: one workgroup per unit walks them and fetches ahead across the epilogue
             auto kernel = gemm_abt_w4_kernel<DT, OT, 3, true>;
             const int lds_bytes = (3 * 256 + 2 * 256) * ROW_BYTES;
