@@ -566,20 +566,23 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_abt_kernel(SP_GEMM_PRELOADED
 // stages against a loop body of two K-tiles): the eight fragment addresses of A are re-based once per K-tile (8
 // vector adds; the square GEMMs, whose loop does not wait, lose 0.5-2 % to them and stay on NSA = 2).  Within a K-tile the B fetches go out before the A fetches, so that at the boundary
 // "everything but the 8 youngest fetches has landed" is exactly "tile kt + 1 is complete".
-// PERSIST (with NSA = 3; beta = 0, one batch member): one workgroup per compute unit walks tiles blockIdx.x,
+// PERSIST (beta = 0, one batch member): one workgroup per compute unit walks tiles blockIdx.x,
 // blockIdx.x + gridDim.x, ... (the same tile -> XCD map as one workgroup per tile), and the fetch stream runs on into
 // the NEXT tile: where the last K-tiles of a tile would re-fetch the last tile into dead stages, they fetch A tiles
 // 0-2 and B tile 0 of the next tile (the A ring keeps rotating across tiles; B tile 0 lands in B stage 0 because nk
 // is even).  The epilogue's staging strips move to the second B stage (XOR-swizzled instead of padded, so that they
 // fit), and B tile 1 follows once the strips are free.  What a tile's first fetches take to arrive -- 6-8 k cycles
 // when every unit asks at once -- and the 2-4 k cycles between a workgroup's end and its successor's start are then
-// spent multiplying and storing.
+// spent multiplying and storing.  With NSA = 2 (long K, where the three-stage loop's extra instructions cost more than
+// its lead returns) the same: the last two K-tiles fetch K-tiles 0 and 1 of the next tile into the two stages as they
+// are released, and the strips live in the 32 KiB of LDS that two stages of 64 KiB leave free, so nothing waits for
+// the epilogue's stores either.
 template <int DT, int OT, int NSA = 2, bool PERSIST = false>
 __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, const GemmArgs g_rest) {
     SP_GEMM_TAKE_PRELOADED;
     static_assert(DT != SP_F32, "16-bit inputs only");
     static_assert(NSA == 2 || NSA == 3, "two stages [A][B], or three A stages followed by two B stages");
-    static_assert(!PERSIST || NSA == 3, "the persistent form uses the second B stage of the three-A-stage layout for its epilogue");
+    static_assert(NSA == 2 || NSA == 3, "two combined stages, or three A stages next to two B stages");
     constexpr int BM = 256, BN = 256, NW = 4, ES = 2;
     constexpr int BK = ROW_BYTES / ES;
     constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
@@ -816,11 +819,18 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
             }
             rebase_a(0, a_next);
         } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            // (PERSIST, first K-tile of a tile whose first two K-tiles came in during the previous tile: both have
+            //  landed, and what is outstanding are the previous epilogue's stores, which nobody has to wait for)
+            if (!(PERSIST && prefetched && kt == 0)) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
             __syncthreads();
-            const int adv = kt + 2 < nk ? ROW_BYTES : 0;
-            sA += adv;
-            sB += adv;
+            if (PERSIST && has_next && kt + 2 >= nk) {       // the stream goes on with the next tile's K-tiles 0 and 1
+                sA = kt + 2 == nk ? next_a : sA + ROW_BYTES;
+                sB = kt + 2 == nk ? next_b : sB + ROW_BYTES;
+            } else {
+                const int adv = kt + 2 < nk ? ROW_BYTES : 0;
+                sA += adv;
+                sB += adv;
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
         row1(ST_, std::integral_constant<int, 0>{});
@@ -843,12 +853,13 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
     // ---- epilogue: per 16-row accumulator row, the wave transposes 16 x 128 values through a private LDS strip
     //      and writes C (and, for beta != 0, reads it) 16 bytes per lane: 512-byte row segments, two rows per
     //      instruction for f32 output, 256-byte segments, four rows per instruction for 16-bit output ----
-    // (PERSIST: rows of 512 bytes without padding in the second B stage, 16-byte chunk c of row r in slot c ^ r)
+    // (PERSIST: rows of 512 bytes without padding, 16-byte chunk c of row r in slot c ^ r -- in the second B stage
+    //  with three A stages, in the 32 KiB that two combined stages leave free otherwise)
     constexpr int EPI_STRIDE = PERSIST ? 128 * 4 : 128 * 4 + 16;
     static_assert(NW * 16 * EPI_STRIDE <= 2 * STAGE_BYTES, "epilogue staging must fit the tile buffers");
     static_assert(!PERSIST || NW * 16 * EPI_STRIDE <= B_BYTES, "epilogue staging must fit one B stage");
     __syncthreads();
-    unsigned char* strip = lds + (PERSIST ? B_BASE3 + B_BYTES : 0) + wave * (16 * EPI_STRIDE);
+    unsigned char* strip = lds + (!PERSIST ? 0 : NSA == 3 ? B_BASE3 + B_BYTES : 2 * STAGE_BYTES) + wave * (16 * EPI_STRIDE);
     auto strip_at = [&](int row, int chunk) {        // byte offset of 16-byte chunk `chunk` of strip row `row`
         return row * EPI_STRIDE + ((PERSIST ? chunk ^ (row & 15) : chunk) << 4);
     };
@@ -928,14 +939,18 @@ __global__ __launch_bounds__(256) void gemm_abt_w4_kernel(SP_GEMM_PRELOADED, con
         else write_tile(std::false_type{}, std::false_type{}, through_t{});
     }
     if (!PERSIST || !has_next) break;
-    // the stores are acknowledged (the next tile's first fetches landed before the epilogue), here and (barrier)
-    // everywhere; the strips are free: B tile 1 goes into the stage they occupied.  The A ring rotates on: a_cur is
-    // the stage of the next tile's K-tile 0, and its fragment addresses were re-based at the last boundary.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    sB += ROW_BYTES;
+    if constexpr (NSA == 3) {
+        // the stores are acknowledged (the next tile's first fetches landed before the epilogue), here and (barrier)
+        // everywhere; the strips are free: B tile 1 goes into the stage they occupied.  The A ring rotates on: a_cur
+        // is the stage of the next tile's K-tile 0, and its fragment addresses were re-based at the last boundary.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        sB += ROW_BYTES;
 #pragma unroll
-    for (int q = 8; q < NI; ++q) dma_plain(q, 1);
+        for (int q = 8; q < NI; ++q) dma_plain(q, 1);
+    }
+    // (two combined stages: K-tiles 0 and 1 of the next tile are in their stages since the wait behind the main
+    //  loop, sA and sB point at K-tile 1 as after a prologue, and the strips have a place of their own)
     vblock = next_block;
     m0 = next_m0;
     n0 = next_n0;
@@ -1097,6 +1112,9 @@ static int launch_tiled(const GemmArgs& g, hipStream_t stream) {
 #ifndef SP_W4_PERSIST
 #define SP_W4_PERSIST 1
 #endif
+#ifndef SP_W4_PERSIST2
+#define SP_W4_PERSIST2 1
+#endif
 #ifndef SP_W4_NSA3_MODE
 #define SP_W4_NSA3_MODE 2      // 0: never, 1: always (for tests of the variant), 2: tall shapes
 #endif
@@ -1135,6 +1153,25 @@ static int launch_four_waves(const GemmArgs& g, hipStream_t stream) {
             if (OT == SP_F32 && nk <= 16 && tiles >= 3l * cus) {
                 gp.phase_groups = 2;
                 gp.phase_skew = 3 + nk / 2;
+                gp.store_policy = ST_STREAM;
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)cus, 1), dim3(256), lds_bytes, stream, SP_GEMM_PRELOADED_ARGS(gp), gp);
+            return check_launch("sp_gemm_abt");
+        }
+        if (SP_W4_PERSIST2 && !three_a_stages(g) && g.K / 64 <= 32 && g.batch == 1 && g.beta == 0.f && cus % 8 == 0 &&
+            tiles >= 3l * cus) {
+            // medium K, three or more tiles per compute unit: the two-stage loop walking tiles without a prologue per
+            // tile, in two phase groups with streamed stores for f32 output (us, one workgroup per tile / this form:
+            // 8192 x 8192 x 1024 127.6 / 122; 8192 x 8192 x 2048 214 / 206; 12288 x 4096 x 1024 94.4 / 90.4).  From 64
+            // K-tiles up the epilogue is too small a part of a tile: 8192^3 697 / 705-713, with or without groups.
+            auto kernel = gemm_abt_w4_kernel<DT, OT, 2, true>;
+            const int lds_bytes = (2 * (256 + 256) + 256) * ROW_BYTES;
+            const int rc = ensure_dynamic_lds((const void*)kernel, lds_bytes);
+            if (rc != SP_OK) return rc;
+            GemmArgs gp = g;
+            if (OT == SP_F32) {
+                gp.phase_groups = 2;
+                gp.phase_skew = 5;
                 gp.store_policy = ST_STREAM;
             }
             hipLaunchKernelGGL(kernel, dim3((unsigned)cus, 1), dim3(256), lds_bytes, stream, SP_GEMM_PRELOADED_ARGS(gp), gp);

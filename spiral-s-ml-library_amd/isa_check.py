@@ -16,7 +16,9 @@ bite the hand-scheduled kernels, both silently (wrong numbers, no error):
 `scan` reports every v_mfma whose source registers were written by one of the two instructions before it,
 every wide store whose data registers are written by one of the two instructions behind it, and every
 instruction that touches an MFMA's result too early; the build runs it
-over the device assembly of every source with such asm and fails on a hit.
+over the device assembly of every source with such asm and fails on a hit.  The scan follows the listing, not
+the control flow: it forgets what it has seen at an unconditional branch (the next line is reached through its
+label only) and treats every other label as fall-through.
 """
 import re
 
@@ -68,6 +70,10 @@ def scan(lines):
         if op.startswith("v_mfma") and args:
             dst = _regs(args[0])
             results = [r for r in results if not (r[1] & dst)] + [[0, dst, s]]
+        if op in ("s_branch", "s_endpgm", "s_setpc_b64"):
+            # what follows in the listing is not what runs next: it is reached through its label only
+            window, stores, results = [], [], []
+            continue
         is_valu = op.startswith("v_") and not op.startswith("v_cmp")
         if is_valu and args:
             written = _regs(args[0])

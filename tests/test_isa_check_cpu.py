@@ -83,6 +83,10 @@ kernel_d:
 \tds_write_b128 v50, v[10:13]
 \ts_nop 0
 \tglobal_store_dwordx4 v[52:53], v[10:13], off
+\tv_mfma_f32_16x16x32_f16 a[8:11], v[30:33], v[6:9], a[8:11]
+\ts_branch .LBB0_1
+.LBB0_2:
+\tv_accvgpr_write_b32 a8, 0
 """
 
 
