@@ -60,7 +60,7 @@ def check(LY, x, ws, u, dtype, head="softmax_regret_matching", mask=0, biases=No
 
 
 def test_config3_leduc_policy(LY):
-    """BASELINE config 3: batch 16384, 32 -> 256 -> 256 -> 256 -> 3, f16, softmax head, regret-matching sampling."""
+    """The benchmark's policy-network workload: batch 16384, 32 -> 256 -> 256 -> 256 -> 3, f16, softmax head, regret-matching sampling."""
     announce("mlp config 3")
     rng = np.random.default_rng(3)
     x, ws, u = make_problem(rng, 16384, [32, 256, 256, 256, 3], "f16")
@@ -161,7 +161,7 @@ def test_masked_head_without_logits(LY, dtype, batch, dims, head, mask):
 
 
 @pytest.mark.parametrize("dims,head,mask,batch,dtype,with_bias", [
-    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 16384, "f16", False),     # BASELINE config 3
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 16384, "f16", False),     # the benchmark's policy network
     ([32, 256, 256, 256, 3], "softmax", 0, 1, "bf16", False),                        # a single row
     ([32, 256, 256, 3], "softmax_regret_matching", 0, 100, "f16", True),             # three layers
     ([32, 256, 256, 256, 256, 5], "softmax_regret_matching", 0, 333, "bf16", True),  # five layers: refills into both register sets

@@ -389,7 +389,7 @@ def test_sampling_edge_cases(P):
 
 
 def test_row_ops_full_size(P):
-    """BASELINE config 5: 65536 x 256 f32 logits ~ N(0, sigma=2), one uniform per row."""
+    """The benchmark's row-primitive workload: 65536 x 256 f32 logits ~ N(0, sigma=2), one uniform per row."""
     announce("row_ops full size 65536x256")
     rng = np.random.default_rng(5)
     rows, cols = 65536, 256
