@@ -338,11 +338,11 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             const int col = c * 4 * T + 4 * l;
             if (ok[c]) {
                 if (out_ptr != nullptr)
-                    *reinterpret_cast<float4*>(out_ptr + row * (long)cols + col) =
-                        make_float4(p[c][0], p[c][1], p[c][2], p[c][3]);
+                    store16_through(reinterpret_cast<f32x4*>(out_ptr + row * (long)cols + col),
+                                    f32x4{p[c][0], p[c][1], p[c][2], p[c][3]});
                 if (cdf_ptr != nullptr)
-                    *reinterpret_cast<float4*>(cdf_ptr + row * (long)cols + col) =
-                        make_float4(cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]);
+                    store16_through(reinterpret_cast<f32x4*>(cdf_ptr + row * (long)cols + col),
+                                    f32x4{cdf[c][0], cdf[c][1], cdf[c][2], cdf[c][3]});
             }
         }
         if (row_ok && l == 0) {
