@@ -230,13 +230,15 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
-            const float inv_len = 1.f / (float)limit;
+            // one division per row, then a multiplication per element (a correctly rounded division is ten
+            // instructions; the quotients differ from p / s by at most one unit in the last place)
+            const float inv_len = 1.f / (float)limit, inv = 1.f / s;
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int j = c * 4 * T + 4 * l + k;
-                    p[c][k] = (j < limit) ? (s != 0.f ? p[c][k] / s : inv_len) : 0.f;
+                    p[c][k] = (j < limit) ? (s != 0.f ? p[c][k] * inv : inv_len) : 0.f;
                 }
         } else if (op == SP_ROW_LN_L2) {
             float s = 0.f;
@@ -248,10 +250,11 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 s = (c == 0) ? sum4(q) : s + sum4(q);
             }
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
+            const float inv = 1.f / s;
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) p[c][k] = (s != 0.f) ? v[c][k] / s : 0.f;
+                for (int k = 0; k < 4; ++k) p[c][k] = (s != 0.f) ? v[c][k] * inv : 0.f;
         } else {  // identity and the scans act on the raw input
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -431,12 +434,12 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
-            const float inv_len = 1.f / (float)limit;
+            const float inv_len = 1.f / (float)limit, inv = 1.f / s;      // as in row_kernel: one division per row
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    p[c][k] = (c * 4 * T + 4 * l + k < limit) ? (s != 0.f ? p[c][k] / s : inv_len) : 0.f;
+                    p[c][k] = (c * 4 * T + 4 * l + k < limit) ? (s != 0.f ? p[c][k] * inv : inv_len) : 0.f;
         } else {
 #pragma unroll
             for (int c = 0; c < C; ++c) {
