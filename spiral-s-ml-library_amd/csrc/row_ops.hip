@@ -366,9 +366,9 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
 // are computed by the same operations in the same order); what differs is the instruction count:
 // padding lanes hold -inf, whose exponential is 0, so no per-element validity tests remain, full
 // waves load and store without predicates, and the max reductions are single DPP instructions.
-// ANYOP = false: plain softmax only (sp_row_ops and the plain softmax ops), the code every other variant is measured
-// against; true: the op is read from the arguments (masked softmax, regret matching), at the price of a larger kernel.
-template <int T, int C, bool MAT, bool ANYOP>
+// OPK: the operation, an instantiation each -- 0 plain softmax (sp_row_ops and the plain softmax ops), 1 masked
+// softmax, 2 regret matching (masked or not: the mask is the row length then).
+template <int T, int C, bool MAT, int OPK>
 __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
     constexpr int ROWS_PER_WAVE = WAVE / T;
     const int lane = threadIdx.x & (WAVE - 1);
@@ -405,7 +405,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
 
         float p[C][4];
         float s = 0.f;
-        if (ANYOP && a.op == SP_ROW_MASKED_SOFTMAX) {
+        if (OPK == 1) {
             // columns past the mask enter as -inf (their exponential is an exact 0) and the shift is the max of
             // the columns inside the mask, as in row_kernel
             float m = NEG_INF;
@@ -423,7 +423,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 for (int k = 0; k < 4; ++k) p[c][k] = fast_exp(p[c][k] - m);
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
-        } else if (ANYOP && (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING)) {
+        } else if (OPK == 2) {
             // local_regret_matching (ml/primitives.spi:718-722, masked :761-780), operation for operation as in
             // row_kernel: positive parts over their sum, the uniform distribution over the mask when that sum is 0
             const int limit = a.mask_size;
@@ -448,7 +448,7 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
         }
-        if (!(ANYOP && (a.op == SP_ROW_REGRET_MATCHING || a.op == SP_ROW_MASKED_REGRET_MATCHING))) {
+        if (OPK != 2) {
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
             const float inv = 1.f / s;
 #pragma unroll
@@ -592,16 +592,16 @@ __device__ __forceinline__ RowArgs with_preloaded(const RowArgs& a, const float*
 }
 
 // MAT = true: probabilities and/or running sums are written out.
-template <int T, int C, bool ANYOP = false>
+template <int T, int C, int OPK = 0>
 __global__ __launch_bounds__(ROW_THREADS) void row_softmax_kernel(const float* x, const float* u, long rows, int cols, const RowArgs a) {
-    row_softmax_body<T, C, true, ANYOP>(with_preloaded(a, x, u, rows, cols));
+    row_softmax_body<T, C, true, OPK>(with_preloaded(a, x, u, rows, cols));
 }
 
 // MAT = false: per-row results only; nothing of the row is written back.
-template <int T, int C, bool ANYOP = false>
+template <int T, int C, int OPK = 0>
 __global__ __launch_bounds__(ROW_THREADS) void row_softmax_scalars_kernel(const float* x, const float* u, long rows, int cols,
                                                                          const RowArgs a) {
-    row_softmax_body<T, C, false, ANYOP>(with_preloaded(a, x, u, rows, cols));
+    row_softmax_body<T, C, false, OPK>(with_preloaded(a, x, u, rows, cols));
 }
 
 // Integer rows: identity and exact scans (two's complement wrap-around).
@@ -822,19 +822,19 @@ static int launch_row(const RowArgs& args, hipStream_t stream, const char* fn) {
     const int c = (int)((a.cols + 4 * t - 1) / (4 * t));
     const int grid = row_grid(a.rows, t);
     rc = dispatch_tc(t, c, [&](auto T_, auto C_) {
-        const bool rows_out = a.out != nullptr || a.cdf != nullptr, any_op = a.op != SP_ROW_SOFTMAX;
-        if (FUSED && rows_out && !any_op)
-            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value, false>), dim3(grid),
-                               dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
-        else if (FUSED && rows_out)
-            hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value, true>), dim3(grid),
-                               dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
-        else if (FUSED && !any_op)   // per-row results only: nothing of the row itself is written back
-            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value, false>), dim3(grid),
-                               dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
-        else if (FUSED)
-            hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value, true>), dim3(grid),
-                               dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
+        const bool rows_out = a.out != nullptr || a.cdf != nullptr;
+        auto fused = [&](auto OPK_) {
+            constexpr int OPK = decltype(OPK_)::value;
+            if (rows_out)
+                hipLaunchKernelGGL((row_softmax_kernel<decltype(T_)::value, decltype(C_)::value, OPK>), dim3(grid),
+                                   dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
+            else   // per-row results only: nothing of the row itself is written back
+                hipLaunchKernelGGL((row_softmax_scalars_kernel<decltype(T_)::value, decltype(C_)::value, OPK>), dim3(grid),
+                                   dim3(ROW_THREADS), 0, stream, a.x, a.u, a.rows, a.cols, a);
+        };
+        if (FUSED && a.op == SP_ROW_SOFTMAX) fused(std::integral_constant<int, 0>{});
+        else if (FUSED && a.op == SP_ROW_MASKED_SOFTMAX) fused(std::integral_constant<int, 1>{});
+        else if (FUSED) fused(std::integral_constant<int, 2>{});
         else
             hipLaunchKernelGGL((row_kernel<decltype(T_)::value, decltype(C_)::value>), dim3(grid), dim3(ROW_THREADS), 0,
                                stream, a);
