@@ -149,13 +149,20 @@ typedef enum {
     SP_ROW_REGRET_MATCHING = 4,         /* local_regret_matching                        primitives.spi:718-722 */
     SP_ROW_MASKED_REGRET_MATCHING = 5,  /* local_masked_regret_matching                 primitives.spi:761-780 */
     SP_ROW_INCLUSIVE_SCAN = 6,          /* local_inclusive_scan_sum                     primitives.spi:323-325 */
-    SP_ROW_EXCLUSIVE_SCAN = 7           /* local_exclusive_scan config 0 (+)            primitives.spi:327 */
+    SP_ROW_EXCLUSIVE_SCAN = 7,          /* local_exclusive_scan config 0 (+)            primitives.spi:327 */
+    SP_ROW_L1_NORMALIZE = 8             /* local_l1_normalize (sp_row_l1_normalize only) primitives.spi:725-729 */
 } sp_row_op;
 
 /* out = op(x) row by row, x and out (rows, cols) f32.  Replaces `row_map f x out`
  * (ml/primitives.spi:514-520) for the lambdas listed in sp_row_op.  mask_size is used by the
  * masked ops only (1 <= mask_size <= cols). */
 int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, int64_t cols, int32_t mask_size, void* stream);
+
+/* out = |x| * (s > threshold ? threshold / s : 1) row by row, s = sum over j of |x[r, j]|: a row whose l1 norm is above
+ * `threshold` (> 0) is scaled down to it, any other row becomes its absolute values.  Replaces
+ * `row_map (local_l1_normalize threshold)` (ml/primitives.spi:725-729; caller ml/cfr.spi:244, the decay of the average
+ * policy).  `out` may be x. */
+int sp_row_l1_normalize(const float* x, float* out, int64_t rows, int64_t cols, float threshold, void* stream);
 
 /* Integer scans (SP_ROW_INCLUSIVE_SCAN / SP_ROW_EXCLUSIVE_SCAN / SP_ROW_IDENTITY) on i32 rows; exact
  * (wrap-around two's complement like the device adds of the reference, test2 :948-950). */
@@ -273,14 +280,30 @@ typedef enum { SP_MAP_COPY = 0, SP_MAP_RELU = 1, SP_MAP_TANH = 2, SP_MAP_SIGMOID
  * (ml/primitives.spi:115-133) for the activation lambdas of ml/layers.spi:353-355. */
 int sp_map_f32(int op, const float* x, float* out, int64_t n, void* stream);
 
-/* Sum of all n elements into out[0], one launch.  dtype: 0 = f32, 1 = i32, 2 = u64.  `workspace` must hold
- * at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial sums with their valid marks;
- * no allocation here).  It must be ZERO-FILLED once before its first use; every call leaves it ready for the
- * next one.  Calls that may run at the same time need a workspace each.  The order of the additions depends
- * on n only, so the f32 result is the same from run to run.
- * Replaces `reduce 0 (+)` / `grid_reduce grid 0 (+)` (ml/primitives.spi:136-197, test6 :1102-1105). */
+/* out[0] = x[0] op x[1] op ... op x[n - 1] over a whole tensor, one launch over the whole device.  op: SP_REDUCE_SUM,
+ * SP_REDUCE_PROD, SP_REDUCE_MAX or SP_REDUCE_MIN with the neutral elements 0, 1, lowest and highest value of the type
+ * (corebase/limit.spi); dtype: 0 = f32, 1 = i32, 2 = u64.  float max / min ignore a NaN operand unless both are NaN.
+ * Replaces `reduce neutral f` / `grid_reduce grid neutral f` (ml/primitives.spi:136-197; `grid_reduce grid 0 max`,
+ * ml/cem.spi:140; `reduce 0 (+)` on u64, test6 :1102-1105).
+ * `workspace` must hold at least sp_reduce_workspace_bytes() bytes of device memory (per-block partial results, each
+ * tagged with a number drawn per launch, and a give-up counter; no allocation here).  Zero-fill it once before its
+ * first use (the counter starts from what it finds; the slots do not depend on it: a partial result only counts when
+ * it carries the tag of the launch that polls it).  Calls that may run at the same time need a workspace each.  The
+ * order of the operations depends on n only, so an f32 result is the same from run to run.
+ * The launch ends with one workgroup waiting for the others' partial results.  That wait is bounded (5 ms unless
+ * sp_reduce_set_poll_limit changed it): when other work keeps part of the launch off the device for longer, the call
+ * gives up, out[0] becomes a NaN (f32) or an all-ones word, the slots are cleared and the workspace's give-up counter
+ * goes up by one.  sp_reduce_status reads that counter (it copies 8 bytes to the host and therefore WAITS for the
+ * stream, the only call of this library that does); a caller that cannot rule out such contention checks it.
+ * sp_reduce_set_poll_limit sets the bound in microseconds for later launches of this process (0 = the default, at most
+ * 10 s; a negative value makes every launch give up without waiting: a way to exercise the give-up path in which
+ * every kernel still runs to its end). */
+int sp_reduce(int op, int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes, void* stream);
+/* sp_reduce with op = SP_REDUCE_SUM. */
 int sp_reduce_sum(int dtype, const void* x, void* out, int64_t n, void* workspace, int64_t workspace_bytes, void* stream);
 int64_t sp_reduce_workspace_bytes(void);
+int sp_reduce_status(const void* workspace, int64_t workspace_bytes, int64_t* give_ups, void* stream);
+int sp_reduce_set_poll_limit(int64_t microseconds);
 
 /* sp_reduce_sum for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
@@ -324,7 +347,13 @@ typedef enum {
  *   biases       NULL, or a host array of n_layers device pointers to f32 (dims[i+1],) (entries may be NULL)
  *   dims         host array of n_layers + 1 layer widths; dims[0] a multiple of 16, hidden widths
  *                multiples of 32, all <= 256; dims[n_layers] <= 64
- *   u            (batch,) f32 in (0, 1], or NULL when action_out is NULL
+ *   u            (batch,) f32 in (0, 1], or NULL
+ *   philox       NULL, or the stream the head draws its uniforms from itself, as the reference's graph run does
+ *                (one generator per thread seeded at the start of the run, ml/layers.spi:339-344; the struct and its
+ *                row -> draw mappings are those of sp_row_sample, SP_PHILOX_LAYER being the graph run's): row r uses
+ *                exactly the uniform sp_philox_uniforms(philox, ., batch, dims[n_layers]) would hand out for it, so no
+ *                uniform tensor is written or read.  dims[n_layers] must then be a multiple of 4 (the row width of
+ *                the reference's sampling op).  With action_out exactly one of u and philox is given.
  *   policy_out   (batch, dims[n_layers]) f32
  *   action_out   (batch,) i32 or NULL
  *   logits_out   (batch, dims[n_layers]) f32 or NULL
@@ -337,8 +366,8 @@ typedef enum {
  * Against an evaluation that rounds its activations the same way everything is within 2e-4.
  */
 int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights, const float* const* biases,
-                   const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,
-                   int64_t batch, int32_t head, int32_t mask_size, void* stream);
+                   const int32_t* dims, const float* u, const sp_philox_t* philox, float* policy_out, int32_t* action_out,
+                   float* logits_out, int64_t batch, int32_t head, int32_t mask_size, void* stream);
 
 /*
  * The same forward pass over weights that were packed once into MFMA operand order: the weights then stream
@@ -356,14 +385,20 @@ int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const
  *   sp_mlp_forward_packed sp_mlp_forward with `packed` in place of `weights`; same results (the k-order of the
  *                         sums is the same).  At most 16 outputs: dims[n_layers] <= 16, or a masked head of at
  *                         most 16 columns without logits_out.  SP_ERR_UNSUPPORTED for any other stack: call
- *                         sp_mlp_forward with the row-major weights instead.
+ *                         sp_mlp_forward with the row-major weights instead.  `packed_bytes` is the size the buffer
+ *                         was packed with and must equal sp_mlp_packed_bytes(n_layers, dims), else SP_ERR_ARG: a
+ *                         buffer packed for another layer count or another class of first width has another size
+ *                         and would be read out of bounds.  The buffer does not record the 16-bit type or the
+ *                         weights' values: handing over a buffer packed from other weights of the same shape is
+ *                         the caller's to avoid.
  */
 int64_t sp_mlp_packed_bytes(int32_t n_layers, const int32_t* dims);
 int sp_mlp_pack_weights(int dtype, int32_t n_layers, const void* const* weights, const int32_t* dims, void* packed,
                         int64_t packed_bytes, void* stream);
-int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void* packed, const float* const* biases,
-                          const int32_t* dims, const float* u, float* policy_out, int32_t* action_out, float* logits_out,
-                          int64_t batch, int32_t head, int32_t mask_size, void* stream);
+int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void* packed, int64_t packed_bytes,
+                          const float* const* biases, const int32_t* dims, const float* u, const sp_philox_t* philox,
+                          float* policy_out, int32_t* action_out, float* logits_out, int64_t batch, int32_t head,
+                          int32_t mask_size, void* stream);
 
 #ifdef __cplusplus
 }

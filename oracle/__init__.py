@@ -20,6 +20,13 @@ Pinning status of each function (what checks it besides its own formula):
   row_ops.discrete_sampling               pinned: golden output_sampling*.txt, output_sample_reduce.txt
   row_ops.reduce_sum                      pinned: golden test6 (closed form 134209536)
   row_ops.transpose_inner                 pinned: golden test5 transpose.txt
+  row_ops.l1_normalize                    PARITY UNPINNED against the reference (no output of it is stored);
+                                           pinned mathematically: rows under the threshold come back as their
+                                           absolute values, rows above it sum to the threshold and keep their
+                                           proportions, a negative entry comes back positive, the l2 norm is not
+                                           what is clamped (tests/test_oracle_math.py)
+  row_ops.reduce_all                      NumPy's own sum / prod / max / min over the flattened tensor (library
+                                           routines); the u64 sum reproduces golden test6
   gemm.gemm_abt                           PARITY UNPINNED against the reference (it stores no GEMM
                                            vectors; its self-test only prints a max-abs-diff,
                                            ml/matmul/run.spi:54-58).  Pinned mathematically instead:

@@ -142,6 +142,28 @@ def regret_matching(x):
         return np.where(s != 0, r / s, inv_len).astype(np.float32)
 
 
+def l1_normalize(x, threshold):
+    """`local_l1_normalize threshold` (ml/primitives.spi:725-729): the absolute values of a row, scaled by
+    threshold / sum when their sum is above the threshold (the norm is clamped, never raised)."""
+    a = np.abs(_f32(x))
+    s = a.sum(axis=-1, keepdims=True, dtype=np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        v = np.where(s > F32(threshold), F32(threshold) / s, F32(1)).astype(np.float32)
+    return (v * a).astype(np.float32)
+
+
+def reduce_all(x, op):
+    """`reduce neutral f` over a whole tensor (ml/primitives.spi:136-197) for f in "+", "*", "max", "min"; integer
+    sums and products wrap around like the device's."""
+    x = np.asarray(x)
+    flat = x.reshape(-1)
+    if op in ("+", "sum"):
+        return flat.sum(dtype=x.dtype) if x.dtype.kind in "iu" else flat.sum(dtype=np.float64).astype(x.dtype)
+    if op in ("*", "prod"):
+        return flat.prod(dtype=x.dtype) if x.dtype.kind in "iu" else flat.prod(dtype=np.float64).astype(x.dtype)
+    return flat.max() if op == "max" else flat.min()
+
+
 def masked_regret_matching(x, size):
     """`local_masked_regret_matching` with mask `j < size` (ml/primitives.spi:761-780)."""
     x = _f32(x)

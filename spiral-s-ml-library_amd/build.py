@@ -74,7 +74,7 @@ def build(force=True, verbose=False):
     """Compile every HIP source and link the shared library.  Returns the library path."""
     os.makedirs(OBJ, exist_ok=True)
     cc = hipcc()
-    headers = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "mlp_common.h"), os.path.join(ROOT, "include", "spiral_mi355.h")]
+    headers = [os.path.join(CSRC, "common.h"), os.path.join(CSRC, "mlp_common.h"), os.path.join(CSRC, "philox.h"), os.path.join(ROOT, "include", "spiral_mi355.h")]
     newest_header = max(os.path.getmtime(h) for h in headers)
 
     def compile_one(src):

@@ -231,7 +231,7 @@ __global__ __launch_bounds__(NW * 64) void mlp_forward_kernel(const MlpArgs a) {
         const int N = a.dims[a.n_layers];
         const int limit = a.mask_size > 0 ? a.mask_size : N;
         float* p = head_rows + lane * MLP_MAX_OUT;   // this row's outputs
-        const float u = a.action != nullptr ? a.u[row] : 1.f;
+        const float u = a.ph.philox_mode >= 0 ? reference_row_uniform(a.ph, row) : a.action != nullptr ? a.u[row] : 1.f;
         if (N <= 8) head_row<8>(head_out(a), p, row, N, limit, u);      // narrow heads run in registers
         else head_row<MLP_MAX_OUT>(head_out(a), p, row, N, limit, u);
     }
@@ -274,8 +274,9 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
     const long batch = a.batch;
     const HeadOut out = head_out(a);
     const int mask_size = a.mask_size;
+    const int ph_mode = a.ph.philox_mode;
     asm volatile("" ::"s"(K0), "s"(NL), "s"(NOUT), "s"(x_ptr), "s"(w0_ptr), "s"(w1_ptr), "s"(b0_ptr), "s"(u_ptr), "s"(batch),
-                 "s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(mask_size));
+                 "s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(mask_size), "s"(ph_mode));
     const int n_chunks = C0 + 4 * (NL - 2) + 1;
     u32x2 tab_w, tab_b;
     {
@@ -511,6 +512,7 @@ __global__ __launch_bounds__(NW * 64) void mlp_h256_kernel(const MlpArgs a) {
         }
     }
     asm volatile("" : "+v"(u_row), "+v"(tab_w), "+v"(tab_b));
+    if (ph_mode >= 0) u_row = reference_row_uniform(a.ph, row_ok ? row : 0);   // the head draws its own uniform
     first_sync();
     run_chunk(IC<0>{}, IC<1>{});
     if constexpr (C0 > 1) {
@@ -624,6 +626,7 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const void* x_first, con
     const long batch = batch_first;
     const HeadOut out = head_out(a);
     const int mask_size = a.mask_size;
+    const int ph_mode = a.ph.philox_mode;
     u32x2 tab_w, tab_b;
     {
         const unsigned char* args = (const unsigned char*)__builtin_amdgcn_kernarg_segment_ptr() + ARGS_OFFSET;
@@ -742,6 +745,7 @@ __global__ __launch_bounds__(256) void mlp_split_kernel(const void* x_first, con
 #pragma unroll
     for (int i = 0; i < KS0; ++i) asm volatile("" : "+v"(xin[i]));
     asm volatile("" : "+v"(u_row), "+v"(tab_w), "+v"(tab_b), "+v"(bias_r[0]), "+v"(bias_r[1]), "+v"(bias_r[2]), "+v"(bias_r[3]));
+    if (ph_mode >= 0) u_row = reference_row_uniform(a.ph, head_ok ? head_row_idx : 0);   // the head draws its own uniform
 #pragma unroll
     for (int i = 0; i < KS0; ++i) {
         const int idx = tid + 256 * i;
@@ -969,9 +973,9 @@ static const void* pick_split_kernel(int dtype, int ks0) {
 }
 
 extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const void* const* weights,
-                              const float* const* biases, const int32_t* dims, const float* u, float* policy_out,
-                              int32_t* action_out, float* logits_out, int64_t batch, int32_t head, int32_t mask_size,
-                              void* stream) {
+                              const float* const* biases, const int32_t* dims, const float* u, const sp_philox_t* philox,
+                              float* policy_out, int32_t* action_out, float* logits_out, int64_t batch, int32_t head,
+                              int32_t mask_size, void* stream) {
     SP_REQUIRE_PTR(x);
     SP_REQUIRE_PTR(policy_out);
     SP_OPTIONAL_PTR(u); SP_OPTIONAL_PTR(action_out); SP_OPTIONAL_PTR(logits_out);
@@ -981,8 +985,11 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
         return fail(SP_ERR_ARG, "sp_mlp_forward: n_layers must be in [1, %d], got %d", MLP_MAX_LAYERS, n_layers);
     if (batch <= 0) return fail(SP_ERR_SHAPE, "sp_mlp_forward: batch must be positive");
     if (head < SP_HEAD_NONE || head > SP_HEAD_SOFTMAX_RM) return fail(SP_ERR_ARG, "sp_mlp_forward: unknown head %d", head);
-    if (action_out != nullptr && u == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward: action requested but u is NULL");
+    if (action_out != nullptr && u == nullptr && philox == nullptr)
+        return fail(SP_ERR_NULL, "sp_mlp_forward: action requested but u and philox are NULL");
+    if (u != nullptr && philox != nullptr) return fail(SP_ERR_ARG, "sp_mlp_forward: at most one of u and philox may be given");
     MlpArgs a{};
+    a.ph.philox_mode = -1;
     for (int i = 0; i <= n_layers; ++i) {
         const int d = dims[i];
         if (d <= 0) return fail(SP_ERR_SHAPE, "sp_mlp_forward: dims[%d] must be positive", i);
@@ -1005,7 +1012,9 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
         a.w[i] = weights[i];
         a.b[i] = biases ? biases[i] : nullptr;
     }
-    int rc = require_gfx950(__func__);
+    int rc = mlp_set_philox(a.ph, philox, batch, dims[n_layers], __func__);
+    if (rc != SP_OK) return rc;
+    rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
     a.x = x; a.n_layers = n_layers; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.nout = dims[n_layers];

@@ -2,6 +2,7 @@
 // batch row (softmax / regret matching / sampling), packed conversions, the LDS DMA.
 #pragma once
 #include "common.h"
+#include "philox.h"
 
 #pragma clang fp contract(off)
 
@@ -36,7 +37,20 @@ struct MlpArgs {
     int mask_size;
     int k0, nout;        // dims[0] and dims[n_layers] once more, so that a kernel needs no dependent load for them
     int out_stride;      // floats between two rows of policy / logits (= dims[n_layers]; nout may be smaller, see sp_mlp_forward)
+    PhiloxStream ph;     // philox_mode >= 0: the head draws its uniform itself (ml/layers.spi:339-344) and `u` is not read
 };
+
+// The Philox stream of a head that draws its own uniforms: the sampling node of the layer graph works on rows of
+// `cols` = the last layer's full width, which the reference's row primitives need to be a multiple of 4.
+inline int mlp_set_philox(PhiloxStream& ph, const sp_philox_t* philox, int64_t batch, int cols, const char* fn) {
+    ph.philox_mode = -1;
+    if (philox == nullptr) return SP_OK;
+    if (cols % 4 != 0)
+        return fail(SP_ERR_ARG, "%s: a head that draws from a Philox stream needs an output width that is a multiple of 4 (the "
+                    "row width of the sampling op whose stream it follows), got %d", fn, cols);
+    ph.cols = cols;
+    return set_philox(ph, philox, batch, (int64_t)cols, fn);
+}
 
 // max(x, 0) and rounding of two f32 values to the 16-bit storage type, packed into one register
 // (v_max_f32 + v_cvt_pk_{f16,bf16}_f32: round to nearest even in hardware).  The max is issued from

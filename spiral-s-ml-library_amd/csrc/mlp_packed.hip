@@ -50,6 +50,7 @@ struct MlpPackedArgs {
     float* logits;
     long batch;
     int head, mask_size, k0, nout, out_stride;
+    PhiloxStream ph;     // philox_mode >= 0: the head draws its uniform itself and `u` is not read
 };
 
 // Where feature-split layer `layer` (0: the first layer with ks0 k-steps, else a hidden layer) keeps the block of
@@ -185,6 +186,7 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const void* x_first, co
     const int mask_size = a.mask_size;
     const float* const u_ptr = u_first;
     const float* const last_bias = a.b[S];
+    const int ph_mode = a.ph.philox_mode;
 
     // ---- per-thread loads: the workgroup's input rows (16-byte pieces, 4 KS0 per row), the uniform of the row
     //      this lane will finish, one bias value per feature-split layer (feature tid) ----
@@ -259,7 +261,11 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const void* x_first, co
     static_for<0, PK_SLOTS_START>([&](auto S_) { slot(IC<0>{}, S_); });
     // every other scalar argument is waited for HERE, once, behind the first loads: a read at the point of use costs
     // a few hundred cycles, and the wait for it also drains the LDS reads in flight
-    asm volatile("" ::"s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(out.stride), "s"(mask_size), "s"(last_bias));
+    asm volatile("" ::"s"(out.policy), "s"(out.action), "s"(out.logits), "s"(out.head), "s"(out.stride), "s"(mask_size), "s"(last_bias),
+                 "s"(ph_mode));
+    // a head that draws its own uniform does so here, while the first loads are on their way
+    float u_ph = 0.f;
+    if (ph_mode >= 0) u_ph = reference_row_uniform(a.ph, head_ok ? head_row_idx : 0);
 
     // ---- operand addresses ----
     // activations: row r, 16-byte piece P (of 32) lives in slot (P & 16) | ((P ^ r) & 15) of the row's 512 bytes
@@ -279,6 +285,7 @@ __global__ __launch_bounds__(256) void mlp_packed_kernel(const void* x_first, co
 #pragma unroll
     for (int i = 0; i < KS0; ++i) asm volatile("" : "+v"(xin[i]));
     asm volatile("" : "+v"(u_row));
+    if (ph_mode >= 0) u_row = u_ph;
 #pragma unroll
     for (int l = 0; l < S; ++l) asm volatile("" : "+v"(bias_in[l]));
 #pragma unroll
@@ -567,9 +574,10 @@ extern "C" int sp_mlp_pack_weights(int dtype, int32_t n_layers, const void* cons
     return check_launch(__func__);
 }
 
-extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void* packed, const float* const* biases,
-                                     const int32_t* dims, const float* u, float* policy_out, int32_t* action_out,
-                                     float* logits_out, int64_t batch, int32_t head, int32_t mask_size, void* stream) {
+extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void* packed, int64_t packed_bytes,
+                                     const float* const* biases, const int32_t* dims, const float* u, const sp_philox_t* philox,
+                                     float* policy_out, int32_t* action_out, float* logits_out, int64_t batch, int32_t head,
+                                     int32_t mask_size, void* stream) {
     SP_REQUIRE_PTR(x);
     SP_REQUIRE_PTR(packed);
     SP_REQUIRE_PTR(policy_out);
@@ -580,13 +588,18 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
         return fail(SP_ERR_ARG, "sp_mlp_forward_packed: n_layers must be in [1, %d], got %d", MLP_MAX_LAYERS, n_layers);
     if (batch <= 0) return fail(SP_ERR_SHAPE, "sp_mlp_forward_packed: batch must be positive");
     if (head < SP_HEAD_NONE || head > SP_HEAD_SOFTMAX_RM) return fail(SP_ERR_ARG, "sp_mlp_forward_packed: unknown head %d", head);
-    if (action_out != nullptr && u == nullptr)
-        return fail(SP_ERR_NULL, "sp_mlp_forward_packed: action requested but u is NULL");
+    if (action_out != nullptr && u == nullptr && philox == nullptr)
+        return fail(SP_ERR_NULL, "sp_mlp_forward_packed: action requested but u and philox are NULL");
+    if (u != nullptr && philox != nullptr) return fail(SP_ERR_ARG, "sp_mlp_forward_packed: at most one of u and philox may be given");
     if (!packed_shape_ok(n_layers, dims))
         return fail(SP_ERR_UNSUPPORTED, "sp_mlp_forward_packed: the packed kernel takes %d to %d layers, hidden widths of 256 and "
                     "a first width that is a multiple of 16", PK_MIN_LAYERS, PK_MAX_LAYERS);
     if (mask_size < 0 || mask_size > dims[n_layers])
         return fail(SP_ERR_ARG, "sp_mlp_forward_packed: mask_size must be in [0, %d], got %d", dims[n_layers], mask_size);
+    // the size names the layout: it depends on the layer count and on how many k-steps the first layer has
+    if (packed_bytes != pk_total_bytes(pk_ks0(dims[0]), n_layers))
+        return fail(SP_ERR_ARG, "sp_mlp_forward_packed: a packed buffer for this stack holds %lld bytes (sp_mlp_packed_bytes), got "
+                    "%lld: it was packed for another stack", (long long)pk_total_bytes(pk_ks0(dims[0]), n_layers), (long long)packed_bytes);
     MlpPackedArgs a{};
     a.nout = dims[n_layers];
     // a masked head whose logits are not asked for is computed for its valid columns only (see sp_mlp_forward)
@@ -600,7 +613,9 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
         if (a.b[i] != nullptr && !aligned16(a.b[i]))
             return fail(SP_ERR_ALIGN, "sp_mlp_forward_packed: biases[%d] is not 16-byte aligned", i);
     }
-    int rc = require_gfx950(__func__);
+    int rc = mlp_set_philox(a.ph, philox, batch, dims[n_layers], __func__);
+    if (rc != SP_OK) return rc;
+    rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
     a.x = x; a.packed = packed; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.out_stride = dims[n_layers];

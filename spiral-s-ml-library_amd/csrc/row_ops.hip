@@ -5,6 +5,7 @@
 //
 // Semantics follow ml/primitives.spi (row_ :423-512, local_* :295-348 and :701-814).
 #include "common.h"
+#include "philox.h"
 
 // The scan/sampling results are compared bit for bit with a CPU restatement, so no operation in
 // this file may be fused or re-associated.
@@ -36,6 +37,7 @@ struct RowArgs {
     int op;                // sp_row_op
     int mask_size;         // columns j < mask_size are valid for the masked ops
     int want_stats;        // rowmax/rowsum are of softmax(x) regardless of op (fused pipeline)
+    float threshold;       // l1_normalize: the norm a row is clamped to
     // philox
     unsigned long long seed;
     int philox_mode;       // -1: none
@@ -46,36 +48,6 @@ struct RowArgs {
     long member_rows;                  // 0: one run; else the rows are stacked runs of member_rows rows each
     unsigned long long member_draws;   // extra draw offset per run
 };
-
-// Philox4x32-10 (Salmon et al., SC'11) with cuRAND's counter layout: key = seed, counter =
-// (group, 0, subsequence_lo, subsequence_hi); returns word `word` of the group, mapped to (0, 1]
-// like curand_uniform (corecuda/random.spi:22-32,84).
-__device__ __forceinline__ void philox_words(unsigned long long seed, unsigned long long subsequence,
-                                             unsigned long long group, unsigned (&w)[4]) {
-    unsigned c0 = (unsigned)group, c1 = (unsigned)(group >> 32), c2 = (unsigned)subsequence,
-             c3 = (unsigned)(subsequence >> 32);
-    unsigned k0 = (unsigned)seed, k1 = (unsigned)(seed >> 32);
-#pragma unroll
-    for (int r = 0; r < 10; ++r) {
-        if (r) {
-            k0 += 0x9E3779B9u;
-            k1 += 0xBB67AE85u;
-        }
-        unsigned hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-        unsigned hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
-        unsigned n0 = hi1 ^ c1 ^ k0, n1 = lo1, n2 = hi0 ^ c3 ^ k1, n3 = lo0;
-        c0 = n0; c1 = n1; c2 = n2; c3 = n3;
-    }
-    w[0] = c0; w[1] = c1; w[2] = c2; w[3] = c3;
-}
-
-__device__ __forceinline__ float philox_uniform(unsigned long long seed, unsigned long long subsequence,
-                                                unsigned long long group, int word) {
-    unsigned w[4];
-    philox_words(seed, subsequence, group, w);
-    const unsigned v = word == 0 ? w[0] : word == 1 ? w[1] : word == 2 ? w[2] : w[3];
-    return (float)v * 2.3283064e-10f + 1.1641532e-10f;
-}
 
 // Two standard normals from two 32-bit draws, the Box-Muller form of curand_normal (corecuda/random.spi:85):
 // u = x 2^-32 + 2^-33, v = 2 pi (y 2^-32 + 2^-33), (sqrt(-2 ln u) sin v, sqrt(-2 ln u) cos v).  The library's own
@@ -90,42 +62,23 @@ __device__ __forceinline__ void box_muller(unsigned x, unsigned y, float& n0, fl
     n1 = s * cs;
 }
 
-// Which (subsequence, 4-word group) the reference's sampling op uses for row r: every thread of
-// the row draws once per element it holds and the draw attached to column 0 wins
-// (ml/primitives.spi:786-791), i.e. the first draw of the row's lane 0 in that row-iteration.
-__device__ __forceinline__ float reference_row_uniform(const RowArgs& a, long r) {
-    unsigned long long draw_offset = a.draw_offset;
-    if (a.member_rows > 0) {              // stacked runs (ensemble members): each restarts the row walk, later in the stream
-        draw_offset += (unsigned long long)(r / a.member_rows) * a.member_draws;
-        r = r % a.member_rows;
-    }
-    const long t = a.cols / 4;            // threads per row in the reference
-    const long per_iter = a.tpb / t;      // rows per block-iteration
-    unsigned long long sub, group;
-    if (a.philox_mode == SP_PHILOX_BLOCK) {
-        sub = (r % per_iter) * t;
-        group = r / per_iter;
-    } else if (a.philox_mode == SP_PHILOX_GRID) {
-        const long it = r / per_iter;
-        sub = (it % a.blocks) * a.tpb + (r % per_iter) * t;
-        group = it / a.blocks;
-    } else if (a.philox_mode == SP_PHILOX_GATHER) {  // row r belongs to thread r
-        const long lt = r % a.tpb;
-        sub = (r / a.tpb) * a.tpb + (lt % per_iter) * t;
-        group = lt / per_iter;
-    } else {  // SP_PHILOX_LAYER: block b = r / rows_per_block walks its own slice (ml/layers.spi:339-344)
-        const long b = r / a.rows_per_block, rb = r % a.rows_per_block;
-        sub = b * a.tpb + (rb % per_iter) * t;
-        group = rb / per_iter;
-    }
-    // the generator is `draw_offset` draws in; this row uses the first draw of its 4-draw group
-    return philox_uniform(a.seed, sub, group + draw_offset / 4, (int)(draw_offset % 4));
-}
-
 // exp(x) = 2^(x * log2 e) on the hardware exp2 unit; relative error about 1e-6 for |x| < 20.
 __device__ __forceinline__ float fast_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f); }
 
 __device__ __forceinline__ float sum4(const float (&v)[4]) { return ((v[0] + v[1]) + v[2]) + v[3]; }
+
+// x / s for many x and one s as x * scale * (1 / (s * scale)): one division per row, and `scale` (a power of two, so
+// both products by it are exact) keeps the reciprocal finite when s lies below 2^-126, where 1 / s alone would be
+// +inf and every quotient inf or NaN.  The quotients differ from a correctly rounded x / s by at most one unit in
+// the last place.
+struct RowDivisor {
+    float scale, inv;
+    __device__ __forceinline__ explicit RowDivisor(float s) {
+        scale = fabsf(s) < 4.7019774e-38f ? 1.8446744e19f : 1.f;     // below 2^-124: times 2^64
+        inv = 1.f / (s * scale);
+    }
+    __device__ __forceinline__ float operator()(float x) const { return (x * scale) * inv; }
+};
 
 template <int T, int C>
 __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
@@ -232,14 +185,30 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
             // one division per row, then a multiplication per element (a correctly rounded division is ten
             // instructions; the quotients differ from p / s by at most one unit in the last place)
-            const float inv_len = 1.f / (float)limit, inv = 1.f / s;
+            const float inv_len = 1.f / (float)limit;
+            const RowDivisor over_s(s);
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
                 for (int k = 0; k < 4; ++k) {
                     const int j = c * 4 * T + 4 * l + k;
-                    p[c][k] = (j < limit) ? (s != 0.f ? p[c][k] * inv : inv_len) : 0.f;
+                    p[c][k] = (j < limit) ? (s != 0.f ? over_s(p[c][k]) : inv_len) : 0.f;
                 }
+        } else if (op == SP_ROW_L1_NORMALIZE) {
+            // local_l1_normalize (ml/primitives.spi:725-729): |x|, scaled down to norm `threshold` when its sum is above it
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = fabsf(v[c][k]);
+                s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
+            }
+            s = group_reduce<T>(s, [](float x, float y) { return x + y; });
+            const float f = s > a.threshold ? a.threshold / s : 1.f;
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+#pragma unroll
+                for (int k = 0; k < 4; ++k) p[c][k] = f * p[c][k];
         } else if (op == SP_ROW_LN_L2) {
             float s = 0.f;
 #pragma unroll
@@ -250,11 +219,11 @@ __global__ __launch_bounds__(ROW_THREADS) void row_kernel(const RowArgs a) {
                 s = (c == 0) ? sum4(q) : s + sum4(q);
             }
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
-            const float inv = 1.f / s;
+            const RowDivisor over_s(s);
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
-                for (int k = 0; k < 4; ++k) p[c][k] = (s != 0.f) ? v[c][k] * inv : 0.f;
+                for (int k = 0; k < 4; ++k) p[c][k] = (s != 0.f) ? over_s(v[c][k]) : 0.f;
         } else {  // identity and the scans act on the raw input
 #pragma unroll
             for (int c = 0; c < C; ++c)
@@ -434,12 +403,13 @@ __device__ __forceinline__ void row_softmax_body(const RowArgs& a) {
                 s = (c == 0) ? sum4(p[c]) : s + sum4(p[c]);
             }
             s = group_reduce<T>(s, [](float x, float y) { return x + y; });
-            const float inv_len = 1.f / (float)limit, inv = 1.f / s;      // as in row_kernel: one division per row
+            const float inv_len = 1.f / (float)limit;
+            const RowDivisor over_s(s);                                  // as in row_kernel: one division per row
 #pragma unroll
             for (int c = 0; c < C; ++c)
 #pragma unroll
                 for (int k = 0; k < 4; ++k)
-                    p[c][k] = (c * 4 * T + 4 * l + k < limit) ? (s != 0.f ? p[c][k] * inv : inv_len) : 0.f;
+                    p[c][k] = (c * 4 * T + 4 * l + k < limit) ? (s != 0.f ? over_s(p[c][k]) : inv_len) : 0.f;
         } else {
 #pragma unroll
             for (int c = 0; c < C; ++c) {
@@ -857,30 +827,6 @@ struct RowKernelNames {
 
 using namespace sp;
 
-static int set_philox(RowArgs& a, const sp_philox_t* philox, int64_t rows, int64_t cols, const char* fn) {
-    if (philox->mode < SP_PHILOX_BLOCK || philox->mode > SP_PHILOX_LAYER)
-        return fail(SP_ERR_ARG, "%s: unknown philox mode %d", fn, philox->mode);
-    const int64_t t = cols / 4;
-    if (philox->threads_per_block <= 0 || philox->threads_per_block % t != 0)
-        return fail(SP_ERR_ARG, "%s: threads_per_block (%d) must be a positive multiple of cols/4 (%lld)", fn,
-                    philox->threads_per_block, (long long)t);
-    if (philox->mode == SP_PHILOX_GRID && philox->blocks_per_grid <= 0)
-        return fail(SP_ERR_ARG, "%s: blocks_per_grid must be positive", fn);
-    if (philox->member_rows < 0 || (philox->member_rows > 0 && rows % philox->member_rows != 0))
-        return fail(SP_ERR_ARG, "%s: member_rows (%lld) must divide rows (%lld)", fn, (long long)philox->member_rows,
-                    (long long)rows);
-    const int64_t run_rows = philox->member_rows > 0 ? philox->member_rows : rows;
-    if (philox->mode == SP_PHILOX_LAYER && (philox->rows_per_block <= 0 || run_rows % philox->rows_per_block != 0))
-        return fail(SP_ERR_ARG, "%s: rows_per_block (%d) must be positive and divide the rows of a run (%lld)", fn,
-                    philox->rows_per_block, (long long)run_rows);
-    a.seed = philox->seed; a.philox_mode = philox->mode; a.tpb = philox->threads_per_block;
-    a.blocks = philox->blocks_per_grid; a.rows_per_block = philox->rows_per_block;
-    a.draw_offset = philox->offset;
-    a.member_rows = philox->member_rows;
-    a.member_draws = philox->member_draws;
-    return SP_OK;
-}
-
 extern "C" int sp_philox_uniforms(const sp_philox_t* philox, float* u_out, int64_t rows, int64_t cols, void* stream) {
     SP_REQUIRE_PTR(u_out);
     if (philox == nullptr) return fail(SP_ERR_NULL, "sp_philox_uniforms: philox is NULL");
@@ -928,6 +874,18 @@ extern "C" int sp_row_map_f32(int op, const float* x, float* out, int64_t rows, 
     a.x = x; a.out = out; a.rows = rows; a.cols = (int)cols; a.op = op; a.mask_size = masked ? mask_size : (int)cols;
     a.philox_mode = -1;
     if (op == SP_ROW_SOFTMAX) return launch_row<true>(a, (hipStream_t)stream, __func__);   // the fused kernel's first half
+    return launch_row<false>(a, (hipStream_t)stream, __func__);
+}
+
+extern "C" int sp_row_l1_normalize(const float* x, float* out, int64_t rows, int64_t cols, float threshold, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(out);
+    int rc = check_rows_cols(__func__, rows, cols);
+    if (rc != SP_OK) return rc;
+    if (!(threshold > 0.f)) return fail(SP_ERR_ARG, "sp_row_l1_normalize: threshold must be positive, got %g", (double)threshold);
+    RowArgs a{};
+    a.x = x; a.out = out; a.rows = rows; a.cols = (int)cols; a.op = SP_ROW_L1_NORMALIZE; a.mask_size = (int)cols;
+    a.threshold = threshold; a.philox_mode = -1;
     return launch_row<false>(a, (hipStream_t)stream, __func__);
 }
 

@@ -70,17 +70,21 @@ SIGNATURES = {
     "sp_row_reduce_f32": (C.c_int, [C.c_int, C.c_int, C.c_int, _P, _P, _I64, _I64, _P]),
     "sp_row_binarize": (C.c_int, [_P, _P, _I64, _I64, C.c_uint32, _P]),
     "sp_map_f32": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
+    "sp_row_l1_normalize": (C.c_int, [_P, _P, _I64, _I64, C.c_float, _P]),
+    "sp_reduce": (C.c_int, [C.c_int, C.c_int, _P, _P, _I64, _P, _I64, _P]),
+    "sp_reduce_status": (C.c_int, [_P, _I64, C.POINTER(C.c_int64), _P]),
+    "sp_reduce_set_poll_limit": (C.c_int, [_I64]),
     "sp_reduce_sum": (C.c_int, [C.c_int, _P, _P, _I64, _P, _I64, _P]),
     "sp_reduce_workspace_bytes": (C.c_int64, []),
     "sp_reduce_sum_static": (C.c_int, [C.c_int, _P, _P, _I64, _P]),
     "sp_reduce_sum_static_max_n": (C.c_int64, []),
     "sp_transpose_inner_b32": (C.c_int, [_P, _P, _I64, _I64, _I64, _P]),
-    "sp_mlp_forward": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
-                                 _I64, _I32, _I32, _P]),
+    "sp_mlp_forward": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(_P), C.POINTER(C.c_int32), _P,
+                                 C.POINTER(PhiloxConfig), _P, _P, _P, _I64, _I32, _I32, _P]),
     "sp_mlp_packed_bytes": (C.c_int64, [_I32, C.POINTER(C.c_int32)]),
     "sp_mlp_pack_weights": (C.c_int, [C.c_int, _I32, C.POINTER(_P), C.POINTER(C.c_int32), _P, _I64, _P]),
-    "sp_mlp_forward_packed": (C.c_int, [C.c_int, _P, _I32, _P, C.POINTER(_P), C.POINTER(C.c_int32), _P, _P, _P, _P,
-                                        _I64, _I32, _I32, _P]),
+    "sp_mlp_forward_packed": (C.c_int, [C.c_int, _P, _I32, _P, _I64, C.POINTER(_P), C.POINTER(C.c_int32), _P,
+                                        C.POINTER(PhiloxConfig), _P, _P, _P, _I64, _I32, _I32, _P]),
 }
 
 
@@ -100,7 +104,7 @@ def load(path=LIB_PATH):
 LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_row_map_f32", "sp_row_map_i32",
                       "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_resample_philox",
                       "sp_row_reduce_f32", "sp_cem_update_mask",
-                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_reduce_sum_static", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
+                      "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_reduce", "sp_row_l1_normalize", "sp_reduce_sum_static", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
                       "sp_mlp_forward_packed"))
 
 

@@ -69,7 +69,7 @@ def pack_weights(weights, into=None):
 
 
 def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None, mask_size=0, want_logits=False,
-                policy_out=None, action_out=None, packed=None):
+                policy_out=None, action_out=None, packed=None, rng=None):
     """policy, action[, logits] = fused forward of relu-MLP + head + discrete sampling.
 
     x: (batch, in) f16/bf16; weights[i]: (out_i, in_i) of the same dtype (the B operand of A.B^T,
@@ -77,7 +77,9 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
     extension, the reference has no bias); u: (batch,) f32 uniforms in (0, 1] or None (no action).
     head: None | "softmax" | "regret_matching" | "softmax_regret_matching"; mask_size > 0 restricts
     the head to columns j < mask_size (masked_* layers, ml/layers.spi:408-432).  packed: the result of
-    pack_weights(weights) -- the stack then runs on the packed kernel and `weights` is not read."""
+    pack_weights(weights) -- the stack then runs on the packed kernel and `weights` is not read.  rng: instead of
+    u, a Philox stream (primitives.philox(...)) the head draws its uniforms from inside the kernel, row r taking
+    what primitives.philox_uniforms(rng, batch, out) hands out for it (ml/layers.spi:339-344)."""
     if packed is not None:
         n, dims = len(packed.dims) - 1, packed.dims
         if packed.dtype != x.dtype:
@@ -94,7 +96,7 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
     policy = policy_out if policy_out is not None else \
         torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device)
     action = action_out
-    if action is None and u is not None:
+    if action is None and (u is not None or rng is not None):
         action = torch.empty((batch,), dtype=torch.int32, device=x.device)
     logits = torch.empty((batch, dims[-1]), dtype=torch.float32, device=x.device) if want_logits else None
     bp = None
@@ -103,14 +105,15 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
                                 for i, b in enumerate(biases)])
     dp = (C.c_int32 * (n + 1))(*dims)
     if packed is not None:
-        check(lib.sp_mlp_forward_packed(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, ptr(packed.buffer), bp, dp,
-                                        ptr(u, torch.float32, "u"), ptr(policy, torch.float32, "policy_out"),
+        check(lib.sp_mlp_forward_packed(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, ptr(packed.buffer),
+                                        packed.buffer.numel(), bp, dp, ptr(u, torch.float32, "u"),
+                                        C.byref(rng) if rng is not None else None, ptr(policy, torch.float32, "policy_out"),
                                         ptr(action, torch.int32, "action_out"), ptr(logits), batch, HEADS[head],
                                         mask_size, stream_ptr()))
     else:
         wp = (C.c_void_p * n)(*[ptr(w, name="weights[%d]" % i) for i, w in enumerate(weights)])
         check(lib.sp_mlp_forward(_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, bp, dp, ptr(u, torch.float32, "u"),
-                                 ptr(policy, torch.float32, "policy_out"), ptr(action, torch.int32, "action_out"),
+                                 C.byref(rng) if rng is not None else None, ptr(policy, torch.float32, "policy_out"), ptr(action, torch.int32, "action_out"),
                                  ptr(logits), batch, HEADS[head], mask_size, stream_ptr()))
     out = (policy, action)
     return out + (logits,) if want_logits else out
@@ -671,7 +674,6 @@ def _build_fused_run(model, plan, ls, static_weights=False):
     probs, action = graph_extract(model)
     q, w, cols = probs.shape
     rng = ls.rng(q, w, cols)
-    u = torch.empty((q * w,), dtype=torch.float32, device=x.device)
     policy, act = _flat(probs), action.reshape(-1)
     n = len(ws)
     dims = [x.shape[1]] + [t.shape[0] for t in ws]
@@ -681,18 +683,16 @@ def _build_fused_run(model, plan, ls, static_weights=False):
         assert t.shape[1] == dims[i], "The K dimension of the A and B tensors must match."
     wp = (C.c_void_p * n)(*[ptr(t, name="weights[%d]" % i) for i, t in enumerate(ws)])
     dp = (C.c_int32 * (n + 1))(*dims)
-    args = (_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, None, dp, ptr(u), ptr(policy, torch.float32, "policy_out"),
-            ptr(act, torch.int32, "action_out"), None, x.shape[0], HEADS[head], top.size)
-    rows = q * w
-    keep = (x, ws, probs, action, u, policy, act)   # the views stay alive as long as the closure does
-
-    # A run restarts the generator from the same seed (ml/layers.spi:339-344), so the uniforms of a (model, seed)
-    # pair are the same in every run: they are drawn once, here.
-    check(lib.sp_philox_uniforms(C.byref(rng), args[6], rows, cols, stream_ptr()))
+    # The head draws its uniforms inside the kernel, from the stream a run of the reference starts at its seed
+    # (ml/layers.spi:339-344): no uniform tensor, no launch of its own, nothing carried over from run to run.
+    args = (_lib.DTYPES[x.dtype], ptr(x, name="x"), n, wp, None, dp, None, C.byref(rng),
+            ptr(policy, torch.float32, "policy_out"), ptr(act, torch.int32, "action_out"), None, x.shape[0], HEADS[head],
+            top.size)
+    keep = (x, ws, probs, action, rng, policy, act)   # the views stay alive as long as the closure does
 
     packed = pack_weights(ws) if static_weights else None
     if packed is not None and builtins.min(dims[-1], top.size or dims[-1]) <= 16:
-        pargs = args[:3] + (ptr(packed.buffer),) + args[4:]
+        pargs = args[:3] + (ptr(packed.buffer), packed.buffer.numel()) + args[4:]
         keep = keep + (packed,)
 
         def run_packed():

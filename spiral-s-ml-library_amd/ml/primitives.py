@@ -61,6 +61,17 @@ def ln_l2(x, out=None):
     return _row_map(_lib.ROW_LN_L2, x, out)
 
 
+def l1_normalize(x, threshold, out=None):
+    """row_map (local_l1_normalize threshold) (ml/primitives.spi:725-729): |x|, scaled down to l1 norm `threshold`
+    where a row's norm is above it (the decay of the average policy, ml/cfr.spi:244)."""
+    rows, cols = _rows_cols(x)
+    if out is None:
+        out = torch.empty_like(x)
+    check(lib.sp_row_l1_normalize(ptr(x, torch.float32, "x"), ptr(out, torch.float32, "out"), rows, cols, threshold,
+                                  stream_ptr()))
+    return out
+
+
 def regret_matching(x, out=None):
     """row_map local_regret_matching (ml/primitives.spi:718-722)."""
     return _row_map(_lib.ROW_REGRET_MATCHING, x, out)
@@ -332,8 +343,13 @@ def reduce_2d(neutral_element, f, from_, to=None):
 
 def reduce_max(x):
     """`grid_reduce grid 0 max norms` of the CEM update's weight-norm print (ml/cem.spi:140): the largest element of a
-    tensor whose element count is a multiple of 4, as a 0-d tensor (all elements treated as one row)."""
-    return row_reduce(x.reshape(1, -1), "max")[0]
+    tensor, as a 0-d tensor; one launch over the whole device (sp_reduce)."""
+    return reduce("max", x)
+
+
+def reduce_min(x):
+    """`reduce limit.max min` over a whole tensor (ml/primitives.spi:176-197)."""
+    return reduce("min", x)
 
 
 def grid_transpose(x, out=None):
@@ -354,18 +370,43 @@ def map(op, x, out=None):  # noqa: A001  (the reference's name, ml/primitives.sp
 _workspace = {}
 
 
-def reduce_sum(x):
-    """reduce 0 (+) / grid_reduce grid 0 (+) over a whole tensor (ml/primitives.spi:176-197).
-    f32, i32 or u64 (carried as int64 by torch).  Returns a 0-d tensor on the device."""
-    code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
-    key = x.device.index
+def _reduce_workspace(device):
+    key = device.index
     if key not in _workspace:
-        # zero-filled once: the kernel keeps the blocks' valid marks in it and leaves them at zero after every call
-        _workspace[key] = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=x.device)
-    ws = _workspace[key]
+        # zero-filled once: the give-up counter behind the blocks' slots starts from what it finds
+        _workspace[key] = torch.zeros(lib.sp_reduce_workspace_bytes(), dtype=torch.uint8, device=device)
+    return _workspace[key]
+
+
+def reduce(f, x):  # noqa: A001  (the reference's name, ml/primitives.spi:176)
+    """`reduce neutral f` / `grid_reduce grid neutral f` over a whole tensor (ml/primitives.spi:136-197) for f in
+    {"+", "*", "max", "min"} with its own neutral element.  f32, i32 or u64 (carried as int64 by torch).  Returns a
+    0-d tensor on the device."""
+    op = {"+": _lib.REDUCE_SUM, "sum": _lib.REDUCE_SUM, "*": _lib.REDUCE_PROD, "prod": _lib.REDUCE_PROD,
+          "max": _lib.REDUCE_MAX, "min": _lib.REDUCE_MIN}[f]
+    code = {torch.float32: 0, torch.int32: 1, torch.int64: 2}[x.dtype]
+    ws = _reduce_workspace(x.device)
     out = torch.empty(4, dtype=x.dtype, device=x.device)  # 16-byte aligned scalar slot
-    check(lib.sp_reduce_sum(code, ptr(x, name="x"), ptr(out), x.numel(), ptr(ws), ws.numel(), stream_ptr()))
+    check(lib.sp_reduce(op, code, ptr(x, name="x"), ptr(out), x.numel(), ptr(ws), ws.numel(), stream_ptr()))
     return out[0]
+
+
+grid_reduce = reduce
+
+
+def reduce_sum(x):
+    """reduce 0 (+) / grid_reduce grid 0 (+) over a whole tensor (ml/primitives.spi:176-197)."""
+    return reduce("+", x)
+
+
+def reduce_give_ups(device=None):
+    """How often a reduce on this device's workspace gave up waiting for its partial results (sp_reduce_status; waits
+    for the current stream).  0 unless other work kept part of a launch off the device for milliseconds."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    ws = _reduce_workspace(dev)
+    n = C.c_int64(0)
+    check(lib.sp_reduce_status(ptr(ws), ws.numel(), C.byref(n), stream_ptr()))
+    return n.value
 
 
 def reduce_sum_static(x, out):

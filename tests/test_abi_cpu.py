@@ -123,6 +123,16 @@ def test_misc_argument_errors(L):
     assert lib.sp_map_f32(0, p, p, 6, None) == -2
     assert lib.sp_map_f32(0, None, p, 8, None) == -1
     assert lib.sp_reduce_sum(0, p, p, 8, p, 16, None) == -5
+    big = lib.sp_reduce_workspace_bytes()
+    assert lib.sp_reduce(4, 0, p, p, 8, p, big, None) == -5 and "op must be" in _err(L)     # no whole-tensor average
+    assert lib.sp_reduce(2, 3, p, p, 8, p, big, None) == -4
+    assert lib.sp_reduce(2, 0, p, p, 0, p, big, None) == -2
+    assert lib.sp_reduce(2, 0, p, p, 8, None, big, None) == -1
+    assert lib.sp_reduce_status(p, 16, C.byref(C.c_int64()), None) == -5
+    assert lib.sp_reduce_status(p, big, None, None) == -1
+    assert lib.sp_reduce_set_poll_limit(20000000) == -5 and lib.sp_reduce_set_poll_limit(0) == 0
+    assert lib.sp_row_l1_normalize(p, p, 4, 8, 0.0, None) == -5 and "threshold" in _err(L)
+    assert lib.sp_row_l1_normalize(p, None, 4, 8, 1.0, None) == -1
     assert lib.sp_reduce_workspace_bytes() >= 1024
     assert lib.sp_transpose_inner_b32(p, p, 1, 8, 8, None) == -5
     assert lib.sp_transpose_inner_b32(p, C.c_void_p(0x4000), 0, 8, 8, None) == -2
@@ -134,8 +144,8 @@ def test_mlp_argument_errors(L):
     p = C.c_void_p(0x5000)
     w = (C.c_void_p * 2)(p, p)
     dims = lambda *d: (C.c_int32 * len(d))(*d)
-    call = lambda dtype=1, x=p, n=2, ws=w, d=dims(32, 64, 3), u=None, pol=p, act=None, batch=8, head=3, mask=0: \
-        lib.sp_mlp_forward(dtype, x, n, ws, None, d, u, pol, act, None, batch, head, mask, None)
+    call = lambda dtype=1, x=p, n=2, ws=w, d=dims(32, 64, 3), u=None, ph=None, pol=p, act=None, batch=8, head=3, mask=0: \
+        lib.sp_mlp_forward(dtype, x, n, ws, None, d, u, ph, pol, act, None, batch, head, mask, None)
     assert call(dtype=0) == -4
     assert call(x=None) == -1
     assert call(n=0) == -5 and call(n=9) == -5
@@ -148,6 +158,14 @@ def test_mlp_argument_errors(L):
     assert call(mask=4) == -5
     assert call(act=p) == -1  # action without u
     assert call(ws=(C.c_void_p * 2)(p, None)) == -1
+    # a head that draws its own uniforms: one of u / philox, and the output width must be a row width of the
+    # reference's sampling op (a multiple of 4) whose 4-column thread groups divide the block
+    ph = L.PhiloxConfig(12344321, 0, L.PHILOX_LAYER, 256, 24, 8, 0, 0)
+    assert call(act=p, u=p, ph=C.byref(ph)) == -5 and "at most one" in _err(L)
+    assert call(act=p, ph=C.byref(ph)) == -5 and "multiple of 4" in _err(L)
+    assert call(act=p, ph=C.byref(ph), d=dims(32, 64, 64), batch=24 * 8 + 1) == -5 and "rows_per_block" in _err(L)
+    bad = L.PhiloxConfig(12344321, 0, 9, 256, 24, 8, 0, 0)
+    assert call(act=p, ph=C.byref(bad), d=dims(32, 64, 64)) == -5 and "philox mode" in _err(L)
 
 
 def test_packed_mlp_argument_errors(L):
@@ -167,8 +185,13 @@ def test_packed_mlp_argument_errors(L):
     assert lib.sp_mlp_pack_weights(1, 4, w, d, p, 1000, None) == -5 and "must hold" in _err(L)
     assert lib.sp_mlp_pack_weights(1, 4, w, dims(32, 256, 128, 256, 3), p, 1 << 20, None) == -6
     assert lib.sp_mlp_pack_weights(1, 4, (C.c_void_p * 4)(p, None, p, p), d, p, 1 << 20, None) == -1
-    call = lambda dtype=1, x=p, n=4, pk=p, dd=d, u=None, pol=p, act=None, logits=None, batch=8, head=1, mask=0: \
-        lib.sp_mlp_forward_packed(dtype, x, n, pk, None, dd, u, pol, act, logits, batch, head, mask, None)
+    size = lib.sp_mlp_packed_bytes(4, d)
+    call = lambda dtype=1, x=p, n=4, pk=p, nbytes=size, dd=d, u=None, pol=p, act=None, logits=None, batch=8, head=1, mask=0: \
+        lib.sp_mlp_forward_packed(dtype, x, n, pk, nbytes, None, dd, u, None, pol, act, logits, batch, head, mask, None)
+    # a buffer packed for another stack (another layer count, another class of first width) has another size
+    assert call(nbytes=lib.sp_mlp_packed_bytes(3, dims(32, 256, 256, 3))) == -5 and "another stack" in _err(L)
+    assert call(nbytes=lib.sp_mlp_packed_bytes(4, dims(64, 256, 256, 256, 3))) == -5
+    assert call(nbytes=size + 16) == -5
     assert call(dtype=0) == -4
     assert call(pk=None) == -1
     assert call(batch=0) == -2

@@ -302,13 +302,13 @@ def test_four_wave_kernel_on_tall_shapes_is_exact_on_integers(MM, dtype):
 
 
 @pytest.mark.parametrize("m,n,k", [(65536, 256, 1152), (65536, 2048, 512), (4096, 512, 8192), (6144, 8192, 256),
-                                   (8192, 6144, 1152)])
+                                   (8192, 6144, 1152), (8192, 8192, 128)])
 def test_streamed_and_written_through_outputs_are_exact_on_integers(MM, m, n, k):
     """The stores of C carry a cache policy chosen per launch: written through the L2, or -- operands of 140 MiB and
     more, or an output of 384 MiB and more -- streamed past the caches.  The streamed form on the eight-wave kernel
     (144 MiB of A), on the persistent four-wave kernel in two phase groups (512 MiB of C; a short-K problem with three
-    tiles per compute unit; the two-stage persistent form at 18 K-tiles) and the written-through form on a square-ish problem, each with every epilogue option,
-    exact on small integers."""
+    tiles per compute unit; the two-stage persistent form at 18 K-tiles and at its shortest, two K-tiles, where every
+    tile boundary hands over to the next tile's fetches at its first K-tile) and the written-through form on a square-ish problem, each with every epilogue option, exact on small integers."""
     announce("gemm store policies, integer problems %dx%dx%d" % (m, n, k))
     t = TORCH["bf16"]
     a = ((np.arange(m * k, dtype=np.int64).reshape(m, k) * 7 + 3) % 5 - 2).astype(np.float32)

@@ -258,3 +258,44 @@ def test_results_do_not_change_from_run_to_run(LY, dims, mask, with_bias, packed
         for a, b in zip(first, again):
             assert torch.equal(a, b)
 
+
+
+@pytest.mark.parametrize("dims,mask,batch,want_logits,packed,mode", [
+    ([32, 96, 160, 8], 0, 24 * 13, False, False, "layer"),               # the general kernel
+    ([128, 256, 256, 64], 40, 24 * 9, True, False, "layer"),             # 256-wide hidden layers, wide head
+    ([32, 256, 256, 256, 64], 3, 16384, False, False, "layer"),          # feature-split kernel, head of 3 valid columns of 64
+    ([32, 256, 256, 256, 64], 3, 16384, False, True, "layer"),           # the same on packed weights
+    ([32, 256, 256, 256, 4], 0, 1000, False, True, "block"),             # packed, plain head, the block-level stream
+    ([64, 256, 256, 16], 0, 40000, False, False, "grid"),                # more rows than one round of workgroups
+])
+def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed, mode):
+    """A head given a Philox stream instead of a tensor of uniforms (the reference seeds one generator per thread
+    and the sampling node draws in the kernel, ml/layers.spi:339-344): every row must use exactly the uniform
+    sp_philox_uniforms hands out for it -- same policy bits, same actions as the run that reads those uniforms
+    from a tensor -- and those uniforms are the stream the golden sampled indices pin."""
+    from ml import _lib, primitives
+    from oracle import philox as ophilox
+    announce("mlp philox head dims=%s mask=%d batch=%d packed=%s mode=%s" % (dims, mask, batch, packed, mode))
+    rng = np.random.default_rng(sum(dims) + batch)
+    x, ws, _ = make_problem(rng, batch, dims, "f16")
+    xd, wd = dev(x, torch.float16), [dev(w, torch.float16) for w in ws]
+    pk = LY.pack_weights(wd) if packed else None
+    cols = dims[-1]
+    if mode == "layer":
+        q = 24
+        cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=q, rows_per_block=batch // q, offset=8)
+        want_u = ophilox.row_uniforms_layer(q, batch // q, cols, offset=8)
+    elif mode == "block":
+        cfg = primitives.philox(_lib.PHILOX_BLOCK)
+        want_u = ophilox.row_uniforms_block(batch, cols)
+    else:
+        cfg = primitives.philox(_lib.PHILOX_GRID, blocks_per_grid=24)
+        want_u = ophilox.row_uniforms_grid(batch, cols, blocks=24)
+    u = primitives.philox_uniforms(cfg, batch, cols)
+    assert (host(u) == np.asarray(want_u, dtype=np.float32).reshape(-1)).all()
+    head = "softmax_regret_matching"
+    with_u = LY.mlp_forward(xd, wd, None, head, u, mask, want_logits, packed=pk)
+    with_rng = LY.mlp_forward(xd, wd, None, head, None, mask, want_logits, packed=pk, rng=cfg)
+    for a, b in zip(with_u, with_rng):
+        assert torch.equal(a, b)
+    assert (host(with_rng[1]) == orow.discrete_sampling(host(with_rng[0]), host(u))).all()

@@ -505,3 +505,109 @@ def test_results_do_not_change_from_run_to_run(P):
             assert torch.equal(first[k], again[k]), k
         assert torch.equal(P.reduce_sum(x), total)
 
+
+
+@pytest.mark.parametrize("rows,cols", [(3, 12), (130, 64), (257, 256), (7, 1000)])
+def test_l1_normalize(P, rows, cols):
+    """row_map (local_l1_normalize threshold) (ml/primitives.spi:725-729) against the oracle; rows on both sides of the
+    threshold, and in place."""
+    announce("l1_normalize rows=%d cols=%d" % (rows, cols))
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal((rows, cols)).astype(np.float32)
+    x[::2] *= np.float32(0.01)                       # every other row stays under the threshold
+    thr = float(np.abs(x).sum(axis=1).mean())
+    want = orow.l1_normalize(x, thr)
+    xd = dev(x)
+    got = host(P.l1_normalize(xd, thr))
+    assert ogemm.rel_frobenius(got, want) < FLOAT_TOL and (got >= 0).all()
+    norms = np.abs(x).sum(axis=1)
+    assert (got[norms <= thr * 0.999] == np.abs(x)[norms <= thr * 0.999]).all()       # untouched rows: exact |x|
+    assert np.abs(got[norms > thr].sum(axis=1) - thr).max() < 1e-5 * thr * cols ** 0.5
+    P.l1_normalize(xd, thr, out=xd)
+    assert (host(xd) == got).all()
+
+
+@pytest.mark.parametrize("cols", [4, 64, 256, 1024])
+def test_rows_whose_sum_is_subnormal(P, cols):
+    """Regret matching and ln_l2 divide by a row sum.  The kernels do that with one reciprocal per row; a sum below
+    2^-126 must still give the quotients (a distribution), not infinities and NaNs."""
+    announce("subnormal row sums cols=%d" % cols)
+    tiny = np.float32(2.0 ** -140)
+    x = np.full((6, cols), -1.0, dtype=np.float32)
+    x[0, 0], x[0, 1] = tiny, 3 * tiny                 # sum 2^-138
+    x[1, cols - 1] = np.float32(2.0 ** -149)          # the smallest positive number alone
+    x[2, :2] = np.float32(2.0 ** -127)                # sum 2^-126: the first normal number
+    x[3, :4] = [1.0, 2.0, 3.0, 2.0]                   # an ordinary row between them
+    x[4, 0], x[4, 2] = np.float32(2.0 ** -130), np.float32(2.0 ** -129)
+    x[5, :] = 0                                       # sum exactly 0: the uniform branch
+    xd = dev(x)
+    want = orow.regret_matching(x)
+    got = host(P.regret_matching(xd))
+    assert np.isfinite(got).all() and np.abs(got - want).max() <= 2e-7 and np.abs(got.sum(axis=1) - 1).max() < 1e-6
+    assert (got[0, :2] == [0.25, 0.75]).all() and got[1, cols - 1] == 1 and (got[5] == np.float32(1) / np.float32(cols)).all()
+    u = np.full(6, 0.5, dtype=np.float32)
+    probs, sample = P.regret_matching_and_discrete_sampling(xd, u=dev(u))[:2]
+    assert (host(probs) == got).all()                                         # the fused kernel: the same bits
+    assert (host(sample)[:3] == [1, cols - 1, 0]).all()
+    size = min(cols, 3)
+    assert np.isfinite(host(P.masked_regret_matching(xd, size))).all()
+    # ln_l2: x / sum(x^2) with a subnormal sum of squares; the quotients themselves are large but finite
+    y = np.zeros((2, cols), dtype=np.float32)
+    y[0, 0], y[0, 1] = np.float32(2.0 ** -68), np.float32(2.0 ** -70)        # squares 2^-136, 2^-140
+    y[1, :2] = [3.0, 4.0]
+    got = host(P.ln_l2(dev(y)))
+    want = orow.ln_l2(y)
+    assert np.isfinite(got).all() and ogemm.rel_frobenius(got, want) < FLOAT_TOL
+
+
+@pytest.mark.parametrize("n", [1, 5, 4096, 262144 + 3, 65536 * 256])
+def test_whole_tensor_reduce_ops(P, n):
+    """`reduce neutral f` over the whole device for f in +, *, max, min (ml/primitives.spi:136-197; `grid_reduce grid 0
+    max`, ml/cem.spi:140): integers exact, float max / min exact, float product against float64."""
+    announce("reduce ops n=%d" % n)
+    rng = np.random.default_rng(n + 1)
+    xf = rng.standard_normal(n, dtype=np.float32)
+    xd = dev(xf)
+    assert float(P.reduce_max(xd)) == float(xf.max()) and float(P.reduce_min(xd)) == float(xf.min())
+    assert float(P.reduce("max", xd)) == float(orow.reduce_all(xf, "max"))
+    near_one = (1 + rng.standard_normal(min(n, 1 << 16), dtype=np.float32) * np.float32(1e-3)).astype(np.float32)
+    want = float(near_one.astype(np.float64).prod())
+    assert abs(float(P.reduce("*", dev(near_one))) - want) <= 1e-4 * abs(want)
+    xi = rng.integers(-2 ** 30, 2 ** 30, size=n, dtype=np.int32)
+    xid = dev(xi)
+    assert int(P.reduce("max", xid)) == int(xi.max()) and int(P.reduce("min", xid)) == int(xi.min())
+    assert int(P.reduce("+", xid)) == int(orow.reduce_all(xi, "+"))           # wraps around like the device's adds
+    small = rng.integers(-3, 4, size=min(n, 4096), dtype=np.int32)
+    assert int(P.reduce("*", dev(small))) == int(orow.reduce_all(small, "*"))
+    xu = rng.integers(0, 2 ** 62, size=min(n, 1 << 20), dtype=np.int64)
+    xud = dev(xu)
+    assert int(P.reduce("max", xud)) == int(xu.max()) and int(P.reduce("min", xud)) == int(xu.min())
+    # all negative floats / the lowest int: the neutral elements are -inf and the type's minimum, not 0
+    neg = -np.abs(xf) - 1
+    assert float(P.reduce_max(dev(neg))) == float(neg.max())
+    assert int(P.reduce("max", dev(np.full(max(n, 4), -2 ** 31, dtype=np.int32)))) == -2 ** 31
+
+
+def test_reduce_gives_up_cleanly_and_recovers(P):
+    """The wait at the end of a whole-tensor reduce is bounded.  With a bound below zero the collecting workgroup does
+    not wait at all, so it stops before the other workgroups of a 256 MiB sum have published: the result is a NaN, the
+    workspace's give-up counter goes up, every kernel still runs to its end, and the next call -- which finds
+    whatever the late workgroups left in their slots -- is right again."""
+    from ml import _lib
+    announce("reduce give-up")
+    x = torch.ones(1 << 26, dtype=torch.float32, device="cuda")
+    torch.cuda.synchronize()
+    before = P.reduce_give_ups()
+    assert float(P.reduce_sum(x)) == float(1 << 26)
+    _lib.check(_lib.lib.sp_reduce_set_poll_limit(-1))
+    try:
+        gave_up = P.reduce_sum(x)
+        torch.cuda.synchronize()
+    finally:
+        _lib.check(_lib.lib.sp_reduce_set_poll_limit(0))
+    assert np.isnan(float(gave_up))
+    assert P.reduce_give_ups() == before + 1
+    for _ in range(3):
+        assert float(P.reduce_sum(x)) == float(1 << 26)
+        assert int(P.reduce("max", x.view(torch.int32))) == int(np.float32(1).view(np.int32))
+    assert P.reduce_give_ups() == before + 1

@@ -260,3 +260,34 @@ def test_row_reduce_by_hand():
     assert row_ops.row_reduce(x, "average").tolist() == [0.625, 2.0]
     assert row_ops.row_reduce(x, "sum", "square", "sqrt").tolist() == [np.float32(np.sqrt(14.25)), 4.0]
     assert row_ops.row_reduce(x, "max", "abs").tolist() == [3.0, 2.0]
+
+
+def test_l1_normalize_by_hand():
+    # (ml/primitives.spi:725-729) rows 0 and 1: l1 norm 8 > 4 -> halved, signs dropped; row 2: norm 2 <= 4 -> |x| as is;
+    # row 3: norm exactly at the threshold is not scaled; an l2 clamp would leave row 0 (l2 norm 4) untouched
+    x = np.array([[2, -2, 2, -2], [8, 0, 0, 0], [-1, 0.5, 0, -0.5], [1, -1, 1, -1]], dtype=np.float32)
+    want = np.array([[1, 1, 1, 1], [4, 0, 0, 0], [1, 0.5, 0, 0.5], [1, 1, 1, 1]], dtype=np.float32)
+    assert (row_ops.l1_normalize(x, 4.0) == want).all()
+    rng = np.random.default_rng(5)
+    y = rng.standard_normal((64, 32)).astype(np.float32) * 3
+    out = row_ops.l1_normalize(y, 10.0)
+    norms = np.abs(y).sum(axis=1)
+    assert (out >= 0).all()
+    assert np.allclose(out.sum(axis=1), np.minimum(norms, 10.0), rtol=1e-5)
+    assert np.allclose(out * norms[:, None], np.abs(y) * out.sum(axis=1)[:, None], rtol=1e-4)   # proportions kept
+    assert (row_ops.l1_normalize(np.zeros((2, 4), np.float32), 1.0) == 0).all()                 # no 0 / 0
+
+
+def test_regret_matching_of_a_subnormal_sum_is_a_distribution():
+    # the positive parts add up to a subnormal number: r / s is still an ordinary quotient
+    tiny = np.float32(2.0 ** -140)
+    x = np.array([[tiny, -1, 3 * tiny, 0]], dtype=np.float32)
+    p = row_ops.regret_matching(x)
+    assert np.isfinite(p).all() and (p == np.array([[.25, 0, .75, 0]], dtype=np.float32)).all()
+
+
+def test_reduce_all_by_hand():
+    x = np.array([[3, -7, 2, 5], [1, 4, -2, 6]], dtype=np.int32)
+    assert row_ops.reduce_all(x, "+") == 12 and row_ops.reduce_all(x, "max") == 6 and row_ops.reduce_all(x, "min") == -7
+    assert row_ops.reduce_all(x, "*") == 3 * -7 * 2 * 5 * 1 * 4 * -2 * 6
+    assert row_ops.reduce_all(np.arange(16384, dtype=np.uint64), "+") == 134209536      # the reference's test6
