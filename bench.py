@@ -233,12 +233,12 @@ def main():
                 # made when the weights are set, like a transpose at model load); every timed step is one
                 # sp_mlp_forward_packed launch that reads nothing but the packed buffer, x and u
                 pk = layers.pack_weights(wd)
-                call = (_lib.SP_F16, _lib.ptr(xd), 4, _lib.ptr(pk.buffer), None, dp, _lib.ptr(ud), _lib.ptr(policy),
-                        _lib.ptr(action), None, batch, _lib.HEAD_SOFTMAX_RM, 0)
+                call = (_lib.SP_F16, _lib.ptr(xd), 4, _lib.ptr(pk.buffer), pk.buffer.numel(), None, dp, _lib.ptr(ud), None,
+                        _lib.ptr(policy), _lib.ptr(action), None, batch, _lib.HEAD_SOFTMAX_RM, 0)
                 fn = lambda: _lib.check(_lib.lib.sp_mlp_forward_packed(*call, _lib.stream_ptr()))
             else:
-                call = (_lib.SP_F16, _lib.ptr(xd), 4, wp, None, dp, _lib.ptr(ud), _lib.ptr(policy), _lib.ptr(action), None,
-                        batch, _lib.HEAD_SOFTMAX_RM, 0)
+                call = (_lib.SP_F16, _lib.ptr(xd), 4, wp, None, dp, _lib.ptr(ud), None, _lib.ptr(policy), _lib.ptr(action),
+                        None, batch, _lib.HEAD_SOFTMAX_RM, 0)
                 fn = lambda: _lib.check(_lib.lib.sp_mlp_forward(*call, _lib.stream_ptr()))
             wall, ev = time_launches(fn, max(K, 200), W)
             want_p, want_a, _ = olayers.mlp_forward(x, ws, u=u)

@@ -76,6 +76,13 @@ typedef struct {
 } sp_kernel_info_t;
 int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
 
+/* Measurement aid: out[0] = the compute units' cycle counter, out[1] = the constant 100 MHz counter, both read by
+ * one wave at the point of `stream` where the call is enqueued.  Two samples around a stretch of work give the clock
+ * the units actually ran at during it: (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz -- on power-limited kernels
+ * well below the nominal 2.4 GHz that the published peak rates assume.  `out` is device memory (16 bytes).  Stands
+ * beside the host-side device probing of corecuda/base.spi:73; the reference has no counterpart. */
+int sp_clock_sample(uint64_t* out, void* stream);
+
 /* ------------------------------------------------------------------------------------------ */
 /* GEMM                                                                                        */
 /* ------------------------------------------------------------------------------------------ */

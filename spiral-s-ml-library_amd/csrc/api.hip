@@ -93,9 +93,29 @@ static std::vector<KernelEntry>& registry() {
 
 void register_kernel(const char* name, const void* fn, int threads) { registry().push_back({name, fn, threads}); }
 
+// One wave writes the shader clock counter (s_memtime: counts the cycles the compute units run at, so it slows
+// down with the clock) and the constant 100 MHz counter (s_memrealtime) side by side.  A single workgroup always
+// lands on the same XCD, so two samples read the same pair of counters.
+__global__ void clock_sample_kernel(unsigned long long* out) {
+    if (threadIdx.x == 0) {
+        const unsigned long long cycles = __builtin_amdgcn_s_memtime();
+        const unsigned long long ticks = __builtin_amdgcn_s_memrealtime();
+        out[0] = cycles;
+        out[1] = ticks;
+    }
+}
+
 }  // namespace sp
 
 using namespace sp;
+
+extern "C" int sp_clock_sample(uint64_t* out, void* stream) {
+    SP_REQUIRE_PTR(out);
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
+    return check_launch(__func__);
+}
 
 extern "C" const char* sp_last_error_string(void) { return error_buffer(); }
 

@@ -1035,6 +1035,19 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
     if (h256 && head != SP_HEAD_NONE && logits_out == nullptr && mask_size > 0 && mask_size <= 16 &&
         mask_size < dims[n_layers])
         a.nout = mask_size;
+    if (h256 && mlp_resident_takes(n_layers, dims, a.nout) &&
+        (batch + 63) / 64 >= (long)SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR * cus) {
+        // many tiles per compute unit: the kernel that loads the weights once and keeps them in registers
+        MlpResidentArgs r{};
+        r.x = x; r.u = u; r.policy = policy_out; r.action = action_out; r.logits = logits_out;
+        r.batch = batch; r.head = head; r.mask_size = mask_size; r.k0 = a.k0; r.nout = a.nout; r.out_stride = a.out_stride;
+        r.ph = a.ph;
+        for (int i = 0; i < n_layers; ++i) {
+            r.w[i] = a.w[i];
+            r.b[i] = a.b[i];
+        }
+        return mlp_resident_launch(dtype, false, n_layers, r, (hipStream_t)stream, __func__);
+    }
     const void* kernel;
     int lds_bytes = MLP_STAGES * MLP_STAGE_BYTES + 1024;   // weight ring + the dummy DMA target
     int rows_per_block = nw * 16;

@@ -40,6 +40,34 @@ struct MlpArgs {
     PhiloxStream ph;     // philox_mode >= 0: the head draws its uniform itself (ml/layers.spi:339-344) and `u` is not read
 };
 
+// Arguments of the kernel that keeps a stack's weights in registers and walks over many 64-row tiles per compute
+// unit (mlp_resident.hip); both sp_mlp_forward and sp_mlp_forward_packed hand large batches to it.
+struct MlpResidentArgs {
+    const void* x;
+    const void* packed;                  // packed weights (PACKED instantiations)
+    const void* w[4];                    // row-major weights (the others)
+    const float* b[4];
+    const float* u;
+    float* policy;
+    int* action;
+    float* logits;
+    long batch;
+    int tiles;
+    int head, mask_size, k0, nout, out_stride;
+    PhiloxStream ph;
+};
+
+bool mlp_resident_takes(int n_layers, const int32_t* dims, int nout);
+int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a, hipStream_t stream, const char* what);
+// Tiles per compute unit from which the resident kernel is used (its one-time load of all weights has to pay):
+// packed weights stream in at the texture path's full rate, row-major ones at about a quarter of it.
+#ifndef SP_MLP_RESIDENT_MIN_TILES_PACKED
+#define SP_MLP_RESIDENT_MIN_TILES_PACKED 2
+#endif
+#ifndef SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR
+#define SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR 4
+#endif
+
 // The Philox stream of a head that draws its own uniforms: the sampling node of the layer graph works on rows of
 // `cols` = the last layer's full width, which the reference's row primitives need to be a multiple of 4.
 inline int mlp_set_philox(PhiloxStream& ph, const sp_philox_t* philox, int64_t batch, int cols, const char* fn) {

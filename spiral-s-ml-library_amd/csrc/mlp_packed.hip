@@ -619,6 +619,16 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
     if (rc != SP_OK) return rc;
     a.x = x; a.packed = packed; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.out_stride = dims[n_layers];
+    if (mlp_resident_takes(n_layers, dims, a.nout) &&
+        (batch + PK_ROWS - 1) / PK_ROWS >= (long)SP_MLP_RESIDENT_MIN_TILES_PACKED * device_cu_count()) {
+        // several tiles per compute unit: the kernel that loads the weights once and keeps them in registers
+        MlpResidentArgs r{};
+        r.x = x; r.packed = packed; r.u = u; r.policy = policy_out; r.action = action_out; r.logits = logits_out;
+        r.batch = batch; r.head = head; r.mask_size = mask_size; r.k0 = a.k0; r.nout = a.nout; r.out_stride = a.out_stride;
+        r.ph = a.ph;
+        for (int i = 0; i < n_layers; ++i) r.b[i] = a.b[i];
+        return mlp_resident_launch(dtype, true, n_layers, r, (hipStream_t)stream, __func__);
+    }
     const int ks0 = pk_ks0(dims[0]);
     const bool plain = a.nout <= 4 && a.out_stride == a.nout && logits_out == nullptr && action_out != nullptr && a.b[n_layers - 1] == nullptr;
     const void* kernel = dtype == SP_F16 ? pick_packed_kernel<SP_F16>(ks0, n_layers, plain) : pick_packed_kernel<SP_BF16>(ks0, n_layers, plain);

@@ -54,6 +54,7 @@ SIGNATURES = {
     "sp_last_error_string": (C.c_char_p, []),
     "sp_device_info": (C.c_int, [C.POINTER(DeviceInfo)]),
     "sp_kernel_info": (C.c_int, [C.c_char_p, C.POINTER(KernelInfo)]),
+    "sp_clock_sample": (C.c_int, [_P, _P]),
     "sp_gemm_abt": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, _P, _I64, _I64, _I64, _F, _F, _U32, _P]),
     "sp_gemm_abt_batched": (C.c_int, [C.c_int, C.c_int, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, _I64, _I64, _F, _F,
                                       _U32, _P]),

@@ -282,7 +282,7 @@ def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed,
     pk = LY.pack_weights(wd) if packed else None
     cols = dims[-1]
     if mode == "layer":
-        q = 24
+        q = 24 if batch % 24 == 0 else 32
         cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=q, rows_per_block=batch // q, offset=8)
         want_u = ophilox.row_uniforms_layer(q, batch // q, cols, offset=8)
     elif mode == "block":
@@ -299,3 +299,61 @@ def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed,
     for a, b in zip(with_u, with_rng):
         assert torch.equal(a, b)
     assert (host(with_rng[1]) == orow.discrete_sampling(host(with_rng[0]), host(u))).all()
+
+
+@pytest.mark.parametrize("dims,head,mask,batch,dtype,with_bias,packed", [
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 70000, "f16", False, True),    # the benchmark's network, ragged last tile
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 70000, "f16", False, False),   # ... from the row-major weights
+    ([32, 256, 256, 256, 3], "softmax", 0, 300000, "bf16", "all", True),                  # 18 tiles per compute unit
+    ([16, 256, 256, 4], "softmax_regret_matching", 0, 66000, "f16", True, False),         # three layers, a 16-wide first layer
+    ([48, 256, 256, 256, 16], "softmax", 0, 66000, "bf16", True, False),                  # two first-layer k-steps, K0 not a multiple of 32, 16 outputs
+    ([64, 256, 256, 12], "softmax", 7, 40000, "f16", "only1", True),                      # masked head with logits, head staged in LDS
+    ([32, 256, 256, 256, 2], "softmax_regret_matching", 0, 32768 + 5, "bf16", False, True),
+])
+def test_weights_resident_in_registers(LY, dims, head, mask, batch, dtype, with_bias, packed):
+    """Batches of several 64-row tiles per compute unit run on the kernel that loads the weights once and keeps them in
+    registers while it walks over its tiles (from two tiles per unit with packed weights, from four with row-major
+    ones): against the oracle like every other kernel, and bit for bit against the per-tile packed kernel run on the
+    same rows in slices small enough to stay on that kernel (same operand layout, same order of the sums)."""
+    announce("mlp resident %s head=%s mask=%d batch=%d %s bias=%s packed=%s" % (dims, head, mask, batch, dtype, with_bias, packed))
+    rng = np.random.default_rng(sum(dims) + batch + 7)
+    x, ws, u = make_problem(rng, batch, dims, dtype)
+    biases = None
+    if with_bias:
+        biases = [rng.standard_normal(d, dtype=np.float32) * np.float32(0.1) for d in dims[1:]]
+        if with_bias == "only1":
+            biases = [b if l == 1 else None for l, b in enumerate(biases)]
+        elif with_bias != "all":
+            biases[1] = None
+    policy, action = check(LY, x, ws, u, dtype, head, mask, biases, packed=packed)
+    t = TORCH[dtype]
+    wd = [dev(w, t) for w in ws]
+    bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
+    pk = LY.pack_weights(wd)
+    step = 16384
+    for lo in range(0, batch, step):
+        hi = min(batch, lo + step)
+        p, a = LY.mlp_forward(dev(x[lo:hi], t), None, bd, head, dev(u[lo:hi]), mask, packed=pk)
+        assert (host(p) == policy[lo:hi]).all() and (host(a) == action[lo:hi]).all(), lo
+
+
+def test_resident_kernel_run_to_run_and_philox(LY):
+    """The resident kernel gives the same bits on every launch, and with a Philox stream in place of the uniforms tensor
+    it draws for every tile of its walk what sp_philox_uniforms hands out for those rows."""
+    from ml import _lib, primitives
+    announce("mlp resident run-to-run + philox")
+    rng = np.random.default_rng(41)
+    batch, dims = 24 * 4096, [32, 256, 256, 256, 64]
+    x, ws, _ = make_problem(rng, batch, dims, "f16")
+    xd, wd = dev(x, torch.float16), [dev(w, torch.float16) for w in ws]
+    pk = LY.pack_weights(wd)
+    cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=24, rows_per_block=4096)
+    u = primitives.philox_uniforms(cfg, batch, 64)
+    for packed in (pk, None):
+        first = [t.clone() for t in LY.mlp_forward(xd, wd, None, "softmax", u, 3, packed=packed)]
+        for _ in range(2):
+            again = LY.mlp_forward(xd, wd, None, "softmax", u, 3, packed=packed)
+            assert all(torch.equal(a, b) for a, b in zip(first, again))
+        drawn = LY.mlp_forward(xd, wd, None, "softmax", None, 3, packed=packed, rng=cfg)
+        assert all(torch.equal(a, b) for a, b in zip(first, drawn))
+        assert (host(first[1]) == orow.discrete_sampling(host(first[0]), host(u))).all()
