@@ -4,11 +4,15 @@
 // weights into every compute unit: 274 KiB per unit for 32 -> 256 -> 256 -> 256 -> 3 at the texture path's 64 bytes
 // per cycle is as long as the 4.5 k cycles of MFMA work of a 64-row tile, and a workgroup that starts cold pays
 // the latency of its first loads on top.  When a unit has more than one tile to do, none of that needs repeating:
-// a workgroup of four waves, one per SIMD with 512 registers each, holds ALL the weights of a stack with up to two
-// 256 x 256 layers -- wave w keeps output features 64 w .. 64 w + 63 of every feature-split layer (16 or 32 + 128 +
-// 128 registers) and the at most 16 rows of the output layer (32 registers), in MFMA operand order -- and walks over
-// the tiles blockIdx.x, blockIdx.x + gridDim.x, ...  A tile then costs its MFMAs, the exchange of activations
-// through LDS (one barrier per layer), the head, and 4 KiB of input.
+// a workgroup of EIGHT waves, two per SIMD with 256 registers each, holds all the 256 x 256 weights of a stack with
+// up to two such layers -- wave v keeps output features 32 v .. 32 v + 31 of each (64 + 64 registers, in MFMA operand
+// order); the few KiB of the first and the last layer sit in LDS -- and walks over the tiles blockIdx.x,
+// blockIdx.x + gridDim.x, ...  A tile then costs its MFMAs, the exchange of activations through LDS (one barrier
+// per layer), the head, and 4 KiB of input.
+// Two waves per SIMD, not one with twice the features: a wave cannot issue anything else in the shadow of its own
+// MFMAs (every LDS read, conversion or wait of a lone wave costs the matrix pipe 4-5 cycles; measured on the
+// four-wave form of this kernel: 3.0-3.2 k cycles per 256 x 256 layer for 2 k cycles of MFMA), its neighbour on the
+// SIMD can.
 //
 // The weights come either packed (sp_mlp_pack_weights: one contiguous KiB per wave-wide load) or straight from the
 // row-major matrices of sp_mlp_forward: in operand order a lane then touches half a cache line of a row of its
@@ -25,17 +29,19 @@
 namespace sp {
 
 constexpr int RS_ROWS = 64;                              // batch rows per tile
+constexpr int RS_WAVES = 8;
+constexpr int RS_THREADS = RS_WAVES * 64;
 constexpr int RS_ACT_BYTES = RS_ROWS * 512;              // one activation buffer: 64 rows x 256 features x 2 bytes
-constexpr int RS_X_OFF = 2 * RS_ACT_BYTES;               // two input buffers, 64 rows x 128 bytes (a tile's inputs are
-constexpr int RS_X_BYTES = RS_ROWS * 128;                //   written while the tile before it is still computed)
+constexpr int RS_X_OFF = 3 * RS_ACT_BYTES;               // three of those, then two input buffers, 64 rows x 128 bytes
+constexpr int RS_X_BYTES = RS_ROWS * 128;                //   (a tile's inputs are written while the tile before it is computed)
 constexpr int RS_BIAS_OFF = RS_X_OFF + 2 * RS_X_BYTES;   // the biases of the feature-split layers, 256 f32 each
-constexpr int RS_HEAD_OFF = RS_BIAS_OFF + 3 * 1024;      // a KiB per wave: the outputs of a head wider than 4
+constexpr int RS_HEAD_OFF = RS_BIAS_OFF + 3 * 1024;      // a KiB per 16 rows: the outputs of a head wider than 4
 constexpr int RS_WL_OFF = RS_HEAD_OFF + 4 * 1024;        // the output layer's weights: 8 k-steps x 1 KiB
-constexpr int RS_W0_OFF = RS_WL_OFF + 8 * 1024;          // the first layer's: per wave KS0 k-steps x 4 tiles x 1 KiB
-constexpr int RS_LDS_TOTAL = RS_W0_OFF + 4 * 2 * 4096;
+constexpr int RS_W0_OFF = RS_WL_OFF + 8 * 1024;          // the first layer's: per wave KS0 k-steps x 2 tiles x 1 KiB
+constexpr int rs_lds_total(int ks0) { return RS_W0_OFF + RS_WAVES * ks0 * 2048; }
 
 #ifdef SP_RS_TIMELINE
-__device__ unsigned long long sp_rs_timeline[256 * 4 * 16 * 8];
+__device__ unsigned long long sp_rs_timeline[256 * 8 * 16 * 8];
 #endif
 
 template <int FROM, int TO, typename F>
@@ -49,14 +55,15 @@ __device__ __forceinline__ void rs_static_for(F&& f) {
 // KS0: 32-wide k-steps of the first layer (1 or 2); NL: layers (3 or 4); PLAIN: at most 4 dense policy columns and an
 // action, no logits, no bias on the output layer; PACKED: the weights are in the layout of sp_mlp_pack_weights.
 template <int DT, int KS0, int NL, bool PLAIN, bool PACKED>
-__global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs a) {
+__global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResidentArgs a) {
     constexpr int S = NL - 1;                                // feature-split layers 0 .. S - 1
-    static_assert(S == 2 || S == 3, "one or two 256 x 256 layers fit the registers next to the first and the last layer");
+    static_assert(S == 2 || S == 3, "one or two 256 x 256 layers fit the registers");
     static_assert(KS0 == 1 || KS0 == 2, "a first layer of at most 64 inputs");
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);      // 0..7: features 32 wave .. 32 wave + 31
+    const int w4 = wave >> 1, wp = wave & 1;                        // ... = tile pair wp of the 64-feature slice w4
     const int j = lane & 15, q = lane >> 4;
     const u32x4 zero_u4 = {0u, 0u, 0u, 0u};
     const int K0 = a.k0, NOUT = a.nout;
@@ -76,22 +83,23 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
         const float* b = a.b[l];
         if (b != nullptr) {
             has_bias |= 1u << l;
-            *reinterpret_cast<float*>(lds + RS_BIAS_OFF + l * 1024 + tid * 4) = b[tid];
+            if (tid < 256) *reinterpret_cast<float*>(lds + RS_BIAS_OFF + l * 1024 + tid * 4) = b[tid];
         }
     }
 
     // ---- the weights, once.  The 256 x 256 layers go into the accumulation registers and stay there (block (k-step,
     //      feature tile) = 4 registers: lane (i, q) holds the 8 K-values 32 ks + 8 q .. of feature row i of the
-    //      tile); the first layer's few blocks (this wave's) and the output layer's eight (everybody's) go to LDS in
-    //      the same order, from where a tile reads them back with one ds_read_b128 each ----
-    // (The second 256 x 256 layer keeps its last k-step in ordinary registers: with all 256 accumulation registers
-    //  spoken for the register allocator parks one block elsewhere and copies it in front of every use.)
-    u32x4 W1[8][4], W2[S == 3 ? 7 : 1][4], W2v[4];
+    //      tile; this wave's tiles are 2 wp and 2 wp + 1 of the four that make up slice w4); the first layer's few
+    //      blocks (this wave's) and the output layer's eight (everybody's) go to LDS in the same order, from where a
+    //      tile reads them back with one ds_read_b128 each ----
+    // (The second 256 x 256 layer keeps its last k-step in ordinary registers: a file that is spoken for to the last
+    //  register makes the allocator park a block elsewhere and copy it in front of every use.)
+    u32x4 W1[8][2], W2[S == 3 ? 7 : 1][2], W2v[2];
     {
         const int i16 = lane & 15;
-        // feature row of lane i in tile t of this wave: 64 w + 32 (t / 2) + 8 (i / 4) + 4 (t % 2) + i % 4
+        // feature row of lane i in tile t of slice w4: 64 w4 + 32 (t / 2) + 8 (i / 4) + 4 (t % 2) + i % 4
         const unsigned lane_row = (unsigned)(8 * (i16 >> 2) + (i16 & 3));
-        unsigned char* const w0_lds = lds + RS_W0_OFF + wave * (KS0 * 4096) + lane * 16;
+        unsigned char* const w0_lds = lds + RS_W0_OFF + wave * (KS0 * 2048) + lane * 16;
         unsigned char* const wl_lds = lds + RS_WL_OFF + lane * 16;
         if constexpr (PACKED) {
             const unsigned char* const packed = (const unsigned char*)a.packed;
@@ -100,65 +108,66 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W1[ks][t]) : "v"(voff), "s"(packed + first_bytes + ((long)(wave * 8 + ks) * 4 + t) * 1024) : "memory");
+                for (int h = 0; h < 2; ++h)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W1[ks][h]) : "v"(voff), "s"(packed + first_bytes + ((long)(w4 * 8 + ks) * 4 + 2 * wp + h) * 1024) : "memory");
             if constexpr (S == 3) {
 #pragma unroll
                 for (int ks = 0; ks < 7; ++ks)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W2[ks][t]) : "v"(voff), "s"(packed + first_bytes + 131072 + ((long)(wave * 8 + ks) * 4 + t) * 1024) : "memory");
+                    for (int h = 0; h < 2; ++h)
+                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W2[ks][h]) : "v"(voff), "s"(packed + first_bytes + 131072 + ((long)(w4 * 8 + ks) * 4 + 2 * wp + h) * 1024) : "memory");
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[t]) : "v"(voff), "s"(packed + first_bytes + 131072 + ((long)(wave * 8 + 7) * 4 + t) * 1024) : "memory");
+                for (int h = 0; h < 2; ++h)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[h]) : "v"(voff), "s"(packed + first_bytes + 131072 + ((long)(w4 * 8 + 7) * 4 + 2 * wp + h) * 1024) : "memory");
             }
 #pragma unroll
-            for (int b = 0; b < 4 * KS0; ++b)
-                *reinterpret_cast<u32x4*>(w0_lds + b * 1024) = *reinterpret_cast<const u32x4*>(packed + ((long)wave * KS0 * 4 + b) * 1024 + voff);
+            for (int ks = 0; ks < KS0; ++ks)
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
-                *reinterpret_cast<u32x4*>(wl_lds + (2 * wave + h) * 1024) =
-                    *reinterpret_cast<const u32x4*>(packed + first_bytes + (long)(S - 1) * 131072 + (2 * wave + h) * 1024 + voff);
+                for (int h = 0; h < 2; ++h)
+                    *reinterpret_cast<u32x4*>(w0_lds + (ks * 2 + h) * 1024) =
+                        *reinterpret_cast<const u32x4*>(packed + ((long)(w4 * KS0 + ks) * 4 + 2 * wp + h) * 1024 + voff);
+            *reinterpret_cast<u32x4*>(wl_lds + wave * 1024) =
+                *reinterpret_cast<const u32x4*>(packed + first_bytes + (long)(S - 1) * 131072 + wave * 1024 + voff);
         } else {
-            // row-major: base of (tile t) = row 64 w + 32 (t / 2) + 4 (t % 2), k-step ks = 64 bytes further per step;
-            // the lane adds its row inside the tile and its quarter of the k-step
+            // row-major: base of tile t = row 64 w4 + 32 (t / 2) + 4 (t % 2), i.e. 64 w4 + 32 wp + 4 h for this wave's
+            // tile h; k-step ks = 64 bytes further per step; the lane adds its row inside the tile and its quarter
             const unsigned char* const w0 = (const unsigned char*)a.w[0];
             const unsigned char* const w1 = (const unsigned char*)a.w[1];
             const unsigned char* const w2 = (const unsigned char*)a.w[S == 3 ? 2 : 1];
             const unsigned char* const wl = (const unsigned char*)a.w[S];
             const unsigned vo_h = (unsigned)((lane_row * 256 + 8 * q) * 2);
+            const long tile_row = 64 * w4 + 32 * wp;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W1[ks][t]) : "v"(vo_h), "s"(w1 + (long)(64 * wave + 32 * (t >> 1) + 4 * (t & 1)) * 512 + ks * 64) : "memory");
+                for (int h = 0; h < 2; ++h)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W1[ks][h]) : "v"(vo_h), "s"(w1 + (tile_row + 4 * h) * 512 + ks * 64) : "memory");
             if constexpr (S == 3) {
 #pragma unroll
                 for (int ks = 0; ks < 7; ++ks)
 #pragma unroll
-                    for (int t = 0; t < 4; ++t)
-                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W2[ks][t]) : "v"(vo_h), "s"(w2 + (long)(64 * wave + 32 * (t >> 1) + 4 * (t & 1)) * 512 + ks * 64) : "memory");
+                    for (int h = 0; h < 2; ++h)
+                        asm volatile("global_load_dwordx4 %0, %1, %2" : "=a"(W2[ks][h]) : "v"(vo_h), "s"(w2 + (tile_row + 4 * h) * 512 + ks * 64) : "memory");
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[t]) : "v"(vo_h), "s"(w2 + (long)(64 * wave + 32 * (t >> 1) + 4 * (t & 1)) * 512 + 7 * 64) : "memory");
+                for (int h = 0; h < 2; ++h)
+                    asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[h]) : "v"(vo_h), "s"(w2 + (tile_row + 4 * h) * 512 + 7 * 64) : "memory");
             }
             // layer 0: rows of K0 values; k-values past K0 are zeros
 #pragma unroll
             for (int ks = 0; ks < KS0; ++ks) {
                 const bool ok = 32 * ks + 8 * q < K0;
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
+                for (int h = 0; h < 2; ++h) {
                     u32x4 v = zero_u4;
-                    if (ok) v = *reinterpret_cast<const u32x4*>(w0 + ((long)(64 * wave + 32 * (t >> 1) + 4 * (t & 1) + lane_row) * K0 + 32 * ks + 8 * q) * 2);
-                    *reinterpret_cast<u32x4*>(w0_lds + (ks * 4 + t) * 1024) = v;
+                    if (ok) v = *reinterpret_cast<const u32x4*>(w0 + ((tile_row + 4 * h + lane_row) * K0 + 32 * ks + 8 * q) * 2);
+                    *reinterpret_cast<u32x4*>(w0_lds + (ks * 2 + h) * 1024) = v;
                 }
             }
             // output layer: MFMA row i is output i; rows past the computed outputs are zeros
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            {
                 u32x4 v = zero_u4;
-                if (i16 < NOUT) v = *reinterpret_cast<const u32x4*>(wl + ((long)i16 * 256 + 32 * (2 * wave + h) + 8 * q) * 2);
-                *reinterpret_cast<u32x4*>(wl_lds + (2 * wave + h) * 1024) = v;
+                if (i16 < NOUT) v = *reinterpret_cast<const u32x4*>(wl + ((long)i16 * 256 + 32 * wave + 8 * q) * 2);
+                *reinterpret_cast<u32x4*>(wl_lds + wave * 1024) = v;
             }
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -172,37 +181,28 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
     auto read_at = [&](int base, int bt, int ks) {
         return *reinterpret_cast<const u32x4*>(lds + base + aoff[ks & 3] + bt * 8192 + (ks >> 2) * 256);
     };
-    // outputs: tiles (p, 0) and (p, 1) give lane (j, q) the features 64 w + 32 p + 8 q .. + 7 of batch row j
-    unsigned pw[2];
-#pragma unroll
-    for (int p = 0; p < 2; ++p) pw[p] = (unsigned)(j * 512 + (wave >> 1) * 256 + (((8 * (wave & 1) + 4 * p + q) ^ j) << 4));
+    // outputs: this wave's two tiles give lane (j, q) the features 64 w4 + 32 wp + 8 q .. + 7 of batch row j
+    const unsigned pw = (unsigned)(j * 512 + (w4 >> 1) * 256 + (((8 * (w4 & 1) + 4 * wp + q) ^ j) << 4));
 
-    // the 16-byte pieces of a tile's input rows this thread moves: piece idx = tid + 256 i, 4 KS0 pieces per row
-    auto load_x = [&](int tile, u32x4 (&xin)[KS0]) {
-        const long row0 = (long)tile * RS_ROWS;
-#pragma unroll
-        for (int i = 0; i < KS0; ++i) {
-            const int idx = tid + 256 * i;
-            const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
-            const bool ok = row0 + r < batch && pc * 8 < K0;
-            xin[i] = zero_u4;
-            if (ok) xin[i] = *reinterpret_cast<const u32x4*>(x_ptr + ((row0 + r) * K0 + pc * 8) * 2);
-        }
+    // the 16-byte piece of a tile's input rows this thread moves (4 KS0 pieces per row: 256 KS0 pieces in all)
+    const int x_r = tid / (4 * KS0), x_pc = tid % (4 * KS0);
+    const bool x_mine = tid < 256 * KS0;
+    // (the load itself is unconditional -- a piece outside the batch or past K0 reads the tensor's first bytes and is
+    //  replaced by zeros when it is stored: a load under a condition would be waited for where the branches meet)
+    auto x_valid = [&](int tile) { return x_mine && (long)tile * RS_ROWS + x_r < batch && x_pc * 8 < K0; };
+    auto load_x = [&](int tile) {
+        const long off = x_valid(tile) ? (((long)tile * RS_ROWS + x_r) * K0 + x_pc * 8) * 2 : 0;
+        return *reinterpret_cast<const u32x4*>(x_ptr + off);
     };
     // inputs: row r, piece pc (of at most 8) lives in slot (pc ^ r) & 7 of the row's 128 bytes
-    auto store_x = [&](int buf, const u32x4 (&xin)[KS0]) {
-#pragma unroll
-        for (int i = 0; i < KS0; ++i) {
-            const int idx = tid + 256 * i;
-            const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
-            *reinterpret_cast<u32x4*>(lds + RS_X_OFF + buf * RS_X_BYTES + r * 128 + (((pc ^ r) & 7) << 4)) = xin[i];
-        }
+    auto store_x = [&](int buf, const u32x4& v, bool valid) {
+        if (x_mine) *reinterpret_cast<u32x4*>(lds + RS_X_OFF + buf * RS_X_BYTES + x_r * 128 + (((x_pc ^ x_r) & 7) << 4)) = valid ? v : zero_u4;
     };
     unsigned xoff[KS0];
 #pragma unroll
     for (int ks = 0; ks < KS0; ++ks) xoff[ks] = (unsigned)(RS_X_OFF + j * 128 + ((((4 * ks + q) ^ j) & 7) << 4));
 
-    f32x4 acc[4][4];                                         // [batch tile][feature tile]
+    f32x4 acc[4][2];                                         // [batch tile][feature tile of this wave]
     // The MFMAs are asm: their weight operand lives in registers the asm loads above filled, which the compiler must
     // neither move nor copy.  It therefore cannot see the wait states an MFMA needs after a vector-ALU write of a
     // register it reads; WAIT puts two in front (used where the compiler's own vector-ALU work is interleaved; the
@@ -235,28 +235,27 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
     // rounding) to `out_base`.  K-steps in order, the activation fragments of the next k-step read one at a time behind
     // the first MFMAs.  The LAST two k-steps (the last one, of a layer that has only one) are walked batch tile by
     // batch tile instead: tile bt's sums are then complete while tiles bt + 1 .. 3 are still being multiplied, and
-    // its outputs are converted and written one packed word per MFMA, in the matrix pipe's shadow; only the last
-    // tile's conversion stands alone.  `before_barrier` runs in front of the barrier that makes the outputs
-    // everyone's inputs.
+    // its outputs are converted and written one packed word per MFMA; only the last tile's conversion stands alone.
+    // `before_barrier` runs in front of the barrier that makes the outputs everyone's inputs.
     auto layer = [&](auto L_, int in_base, int out_base, auto&& before_barrier) {
         constexpr int L = decltype(L_)::value;
         constexpr int KS = L == 0 ? KS0 : 8;
         constexpr int TAILK = KS >= 2 ? 2 : 1;                // k-steps walked batch tile by batch tile
         constexpr int HEADK = KS - TAILK;
         const bool with_bias = (has_bias & (1u << L)) != 0;   // uniform
-        u32x4 W0[L == 0 ? KS0 : 1][4];                        // the first layer's weights come back from LDS
+        u32x4 W0[L == 0 ? KS0 : 1][2];                        // the first layer's weights come back from LDS
         if constexpr (L == 0) {
 #pragma unroll
             for (int ks = 0; ks < KS0; ++ks)
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    W0[ks][t] = *reinterpret_cast<const u32x4*>(lds + RS_W0_OFF + wave * (KS0 * 4096) + (ks * 4 + t) * 1024 + lane * 16);
+                for (int h = 0; h < 2; ++h)
+                    W0[ks][h] = *reinterpret_cast<const u32x4*>(lds + RS_W0_OFF + wave * (KS0 * 2048) + (ks * 2 + h) * 1024 + lane * 16);
         }
-        auto mm = [&](f32x4& c, int ks, int t, const u32x4& x, bool first, auto WAIT_) {
-            if constexpr (L == 0) mfma_v(c, W0[ks][t], x, first, WAIT_);
-            else if constexpr (L == 1) mfma_a(c, W1[ks][t], x, first, WAIT_);
-            else if (ks < 7) mfma_a(c, W2[ks < 7 ? ks : 0][t], x, first, WAIT_);
-            else mfma_v(c, W2v[t], x, first, WAIT_);
+        auto mm = [&](f32x4& c, int ks, int h, const u32x4& x, bool first, auto WAIT_) {
+            if constexpr (L == 0) mfma_v(c, W0[ks][h], x, first, WAIT_);
+            else if constexpr (L == 1) mfma_a(c, W1[ks][h], x, first, WAIT_);
+            else if (ks < 7) mfma_a(c, W2[ks < 7 ? ks : 0][h], x, first, WAIT_);
+            else mfma_v(c, W2v[h], x, first, WAIT_);
         };
         // activation fragment (batch tile bt, k-step ks) of this layer's input
         auto read_in = [&](int bt, int ks) {
@@ -268,12 +267,16 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
         for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_in(bt, 0);
         rs_static_for<0, HEADK>([&](auto KS_) {
             constexpr int ks = decltype(KS_)::value;
-            rs_static_for<0, 4>([&](auto T_) {
-                constexpr int t = decltype(T_)::value;
+            rs_static_for<0, 2>([&](auto H_) {
+                constexpr int h = decltype(H_)::value;
 #pragma unroll
                 for (int bt = 0; bt < 4; ++bt) {
-                    mm(acc[bt][t], ks, t, bf[ks & 1][bt], ks == 0, IC<0>{});
-                    if (t == 0) bf[(ks + 1) & 1][bt] = read_in(bt, ks + 1);
+                    mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<0>{});
+#ifndef SP_RS_ABL_NOREAD
+                    if (h == 0) bf[(ks + 1) & 1][bt] = read_in(bt, ks + 1);
+#else
+                    if (h == 0) bf[(ks + 1) & 1][bt] = bf[ks & 1][bt];
+#endif
                     __builtin_amdgcn_sched_barrier(0);
                 }
             });
@@ -292,34 +295,40 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
         // (two copies, with and without a bias: the test is uniform and made once per layer)
         auto end_of_layer = [&](auto HAS_BIAS_) {
             constexpr bool has_b = decltype(HAS_BIAS_)::value != 0;
-            f32x4 bias_r[4];                                  // [2 p + h]: features 64 w + 32 p + 8 q + 4 h .. + 3
+            f32x4 bias_r[2];                                  // [h]: features 64 w4 + 32 wp + 8 q + 4 h .. + 3
             if constexpr (has_b) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    bias_r[i] = *reinterpret_cast<const f32x4*>(lds + RS_BIAS_OFF + L * 1024 + (64 * wave + 32 * (i >> 1) + 8 * q + 4 * (i & 1)) * 4);
+                for (int h = 0; h < 2; ++h)
+                    bias_r[h] = *reinterpret_cast<const f32x4*>(lds + RS_BIAS_OFF + L * 1024 + (64 * w4 + 32 * wp + 8 * q + 4 * h) * 4);
             }
-            // word E (0..7) of batch tile BT's outputs: group p = E / 4 is the tile pair (2 p, 2 p + 1), one 16-byte write
+            // word E (0..3) of batch tile BT's outputs: tile E / 2, accumulator rows 2 (E % 2) and + 1; one 16-byte write
             u32x4 cv;
             auto convert_word = [&](auto BT_, auto E_) {
                 constexpr int bt = decltype(BT_)::value, e = decltype(E_)::value;
-                constexpr int p = e >> 2, tile = 2 * p + ((e >> 1) & 1), r = 2 * (e & 1);
-                float a0 = acc[bt][tile][r], a1 = acc[bt][tile][r + 1];
+                constexpr int h = e >> 1, r = 2 * (e & 1);
+                float a0 = acc[bt][h][r], a1 = acc[bt][h][r + 1];
                 if constexpr (has_b) {
-                    a0 += bias_r[tile][r];
-                    a1 += bias_r[tile][r + 1];
+                    a0 += bias_r[h][r];
+                    a1 += bias_r[h][r + 1];
                 }
-                cv[e & 3] = pack_relu2<DT>(a0, a1);
-                if constexpr ((e & 3) == 3) *reinterpret_cast<u32x4*>(lds + out_base + pw[p] + bt * 8192) = cv;
+#ifndef SP_RS_ABL_NOCONV
+                cv[e] = pack_relu2<DT>(a0, a1);
+#else
+                cv[e] = __builtin_bit_cast(unsigned, a0);
+#endif
+                if constexpr (e == 3) *reinterpret_cast<u32x4*>(lds + out_base + pw + bt * 8192) = cv;
             };
             rs_static_for<0, 4>([&](auto BT_) {
                 constexpr int bt = decltype(BT_)::value;
-                rs_static_for<0, 4 * TAILK>([&](auto M_) {
+                rs_static_for<0, 2 * TAILK>([&](auto M_) {
                     constexpr int m = decltype(M_)::value;
-                    constexpr int ks = HEADK + m / 4, t = m % 4;
-                    mm(acc[bt][t], ks, t, bf[ks & 1][bt], ks == 0, IC<1>{});
+                    constexpr int ks = HEADK + m / 2, h = m % 2;
+                    // (wait states in front of the MFMA where the bias additions' register traffic surrounds it; the
+                    //  copy without a bias has none of it, and the build's scan of the generated code holds it to that)
+                    mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<has_b ? 1 : 0>{});
                     __builtin_amdgcn_sched_barrier(0);
-                    if constexpr (bt > 0) {                   // the tile before this one is complete: 8 words over these MFMAs
-                        constexpr int per = 8 / (4 * TAILK);
+                    if constexpr (bt > 0) {                   // the tile before this one is complete: 4 words over these MFMAs
+                        constexpr int per = 4 / (2 * TAILK);
                         rs_static_for<0, per>([&](auto I_) { convert_word(IC<bt - 1>{}, IC<per * m + decltype(I_)::value>{}); });
                         __builtin_amdgcn_sched_barrier(0);
                     }
@@ -328,7 +337,7 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
             // the last tile: the s_nops are the wait states between the last MFMA and the first read of its result,
             // which the compiler does not know about
             asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
-            rs_static_for<0, 8>([&](auto E_) { convert_word(IC<3>{}, E_); });
+            rs_static_for<0, 4>([&](auto E_) { convert_word(IC<3>{}, E_); });
         };
         if (with_bias) end_of_layer(IC<1>{});
         else end_of_layer(IC<0>{});
@@ -339,69 +348,62 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
     // ---- the first tile's inputs ----
     int tile = blockIdx.x;
     int xbuf = 0;
-    {
-        u32x4 xin[KS0];
-        load_x(tile, xin);
-        store_x(0, xin);
-    }
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");          // inputs and biases are in LDS
+    store_x(0, load_x(tile), x_valid(tile));
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");          // inputs, biases and the small layers are in LDS
 
 #ifdef SP_RS_TIMELINE
     // measurement build: per wave and tile walked, the cycle counter at every phase boundary (8 words per tile)
     int tl_n = 0;
-#define SP_RS_STAMP(K) do { if (lane == 0 && tl_n < 16) sp_rs_timeline[(((long)blockIdx.x * 4 + wave) * 16 + tl_n) * 8 + (K)] = (K) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); } while (0)
+#define SP_RS_STAMP(K) do { if (lane == 0 && tl_n < 16) sp_rs_timeline[(((long)blockIdx.x * 8 + wave) * 16 + tl_n) * 8 + (K)] = (K) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); } while (0)
 #else
 #define SP_RS_STAMP(K) do {} while (0)
 #endif
+    // The activation buffers rotate A -> B -> C -> A: the output layer of tile n reads a buffer that tile n + 1 does not
+    // write before its second barrier, so a wave that is done with its head goes on without waiting for the others.
+    constexpr int BUF_A = 0, BUF_B = RS_ACT_BYTES, BUF_C = 2 * RS_ACT_BYTES;
     for (;;) {
         SP_RS_STAMP(0);
         const int next = tile + (int)gridDim.x;
         const bool has_next = next < tiles;
         const long row0 = (long)tile * RS_ROWS;
-        const long head_row_idx = row0 + wave * 16 + j;      // the row lanes 0..15 finish
-        const bool head_ok = lane < 16 && head_row_idx < batch;
+        // the head of 16 rows is shared by the two waves that hold slice w4: rows 16 w4 + 8 wp .. + 7 each
+        const long head_row_idx = row0 + w4 * 16 + j;        // the row lanes 0..15 could finish
+        const bool head_ok = lane < 16 && (j >> 3) == wp && head_row_idx < batch;
         float u_row = 1.f;
         if (ph_mode >= 0) u_row = reference_row_uniform(a.ph, head_ok ? head_row_idx : 0);
-        else if (u_ptr != nullptr && head_ok) u_row = u_ptr[head_row_idx];
+        else if (u_ptr != nullptr) u_row = u_ptr[head_ok ? head_row_idx : 0];      // (unconditional per lane, as above)
         __builtin_amdgcn_sched_barrier(0);
 
-        // the next tile's inputs are requested in front of the last feature-split layer and written to the other input
-        // buffer in front of its barrier (a tile past the end is a tile of zeros)
-        u32x4 xnext[KS0];
+        // the next tile's inputs are requested now (they come from HBM and take a microsecond) and written to the other
+        // input buffer in front of the last feature-split layer's barrier (a tile past the end is a tile of zeros)
         auto nothing = [] {};
-        auto fetch_next = [&] { load_x(has_next ? next : tiles, xnext); };
-        auto publish_next = [&] { store_x(xbuf ^ 1, xnext); };
+        const u32x4 xnext = load_x(has_next ? next : tiles);
+        const bool xnext_valid = x_valid(has_next ? next : tiles);
+        __builtin_amdgcn_sched_barrier(0);
+        auto publish_next = [&] { store_x(xbuf ^ 1, xnext, xnext_valid); };
 
-        layer(IC<0>{}, xbuf * RS_X_BYTES, RS_ACT_BYTES, nothing);
+        layer(IC<0>{}, xbuf * RS_X_BYTES, BUF_A, nothing);
         SP_RS_STAMP(1);
         if constexpr (S == 2) {
-            fetch_next();
-            __builtin_amdgcn_sched_barrier(0);
-            layer(IC<1>{}, RS_ACT_BYTES, 0, publish_next);
+            layer(IC<1>{}, BUF_A, BUF_B, publish_next);
             SP_RS_STAMP(2);
         } else {
-            layer(IC<1>{}, RS_ACT_BYTES, 0, nothing);
+            layer(IC<1>{}, BUF_A, BUF_B, nothing);
             SP_RS_STAMP(2);
-            fetch_next();
-            __builtin_amdgcn_sched_barrier(0);
-            layer(IC<2>{}, 0, RS_ACT_BYTES, publish_next);
+            layer(IC<2>{}, BUF_B, BUF_C, publish_next);
         }
         SP_RS_STAMP(3);
 
-        // ---- output layer: rows 16 wave .. + 15 of the tile; MFMA row i is output i ----
-        constexpr int last_in = (S & 1) ? RS_ACT_BYTES : 0;
+        // ---- output layer: rows 16 w4 .. + 15 of the tile (both waves of the pair, each finishes half of the rows);
+        //      MFMA row i is output i ----
+        constexpr int last_in = S == 3 ? BUF_C : BUF_B;
         f32x4 d;
         {
             u32x4 al[8], WL[8];
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) al[ks] = read_at(last_in, wave, ks);
+            for (int ks = 0; ks < 8; ++ks) al[ks] = read_at(last_in, w4, ks);
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) WL[ks] = *reinterpret_cast<const u32x4*>(lds + RS_WL_OFF + ks * 1024 + lane * 16);
-            if constexpr (S == 3) {
-                // the next tile's first layer writes the buffer these reads come from: nobody goes on before
-                // everybody has them
-                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-            }
             // even and odd k-steps add up separately: two chains of four dependent MFMAs instead of one of eight
             f32x4 dd[2];
 #pragma unroll
@@ -427,11 +429,11 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
             if (out.stride > NOUT && (out.stride & 3) == 0) {
                 const int s4 = out.stride >> 2, c0 = (NOUT + 3) >> 2;    // float4 groups per row; the first one that is all zeros
                 fill_end = 4 * c0;
-                const long first_row = row0 + wave * 16;
+                const long first_row = row0 + w4 * 16;
                 float* block = out.policy + first_row * out.stride;
                 for (int idx = lane; idx < 16 * s4; idx += 64) {
                     const int r = idx / s4, c = idx - r * s4;
-                    if (c >= c0 && first_row + r < batch)
+                    if (c >= c0 && (r >> 3) == wp && first_row + r < batch)
                         store16_through(reinterpret_cast<f32x4*>(block + (long)r * out.stride + 4 * c), f32x4{0.f, 0.f, 0.f, 0.f});
                 }
             }
@@ -446,7 +448,7 @@ __global__ __launch_bounds__(256) void mlp_resident_kernel(const MlpResidentArgs
                 if (head_ok) head_row4_any(out.head, out, p, head_row_idx, NOUT, limit, u_row, fill_end);
             } else {
                 // the wave's 16 x NOUT outputs staged in its own KiB of LDS
-                float* head_rows = reinterpret_cast<float*>(lds + RS_HEAD_OFF + wave * 1024);
+                float* head_rows = reinterpret_cast<float*>(lds + RS_HEAD_OFF + w4 * 1024);   // (the pair writes the same values)
                 f32x4 v = d;
                 if (bias != nullptr) {
 #pragma unroll
@@ -498,19 +500,20 @@ int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a,
     const bool plain = a.nout <= 4 && a.out_stride == a.nout && a.logits == nullptr && a.action != nullptr && a.b[n_layers - 1] == nullptr;
     const void* kernel = dtype == SP_F16 ? (packed ? pick_resident<SP_F16, true>(ks0, n_layers, plain) : pick_resident<SP_F16, false>(ks0, n_layers, plain))
                                          : (packed ? pick_resident<SP_BF16, true>(ks0, n_layers, plain) : pick_resident<SP_BF16, false>(ks0, n_layers, plain));
-    int rc = ensure_dynamic_lds(kernel, RS_LDS_TOTAL);
+    const int lds_bytes = rs_lds_total(ks0);
+    int rc = ensure_dynamic_lds(kernel, lds_bytes);
     if (rc != SP_OK) return rc;
     const long cus = device_cu_count();
     const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
     void* args[] = {(void*)&a};
-    hipError_t e = hipLaunchKernel(kernel, dim3(blocks), dim3(256), args, RS_LDS_TOTAL, stream);
+    hipError_t e = hipLaunchKernel(kernel, dim3(blocks), dim3(RS_THREADS), args, lds_bytes, stream);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "%s: launch failed: %s", what, hipGetErrorString(e));
     return check_launch(what);
 }
 
 namespace {
 struct MlpResidentKernelNames {
-    MlpResidentKernelNames() { register_kernel("mlp_forward_resident", (const void*)mlp_resident_kernel<SP_F16, 1, 4, true, true>, 256); }
+    MlpResidentKernelNames() { register_kernel("mlp_forward_resident", (const void*)mlp_resident_kernel<SP_F16, 1, 4, true, true>, RS_THREADS); }
 } mlp_resident_kernel_names;
 }  // namespace
 
@@ -518,6 +521,6 @@ struct MlpResidentKernelNames {
 
 #ifdef SP_RS_TIMELINE
 extern "C" int sp_debug_resident_timeline(unsigned long long* host_out) {
-    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(sp::sp_rs_timeline), sizeof(unsigned long long) * 256 * 4 * 16 * 8);
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(sp::sp_rs_timeline), sizeof(unsigned long long) * 256 * 8 * 16 * 8);
 }
 #endif
