@@ -52,20 +52,23 @@ struct MlpResidentArgs {
     int* action;
     float* logits;
     long batch;
-    int tiles;
+    int tiles;                           // steps of the walk (filled in by mlp_resident_launch)
     int head, mask_size, k0, nout, out_stride;
     PhiloxStream ph;
 };
 
 bool mlp_resident_takes(int n_layers, const int32_t* dims, int nout);
 int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a, hipStream_t stream, const char* what);
-// Tiles per compute unit from which the resident kernel is used (its one-time load of all weights has to pay):
-// packed weights stream in at the texture path's full rate, row-major ones at about a quarter of it.
+// 64-row tiles per compute unit from which the resident kernel is used: its one-time load of all weights has to pay,
+// and it walks tiles in pairs, so few tiles per unit leave units idle in the last round.  Measured against the
+// per-tile kernels (32 -> 256 -> 256 -> 256 -> 3, us per launch, per-tile / resident): packed weights 65536 rows
+// 19.7 / 19.6, 98304 29.1 / 26.7, 131072 39.1 / 33.8, 262144 76.3 / 61.8; row-major weights (which stream in at about
+// a quarter of the rate) 98304 31.8 / 32.7, 131072 42.7 / 39.9, 262144 81.7 / 69.3.
 #ifndef SP_MLP_RESIDENT_MIN_TILES_PACKED
-#define SP_MLP_RESIDENT_MIN_TILES_PACKED 2
+#define SP_MLP_RESIDENT_MIN_TILES_PACKED 6
 #endif
 #ifndef SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR
-#define SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR 4
+#define SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR 8
 #endif
 
 // The Philox stream of a head that draws its own uniforms: the sampling node of the layer graph works on rows of

@@ -8,7 +8,10 @@
 // up to two such layers -- wave v keeps output features 32 v .. 32 v + 31 of each (64 + 64 registers, in MFMA operand
 // order); the few KiB of the first and the last layer sit in LDS -- and walks over the tiles blockIdx.x,
 // blockIdx.x + gridDim.x, ...  A tile then costs its MFMAs, the exchange of activations through LDS (one barrier
-// per layer), the head, and 4 KiB of input.
+// per layer), the head, and 4 KiB of input.  Tiles are walked in PAIRS: every layer is done for both tiles of a pair
+// (128 rows) between two barriers, so the start-up and the drain of a layer -- first fragments on their way, last
+// conversion and write, the barrier -- are paid once per 128 rows, a wave's head finishes 16 rows at once, and the
+// two waves of a SIMD, which drift apart between barriers, fill each other's gaps.
 // Two waves per SIMD, not one with twice the features: a wave cannot issue anything else in the shadow of its own
 // MFMAs (every LDS read, conversion or wait of a lone wave costs the matrix pipe 4-5 cycles; measured on the
 // four-wave form of this kernel: 3.0-3.2 k cycles per 256 x 256 layer for 2 k cycles of MFMA), its neighbour on the
@@ -29,16 +32,16 @@
 namespace sp {
 
 constexpr int RS_ROWS = 64;                              // batch rows per tile
+constexpr int RS_PAIR_ROWS = 2 * RS_ROWS;                // ... per step of a workgroup's walk
 constexpr int RS_WAVES = 8;
 constexpr int RS_THREADS = RS_WAVES * 64;
-constexpr int RS_ACT_BYTES = RS_ROWS * 512;              // one activation buffer: 64 rows x 256 features x 2 bytes
-constexpr int RS_X_OFF = 3 * RS_ACT_BYTES;               // three of those, then two input buffers, 64 rows x 128 bytes
-constexpr int RS_X_BYTES = RS_ROWS * 128;                //   (a tile's inputs are written while the tile before it is computed)
-constexpr int RS_BIAS_OFF = RS_X_OFF + 2 * RS_X_BYTES;   // the biases of the feature-split layers, 256 f32 each
-constexpr int RS_HEAD_OFF = RS_BIAS_OFF + 3 * 1024;      // a KiB per 16 rows: the outputs of a head wider than 4
-constexpr int RS_WL_OFF = RS_HEAD_OFF + 4 * 1024;        // the output layer's weights: 8 k-steps x 1 KiB
-constexpr int RS_W0_OFF = RS_WL_OFF + 8 * 1024;          // the first layer's: per wave KS0 k-steps x 2 tiles x 1 KiB
-constexpr int rs_lds_total(int ks0) { return RS_W0_OFF + RS_WAVES * ks0 * 2048; }
+constexpr int RS_TILE_BYTES = RS_ROWS * 512;             // activations of one tile: 64 rows x 256 features x 2 bytes
+constexpr int RS_ACT_BYTES = 2 * RS_TILE_BYTES;          // ... of a pair
+constexpr int RS_X_OFF = 2 * RS_ACT_BYTES;               // two activation buffers, then the inputs of a pair: 128 rows x 128 bytes
+constexpr int RS_HEAD_OFF = RS_X_OFF + RS_PAIR_ROWS * 128;   // a KiB per wave: the outputs of a head wider than 4
+constexpr int RS_WL_OFF = RS_HEAD_OFF + RS_WAVES * 1024;     // the output layer's weights: 8 k-steps x 1 KiB
+constexpr int RS_LDS_TOTAL = RS_WL_OFF + 8 * 1024;           // = 160 KiB, all of a compute unit's LDS
+static_assert(RS_LDS_TOTAL <= 160 * 1024, "fits the LDS of one compute unit");
 
 #ifdef SP_RS_TIMELINE
 __device__ unsigned long long sp_rs_timeline[256 * 8 * 16 * 8];
@@ -69,37 +72,30 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
     const int K0 = a.k0, NOUT = a.nout;
     const unsigned char* const x_ptr = (const unsigned char*)a.x;
     const long batch = a.batch;
-    const int tiles = a.tiles;
+    const int pairs = a.tiles;                               // steps of the walk: pairs of tiles
     const HeadOut out = HeadOut{a.policy, a.action, a.logits, a.head, a.out_stride};
     const int mask_size = a.mask_size;
     const float* const u_ptr = a.u;
     const float* const last_bias = a.b[S];
     const int ph_mode = a.ph.philox_mode;
-
-    // ---- the biases of the feature-split layers into their LDS table (feature tid of each) ----
     unsigned has_bias = 0;                                   // bit l: layer l has a bias (uniform)
 #pragma unroll
-    for (int l = 0; l < S; ++l) {
-        const float* b = a.b[l];
-        if (b != nullptr) {
-            has_bias |= 1u << l;
-            if (tid < 256) *reinterpret_cast<float*>(lds + RS_BIAS_OFF + l * 1024 + tid * 4) = b[tid];
-        }
-    }
+    for (int l = 0; l < S; ++l)
+        if (a.b[l] != nullptr) has_bias |= 1u << l;
 
-    // ---- the weights, once.  The 256 x 256 layers go into the accumulation registers and stay there (block (k-step,
+    // ---- the weights of the 256 x 256 layers, once: into the accumulation registers, where they stay (block (k-step,
     //      feature tile) = 4 registers: lane (i, q) holds the 8 K-values 32 ks + 8 q .. of feature row i of the
-    //      tile; this wave's tiles are 2 wp and 2 wp + 1 of the four that make up slice w4); the first layer's few
-    //      blocks (this wave's) and the output layer's eight (everybody's) go to LDS in the same order, from where a
-    //      tile reads them back with one ds_read_b128 each ----
+    //      tile; this wave's tiles are 2 wp and 2 wp + 1 of the four that make up slice w4).  The output layer's
+    //      eight blocks (everybody's) go to LDS in the same order; the first layer's few blocks are fetched per
+    //      pair of tiles (they are a KiB or two per wave, and the L2 has them) ----
     // (The second 256 x 256 layer keeps its last k-step in ordinary registers: a file that is spoken for to the last
     //  register makes the allocator park a block elsewhere and copy it in front of every use.)
     u32x4 W1[8][2], W2[S == 3 ? 7 : 1][2], W2v[2];
+    const int i16 = lane & 15;
+    // feature row of lane i in tile t of slice w4: 64 w4 + 32 (t / 2) + 8 (i / 4) + 4 (t % 2) + i % 4
+    const unsigned lane_row = (unsigned)(8 * (i16 >> 2) + (i16 & 3));
+    const long tile_row = 64 * w4 + 32 * wp;                 // first feature row of this wave's tile 0 (tile 1: + 4)
     {
-        const int i16 = lane & 15;
-        // feature row of lane i in tile t of slice w4: 64 w4 + 32 (t / 2) + 8 (i / 4) + 4 (t % 2) + i % 4
-        const unsigned lane_row = (unsigned)(8 * (i16 >> 2) + (i16 & 3));
-        unsigned char* const w0_lds = lds + RS_W0_OFF + wave * (KS0 * 2048) + lane * 16;
         unsigned char* const wl_lds = lds + RS_WL_OFF + lane * 16;
         if constexpr (PACKED) {
             const unsigned char* const packed = (const unsigned char*)a.packed;
@@ -120,23 +116,14 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
                 for (int h = 0; h < 2; ++h)
                     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[h]) : "v"(voff), "s"(packed + first_bytes + 131072 + ((long)(w4 * 8 + 7) * 4 + 2 * wp + h) * 1024) : "memory");
             }
-#pragma unroll
-            for (int ks = 0; ks < KS0; ++ks)
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    *reinterpret_cast<u32x4*>(w0_lds + (ks * 2 + h) * 1024) =
-                        *reinterpret_cast<const u32x4*>(packed + ((long)(w4 * KS0 + ks) * 4 + 2 * wp + h) * 1024 + voff);
             *reinterpret_cast<u32x4*>(wl_lds + wave * 1024) =
                 *reinterpret_cast<const u32x4*>(packed + first_bytes + (long)(S - 1) * 131072 + wave * 1024 + voff);
         } else {
-            // row-major: base of tile t = row 64 w4 + 32 (t / 2) + 4 (t % 2), i.e. 64 w4 + 32 wp + 4 h for this wave's
-            // tile h; k-step ks = 64 bytes further per step; the lane adds its row inside the tile and its quarter
-            const unsigned char* const w0 = (const unsigned char*)a.w[0];
+            // row-major: k-step ks = 64 bytes further per step; the lane adds its row inside the tile and its quarter
             const unsigned char* const w1 = (const unsigned char*)a.w[1];
             const unsigned char* const w2 = (const unsigned char*)a.w[S == 3 ? 2 : 1];
             const unsigned char* const wl = (const unsigned char*)a.w[S];
             const unsigned vo_h = (unsigned)((lane_row * 256 + 8 * q) * 2);
-            const long tile_row = 64 * w4 + 32 * wp;
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
@@ -152,51 +139,66 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
                 for (int h = 0; h < 2; ++h)
                     asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(W2v[h]) : "v"(vo_h), "s"(w2 + (tile_row + 4 * h) * 512 + 7 * 64) : "memory");
             }
-            // layer 0: rows of K0 values; k-values past K0 are zeros
-#pragma unroll
-            for (int ks = 0; ks < KS0; ++ks) {
-                const bool ok = 32 * ks + 8 * q < K0;
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    u32x4 v = zero_u4;
-                    if (ok) v = *reinterpret_cast<const u32x4*>(w0 + ((tile_row + 4 * h + lane_row) * K0 + 32 * ks + 8 * q) * 2);
-                    *reinterpret_cast<u32x4*>(w0_lds + (ks * 2 + h) * 1024) = v;
-                }
-            }
             // output layer: MFMA row i is output i; rows past the computed outputs are zeros
-            {
-                u32x4 v = zero_u4;
-                if (i16 < NOUT) v = *reinterpret_cast<const u32x4*>(wl + ((long)i16 * 256 + 32 * wave + 8 * q) * 2);
-                *reinterpret_cast<u32x4*>(wl_lds + wave * 1024) = v;
-            }
+            u32x4 v = zero_u4;
+            if (i16 < NOUT) v = *reinterpret_cast<const u32x4*>(wl + ((long)i16 * 256 + 32 * wave + 8 * q) * 2);
+            *reinterpret_cast<u32x4*>(wl_lds + wave * 1024) = v;
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
+    // the first layer's blocks of this wave (KS0 k-steps x 2 tiles), as the MFMAs read them; k-values past K0 are zeros
+    auto load_w0 = [&](u32x4 (&w)[KS0][2]) {
+#pragma unroll
+        for (int ks = 0; ks < KS0; ++ks)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if constexpr (PACKED) {
+                    w[ks][h] = *reinterpret_cast<const u32x4*>((const unsigned char*)a.packed + ((long)(w4 * KS0 + ks) * 4 + 2 * wp + h) * 1024 + lane * 16);
+                } else {
+                    const bool ok = 32 * ks + 8 * q < K0;
+                    const u32x4 v = *reinterpret_cast<const u32x4*>((const unsigned char*)a.w[0] + ((tile_row + 4 * h + lane_row) * K0 + (ok ? 32 * ks + 8 * q : 0)) * 2);
+                    w[ks][h] = ok ? v : zero_u4;
+                }
+            }
+    };
 
     // ---- operand addresses ----
-    // activations: row r, 16-byte piece P (of 32) lives in slot (P & 16) | ((P ^ r) & 15) of the row's 512 bytes
+    // activations: row r, 16-byte piece P (of 32) lives in slot (P & 16) | ((P ^ r) & 15) of the row's 512 bytes;
+    // rows 64 g + 16 bt + j: tile g of the pair, batch tile bt
     unsigned aoff[4];
 #pragma unroll
     for (int k4 = 0; k4 < 4; ++k4) aoff[k4] = (unsigned)(j * 512 + (((4 * k4 + q) ^ j) << 4));
-    auto read_at = [&](int base, int bt, int ks) {
-        return *reinterpret_cast<const u32x4*>(lds + base + aoff[ks & 3] + bt * 8192 + (ks >> 2) * 256);
+    auto read_at = [&](int base, int g, int bt, int ks) {
+        return *reinterpret_cast<const u32x4*>(lds + base + aoff[ks & 3] + g * RS_TILE_BYTES + bt * 8192 + (ks >> 2) * 256);
     };
     // outputs: this wave's two tiles give lane (j, q) the features 64 w4 + 32 wp + 8 q .. + 7 of batch row j
     const unsigned pw = (unsigned)(j * 512 + (w4 >> 1) * 256 + (((8 * (w4 & 1) + 4 * wp + q) ^ j) << 4));
 
-    // the 16-byte piece of a tile's input rows this thread moves (4 KS0 pieces per row: 256 KS0 pieces in all)
-    const int x_r = tid / (4 * KS0), x_pc = tid % (4 * KS0);
-    const bool x_mine = tid < 256 * KS0;
-    // (the load itself is unconditional -- a piece outside the batch or past K0 reads the tensor's first bytes and is
-    //  replaced by zeros when it is stored: a load under a condition would be waited for where the branches meet)
-    auto x_valid = [&](int tile) { return x_mine && (long)tile * RS_ROWS + x_r < batch && x_pc * 8 < K0; };
-    auto load_x = [&](int tile) {
-        const long off = x_valid(tile) ? (((long)tile * RS_ROWS + x_r) * K0 + x_pc * 8) * 2 : 0;
-        return *reinterpret_cast<const u32x4*>(x_ptr + off);
+    // the 16-byte pieces of a pair's input rows this thread moves: 4 KS0 pieces per row, 512 KS0 in all, KS0 per thread.
+    // (The loads are unconditional -- a piece outside the batch or past K0 reads the tensor's first bytes and is replaced
+    //  by zeros when it is stored: a load under a condition would be waited for where the branches meet.)
+    auto x_valid = [&](int pair, int i) {
+        const int idx = tid + RS_THREADS * i;
+        const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
+        return (long)pair * RS_PAIR_ROWS + r < batch && pc * 8 < K0;
+    };
+    auto load_x = [&](int pair, u32x4 (&v)[KS0]) {
+#pragma unroll
+        for (int i = 0; i < KS0; ++i) {
+            const int idx = tid + RS_THREADS * i;
+            const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
+            const long off = x_valid(pair, i) ? (((long)pair * RS_PAIR_ROWS + r) * K0 + pc * 8) * 2 : 0;
+            v[i] = *reinterpret_cast<const u32x4*>(x_ptr + off);
+        }
     };
     // inputs: row r, piece pc (of at most 8) lives in slot (pc ^ r) & 7 of the row's 128 bytes
-    auto store_x = [&](int buf, const u32x4& v, bool valid) {
-        if (x_mine) *reinterpret_cast<u32x4*>(lds + RS_X_OFF + buf * RS_X_BYTES + x_r * 128 + (((x_pc ^ x_r) & 7) << 4)) = valid ? v : zero_u4;
+    auto store_x = [&](int pair, const u32x4 (&v)[KS0]) {
+#pragma unroll
+        for (int i = 0; i < KS0; ++i) {
+            const int idx = tid + RS_THREADS * i;
+            const int r = idx / (4 * KS0), pc = idx % (4 * KS0);
+            *reinterpret_cast<u32x4*>(lds + RS_X_OFF + r * 128 + (((pc ^ r) & 7) << 4)) = x_valid(pair, i) ? v[i] : zero_u4;
+        }
     };
     unsigned xoff[KS0];
 #pragma unroll
@@ -231,179 +233,179 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
 #undef SP_RS_MFMA_ALL
 #undef SP_RS_MFMA
 
-    // One feature-split layer L reading the activations at LDS offset `in_base` and writing its outputs (bias, relu,
-    // rounding) to `out_base`.  K-steps in order, the activation fragments of the next k-step read one at a time behind
-    // the first MFMAs.  The LAST two k-steps (the last one, of a layer that has only one) are walked batch tile by
-    // batch tile instead: tile bt's sums are then complete while tiles bt + 1 .. 3 are still being multiplied, and
-    // its outputs are converted and written one packed word per MFMA; only the last tile's conversion stands alone.
-    // `before_barrier` runs in front of the barrier that makes the outputs everyone's inputs.
+
+    u32x4 W0[KS0][2];                                        // the first layer's blocks, fetched anew for every pair of tiles
+
+    // One feature-split layer L for both tiles of the pair, reading the activations at LDS offset `in_base` and
+    // writing its outputs (bias, relu, rounding) to `out_base`.  Per tile: k-steps in order, the activation fragments
+    // of the next k-step read one at a time behind the first MFMAs.  The LAST two k-steps (the last one, of a layer
+    // that has only one) are walked batch tile by batch tile instead: batch tile bt's sums are then complete while
+    // tiles bt + 1 .. 3 are still being multiplied, and its outputs are converted and written one packed word per
+    // MFMA; only the last batch tile's conversion stands alone.  `before_barrier` runs in front of the barrier that
+    // makes the outputs everyone's inputs.
     auto layer = [&](auto L_, int in_base, int out_base, auto&& before_barrier) {
         constexpr int L = decltype(L_)::value;
         constexpr int KS = L == 0 ? KS0 : 8;
         constexpr int TAILK = KS >= 2 ? 2 : 1;                // k-steps walked batch tile by batch tile
         constexpr int HEADK = KS - TAILK;
         const bool with_bias = (has_bias & (1u << L)) != 0;   // uniform
-        u32x4 W0[L == 0 ? KS0 : 1][2];                        // the first layer's weights come back from LDS
-        if constexpr (L == 0) {
-#pragma unroll
-            for (int ks = 0; ks < KS0; ++ks)
-#pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    W0[ks][h] = *reinterpret_cast<const u32x4*>(lds + RS_W0_OFF + wave * (KS0 * 2048) + (ks * 2 + h) * 1024 + lane * 16);
-        }
         auto mm = [&](f32x4& c, int ks, int h, const u32x4& x, bool first, auto WAIT_) {
             if constexpr (L == 0) mfma_v(c, W0[ks][h], x, first, WAIT_);
             else if constexpr (L == 1) mfma_a(c, W1[ks][h], x, first, WAIT_);
             else if (ks < 7) mfma_a(c, W2[ks < 7 ? ks : 0][h], x, first, WAIT_);
             else mfma_v(c, W2v[h], x, first, WAIT_);
         };
-        // activation fragment (batch tile bt, k-step ks) of this layer's input
-        auto read_in = [&](int bt, int ks) {
-            if constexpr (L == 0) return *reinterpret_cast<const u32x4*>(lds + in_base + xoff[ks] + bt * 2048);
-            else return read_at(in_base, bt, ks);
-        };
-        u32x4 bf[2][4];
-#pragma unroll
-        for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_in(bt, 0);
-        rs_static_for<0, HEADK>([&](auto KS_) {
-            constexpr int ks = decltype(KS_)::value;
-            rs_static_for<0, 2>([&](auto H_) {
-                constexpr int h = decltype(H_)::value;
-#pragma unroll
-                for (int bt = 0; bt < 4; ++bt) {
-                    mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<0>{});
-#ifndef SP_RS_ABL_NOREAD
-                    if (h == 0) bf[(ks + 1) & 1][bt] = read_in(bt, ks + 1);
-#else
-                    if (h == 0) bf[(ks + 1) & 1][bt] = bf[ks & 1][bt];
-#endif
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            });
-        });
-        // ---- the end of the layer, batch tile by batch tile ----
-        if constexpr (TAILK == 2) {
-            // fragments of k-step KS - 1 (those of KS - 2 were read behind the MFMAs of the k-step before it, or above)
-            if constexpr (HEADK == 0) {
-#pragma unroll
-                for (int bt = 0; bt < 4; ++bt) bf[1][bt] = read_in(bt, 1);
-            } else {
-#pragma unroll
-                for (int bt = 0; bt < 4; ++bt) bf[(KS - 1) & 1][bt] = read_in(bt, KS - 1);
-            }
-        }
         // (two copies, with and without a bias: the test is uniform and made once per layer)
-        auto end_of_layer = [&](auto HAS_BIAS_) {
-            constexpr bool has_b = decltype(HAS_BIAS_)::value != 0;
-            f32x4 bias_r[2];                                  // [h]: features 64 w4 + 32 wp + 8 q + 4 h .. + 3
-            if constexpr (has_b) {
+        auto both_tiles = [&](auto HAS_BIAS_) {
+        constexpr bool has_b = decltype(HAS_BIAS_)::value != 0;
+        f32x4 bias_r[2];                                      // [h]: features 64 w4 + 32 wp + 8 q + 4 h .. + 3
+        if constexpr (has_b) {
 #pragma unroll
-                for (int h = 0; h < 2; ++h)
-                    bias_r[h] = *reinterpret_cast<const f32x4*>(lds + RS_BIAS_OFF + L * 1024 + (64 * w4 + 32 * wp + 8 * q + 4 * h) * 4);
-            }
-            // word E (0..3) of batch tile BT's outputs: tile E / 2, accumulator rows 2 (E % 2) and + 1; one 16-byte write
-            u32x4 cv;
-            auto convert_word = [&](auto BT_, auto E_) {
-                constexpr int bt = decltype(BT_)::value, e = decltype(E_)::value;
-                constexpr int h = e >> 1, r = 2 * (e & 1);
-                float a0 = acc[bt][h][r], a1 = acc[bt][h][r + 1];
-                if constexpr (has_b) {
-                    a0 += bias_r[h][r];
-                    a1 += bias_r[h][r + 1];
-                }
-#ifndef SP_RS_ABL_NOCONV
-                cv[e] = pack_relu2<DT>(a0, a1);
-#else
-                cv[e] = __builtin_bit_cast(unsigned, a0);
-#endif
-                if constexpr (e == 3) *reinterpret_cast<u32x4*>(lds + out_base + pw + bt * 8192) = cv;
+            for (int h = 0; h < 2; ++h) bias_r[h] = *reinterpret_cast<const f32x4*>(a.b[L] + 64 * w4 + 32 * wp + 8 * q + 4 * h);
+        }
+        rs_static_for<0, 2>([&](auto G_) {
+            constexpr int g = decltype(G_)::value;            // tile of the pair
+            // activation fragment (batch tile bt, k-step ks) of this layer's input
+            auto read_in = [&](int bt, int ks) {
+                if constexpr (L == 0) return *reinterpret_cast<const u32x4*>(lds + xoff[ks] + g * (RS_ROWS * 128) + bt * 2048);
+                else return read_at(in_base, g, bt, ks);
             };
-            rs_static_for<0, 4>([&](auto BT_) {
-                constexpr int bt = decltype(BT_)::value;
-                rs_static_for<0, 2 * TAILK>([&](auto M_) {
-                    constexpr int m = decltype(M_)::value;
-                    constexpr int ks = HEADK + m / 2, h = m % 2;
-                    // (wait states in front of the MFMA where the bias additions' register traffic surrounds it; the
-                    //  copy without a bias has none of it, and the build's scan of the generated code holds it to that)
-                    mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<has_b ? 1 : 0>{});
-                    __builtin_amdgcn_sched_barrier(0);
-                    if constexpr (bt > 0) {                   // the tile before this one is complete: 4 words over these MFMAs
-                        constexpr int per = 4 / (2 * TAILK);
-                        rs_static_for<0, per>([&](auto I_) { convert_word(IC<bt - 1>{}, IC<per * m + decltype(I_)::value>{}); });
+            u32x4 bf[2][4];
+#pragma unroll
+            for (int bt = 0; bt < 4; ++bt) bf[0][bt] = read_in(bt, 0);
+            rs_static_for<0, HEADK>([&](auto KS_) {
+                constexpr int ks = decltype(KS_)::value;
+                rs_static_for<0, 2>([&](auto H_) {
+                    constexpr int h = decltype(H_)::value;
+#pragma unroll
+                    for (int bt = 0; bt < 4; ++bt) {
+                        mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<0>{});
+                        if (h == 0) bf[(ks + 1) & 1][bt] = read_in(bt, ks + 1);
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 });
             });
-            // the last tile: the s_nops are the wait states between the last MFMA and the first read of its result,
-            // which the compiler does not know about
-            asm volatile("s_nop 15\n\ts_nop 3" ::: "memory");
-            rs_static_for<0, 4>([&](auto E_) { convert_word(IC<3>{}, E_); });
+            // ---- the end of the tile's layer, batch tile by batch tile ----
+            if constexpr (TAILK == 2) {
+                // fragments of k-step KS - 1 (those of KS - 2 were read behind the MFMAs of the k-step before it, or above)
+                if constexpr (HEADK == 0) {
+#pragma unroll
+                    for (int bt = 0; bt < 4; ++bt) bf[1][bt] = read_in(bt, 1);
+                } else {
+#pragma unroll
+                    for (int bt = 0; bt < 4; ++bt) bf[(KS - 1) & 1][bt] = read_in(bt, KS - 1);
+                }
+            }
+            {
+                // word E (0..3) of batch tile BT's outputs: tile E / 2, accumulator rows 2 (E % 2) and + 1; one 16-byte write
+                u32x4 cv;
+                auto convert_word = [&](auto BT_, auto E_) {
+                    constexpr int bt = decltype(BT_)::value, e = decltype(E_)::value;
+                    constexpr int h = e >> 1, r = 2 * (e & 1);
+                    float a0 = acc[bt][h][r], a1 = acc[bt][h][r + 1];
+                    if constexpr (has_b) {
+                        a0 += bias_r[h][r];
+                        a1 += bias_r[h][r + 1];
+                    }
+                    cv[e] = pack_relu2<DT>(a0, a1);
+                    if constexpr (e == 3) *reinterpret_cast<u32x4*>(lds + out_base + pw + g * RS_TILE_BYTES + bt * 8192) = cv;
+                };
+                rs_static_for<0, 4>([&](auto BT_) {
+                    constexpr int bt = decltype(BT_)::value;
+                    rs_static_for<0, 2 * TAILK>([&](auto M_) {
+                        constexpr int m = decltype(M_)::value;
+                        constexpr int ks = HEADK + m / 2, h = m % 2;
+                        // (wait states in front of the MFMA where the bias additions' register traffic surrounds it; the
+                        //  copy without a bias has none of it, and the build's scan of the generated code holds it to that)
+                        mm(acc[bt][h], ks, h, bf[ks & 1][bt], ks == 0, IC<has_b ? 1 : 0>{});
+                        __builtin_amdgcn_sched_barrier(0);
+                        if constexpr (bt > 0) {               // the batch tile before this one is complete: 4 words over these MFMAs
+                            constexpr int per = 4 / (2 * TAILK);
+                            rs_static_for<0, per>([&](auto I_) { convert_word(IC<bt - 1>{}, IC<per * m + decltype(I_)::value>{}); });
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    });
+                });
+                // the last batch tile: the s_nops are the wait states between the last MFMA and the first read of its
+                // result, which the compiler does not know about (the accumulators are operands so that it cannot
+                // move their conversion in front of the wait)
+                asm volatile("s_nop 15\n\ts_nop 3" : "+v"(acc[3][0]), "+v"(acc[3][1]) : : "memory");
+                rs_static_for<0, 4>([&](auto E_) { convert_word(IC<3>{}, E_); });
+            }
+        });
         };
-        if (with_bias) end_of_layer(IC<1>{});
-        else end_of_layer(IC<0>{});
+        if (with_bias) both_tiles(IC<1>{});
+        else both_tiles(IC<0>{});
         before_barrier();
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     };
 
-    // ---- the first tile's inputs ----
-    int tile = blockIdx.x;
-    int xbuf = 0;
-    store_x(0, load_x(tile), x_valid(tile));
-    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");          // inputs, biases and the small layers are in LDS
+    // ---- the first pair's inputs and first-layer weights ----
+    int pair = blockIdx.x;
+    {
+        u32x4 xin[KS0];
+        load_x(pair, xin);
+        store_x(pair, xin);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");          // inputs and the output layer's weights are in LDS
 
 #ifdef SP_RS_TIMELINE
-    // measurement build: per wave and tile walked, the cycle counter at every phase boundary (8 words per tile)
+    // measurement build: per wave and step of the walk, the cycle counter at every phase boundary (8 words per step)
     int tl_n = 0;
 #define SP_RS_STAMP(K) do { if (lane == 0 && tl_n < 16) sp_rs_timeline[(((long)blockIdx.x * 8 + wave) * 16 + tl_n) * 8 + (K)] = (K) == 7 ? __builtin_amdgcn_s_memrealtime() : __builtin_amdgcn_s_memtime(); } while (0)
 #else
 #define SP_RS_STAMP(K) do {} while (0)
 #endif
-    // The activation buffers rotate A -> B -> C -> A: the output layer of tile n reads a buffer that tile n + 1 does not
-    // write before its second barrier, so a wave that is done with its head goes on without waiting for the others.
-    constexpr int BUF_A = 0, BUF_B = RS_ACT_BYTES, BUF_C = 2 * RS_ACT_BYTES;
+    // Two activation buffers P and Q.  Three feature-split layers: inputs -> P -> Q -> P, and the output layer reads P,
+    // which the next pair's first layer writes again: a barrier behind the output layer's reads keeps the two apart.
+    // Two: inputs -> P -> Q, the output layer reads Q, and nothing of the next pair touches Q before its second barrier.
+    constexpr int BUF_P = 0, BUF_Q = RS_ACT_BYTES;
     for (;;) {
         SP_RS_STAMP(0);
-        const int next = tile + (int)gridDim.x;
-        const bool has_next = next < tiles;
-        const long row0 = (long)tile * RS_ROWS;
-        // the head of 16 rows is shared by the two waves that hold slice w4: rows 16 w4 + 8 wp .. + 7 each
-        const long head_row_idx = row0 + w4 * 16 + j;        // the row lanes 0..15 could finish
-        const bool head_ok = lane < 16 && (j >> 3) == wp && head_row_idx < batch;
-        float u_row = 1.f;
-        if (ph_mode >= 0) u_row = reference_row_uniform(a.ph, head_ok ? head_row_idx : 0);
-        else if (u_ptr != nullptr) u_row = u_ptr[head_ok ? head_row_idx : 0];      // (unconditional per lane, as above)
+        load_w0(W0);                                         // (a KiB or two from the L2, first in line)
+        const int next = pair + (int)gridDim.x;
+        const bool has_next = next < pairs;
+        float u_row = 1.f;                                   // of the row lanes 0..15 finish
+        {
+            const long r = (long)pair * RS_PAIR_ROWS + wave * 16 + j;
+            const long r_ok = lane < 16 && r < batch ? r : 0;
+            if (ph_mode >= 0) u_row = reference_row_uniform(a.ph, r_ok);
+            else if (u_ptr != nullptr) u_row = u_ptr[r_ok];                        // (unconditional per lane, as above)
+        }
+        // the next pair's inputs are requested now (they come from HBM and take a microsecond) and written over this
+        // pair's in front of the last feature-split layer's barrier (a pair past the end is a pair of zeros)
+        u32x4 xnext[KS0];
+        load_x(has_next ? next : pairs, xnext);
         __builtin_amdgcn_sched_barrier(0);
-
-        // the next tile's inputs are requested now (they come from HBM and take a microsecond) and written to the other
-        // input buffer in front of the last feature-split layer's barrier (a tile past the end is a tile of zeros)
         auto nothing = [] {};
-        const u32x4 xnext = load_x(has_next ? next : tiles);
-        const bool xnext_valid = x_valid(has_next ? next : tiles);
-        __builtin_amdgcn_sched_barrier(0);
-        auto publish_next = [&] { store_x(xbuf ^ 1, xnext, xnext_valid); };
+        auto publish_next = [&] { store_x(has_next ? next : pairs, xnext); };
 
-        layer(IC<0>{}, xbuf * RS_X_BYTES, BUF_A, nothing);
+        layer(IC<0>{}, 0, BUF_P, nothing);
         SP_RS_STAMP(1);
         if constexpr (S == 2) {
-            layer(IC<1>{}, BUF_A, BUF_B, publish_next);
+            layer(IC<1>{}, BUF_P, BUF_Q, publish_next);
             SP_RS_STAMP(2);
         } else {
-            layer(IC<1>{}, BUF_A, BUF_B, nothing);
+            layer(IC<1>{}, BUF_P, BUF_Q, nothing);
             SP_RS_STAMP(2);
-            layer(IC<2>{}, BUF_B, BUF_C, publish_next);
+            layer(IC<2>{}, BUF_Q, BUF_P, publish_next);
         }
         SP_RS_STAMP(3);
 
-        // ---- output layer: rows 16 w4 .. + 15 of the tile (both waves of the pair, each finishes half of the rows);
-        //      MFMA row i is output i ----
-        constexpr int last_in = S == 3 ? BUF_C : BUF_B;
+        // ---- output layer: rows 16 wave .. + 15 of the pair; MFMA row i is output i ----
+        constexpr int last_in = S == 3 ? BUF_P : BUF_Q;
         f32x4 d;
         {
             u32x4 al[8], WL[8];
 #pragma unroll
-            for (int ks = 0; ks < 8; ++ks) al[ks] = read_at(last_in, w4, ks);
+            for (int ks = 0; ks < 8; ++ks) al[ks] = read_at(last_in, wave >> 2, wave & 3, ks);     // (tile wave / 4 of the pair, batch tile wave % 4)
 #pragma unroll
             for (int ks = 0; ks < 8; ++ks) WL[ks] = *reinterpret_cast<const u32x4*>(lds + RS_WL_OFF + ks * 1024 + lane * 16);
+            if constexpr (S == 3) {
+                // the next pair's first layer writes the buffer these reads come from: nobody goes on before everybody
+                // has them
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
             // even and odd k-steps add up separately: two chains of four dependent MFMAs instead of one of eight
             f32x4 dd[2];
 #pragma unroll
@@ -417,6 +419,10 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
             d = dd[0] + dd[1];
         }
         SP_RS_STAMP(4);
+        // (the row numbers are worked out here rather than carried through the layers in registers)
+        const long row0 = (long)pair * RS_PAIR_ROWS;
+        const long head_row_idx = row0 + wave * 16 + j;
+        const bool head_ok = lane < 16 && head_row_idx < batch;
         const float* bias = last_bias;
         const int limit = mask_size > 0 ? mask_size : NOUT;
         if constexpr (PLAIN) {
@@ -429,11 +435,11 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
             if (out.stride > NOUT && (out.stride & 3) == 0) {
                 const int s4 = out.stride >> 2, c0 = (NOUT + 3) >> 2;    // float4 groups per row; the first one that is all zeros
                 fill_end = 4 * c0;
-                const long first_row = row0 + w4 * 16;
+                const long first_row = row0 + wave * 16;
                 float* block = out.policy + first_row * out.stride;
                 for (int idx = lane; idx < 16 * s4; idx += 64) {
                     const int r = idx / s4, c = idx - r * s4;
-                    if (c >= c0 && (r >> 3) == wp && first_row + r < batch)
+                    if (c >= c0 && first_row + r < batch)
                         store16_through(reinterpret_cast<f32x4*>(block + (long)r * out.stride + 4 * c), f32x4{0.f, 0.f, 0.f, 0.f});
                 }
             }
@@ -448,7 +454,7 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
                 if (head_ok) head_row4_any(out.head, out, p, head_row_idx, NOUT, limit, u_row, fill_end);
             } else {
                 // the wave's 16 x NOUT outputs staged in its own KiB of LDS
-                float* head_rows = reinterpret_cast<float*>(lds + RS_HEAD_OFF + w4 * 1024);   // (the pair writes the same values)
+                float* head_rows = reinterpret_cast<float*>(lds + RS_HEAD_OFF + wave * 1024);
                 f32x4 v = d;
                 if (bias != nullptr) {
 #pragma unroll
@@ -465,8 +471,7 @@ __global__ __launch_bounds__(RS_THREADS) void mlp_resident_kernel(const MlpResid
         ++tl_n;
 #endif
         if (!has_next) break;
-        tile = next;
-        xbuf ^= 1;
+        pair = next;
     }
 #undef SP_RS_STAMP
 }
@@ -493,18 +498,18 @@ bool mlp_resident_takes(int n_layers, const int32_t* dims, int nout) {
 // Launches the resident kernel on `a` (every field but `tiles` filled in by the caller, who has checked the stack with
 // mlp_resident_takes): one workgroup per compute unit, fewer when there are fewer tiles.
 int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a, hipStream_t stream, const char* what) {
-    const long tiles = (a.batch + RS_ROWS - 1) / RS_ROWS;
-    if (tiles > 0x7fffffffl - 4096) return fail(SP_ERR_SHAPE, "%s: batch too large", what);
-    a.tiles = (int)tiles;
+    const long pairs = (a.batch + RS_PAIR_ROWS - 1) / RS_PAIR_ROWS;
+    if (pairs > 0x7fffffffl - 4096) return fail(SP_ERR_SHAPE, "%s: batch too large", what);
+    a.tiles = (int)pairs;                                  // the kernel walks pairs of tiles
     const int ks0 = a.k0 <= 32 ? 1 : 2;
     const bool plain = a.nout <= 4 && a.out_stride == a.nout && a.logits == nullptr && a.action != nullptr && a.b[n_layers - 1] == nullptr;
     const void* kernel = dtype == SP_F16 ? (packed ? pick_resident<SP_F16, true>(ks0, n_layers, plain) : pick_resident<SP_F16, false>(ks0, n_layers, plain))
                                          : (packed ? pick_resident<SP_BF16, true>(ks0, n_layers, plain) : pick_resident<SP_BF16, false>(ks0, n_layers, plain));
-    const int lds_bytes = rs_lds_total(ks0);
+    const int lds_bytes = RS_LDS_TOTAL;
     int rc = ensure_dynamic_lds(kernel, lds_bytes);
     if (rc != SP_OK) return rc;
     const long cus = device_cu_count();
-    const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+    const unsigned blocks = (unsigned)(pairs < cus ? pairs : cus);
     void* args[] = {(void*)&a};
     hipError_t e = hipLaunchKernel(kernel, dim3(blocks), dim3(RS_THREADS), args, lds_bytes, stream);
     if (e != hipSuccess) return fail(SP_ERR_DEVICE, "%s: launch failed: %s", what, hipGetErrorString(e));

@@ -302,17 +302,17 @@ def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed,
 
 
 @pytest.mark.parametrize("dims,head,mask,batch,dtype,with_bias,packed", [
-    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 70000, "f16", False, True),    # the benchmark's network, ragged last tile
-    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 70000, "f16", False, False),   # ... from the row-major weights
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 100000, "f16", False, True),   # the benchmark's network, ragged last pair
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 133000, "f16", False, False),  # ... from the row-major weights
     ([32, 256, 256, 256, 3], "softmax", 0, 300000, "bf16", "all", True),                  # 18 tiles per compute unit
-    ([16, 256, 256, 4], "softmax_regret_matching", 0, 66000, "f16", True, False),         # three layers, a 16-wide first layer
-    ([48, 256, 256, 256, 16], "softmax", 0, 66000, "bf16", True, False),                  # two first-layer k-steps, K0 not a multiple of 32, 16 outputs
-    ([64, 256, 256, 12], "softmax", 7, 40000, "f16", "only1", True),                      # masked head with logits, head staged in LDS
-    ([32, 256, 256, 256, 2], "softmax_regret_matching", 0, 32768 + 5, "bf16", False, True),
+    ([16, 256, 256, 4], "softmax_regret_matching", 0, 132000, "f16", True, False),        # three layers, a 16-wide first layer
+    ([48, 256, 256, 256, 16], "softmax", 0, 131100, "bf16", True, False),                 # two first-layer k-steps, K0 not a multiple of 32, 16 outputs
+    ([64, 256, 256, 12], "softmax", 7, 98400, "f16", "only1", True),                      # masked head with logits, head staged in LDS
+    ([32, 256, 256, 256, 2], "softmax_regret_matching", 0, 98304 + 65, "bf16", False, True),   # one row in the second tile of the last pair
 ])
 def test_weights_resident_in_registers(LY, dims, head, mask, batch, dtype, with_bias, packed):
     """Batches of several 64-row tiles per compute unit run on the kernel that loads the weights once and keeps them in
-    registers while it walks over its tiles (from two tiles per unit with packed weights, from four with row-major
+    registers while it walks over its tiles (from six tiles per unit with packed weights, from eight with row-major
     ones): against the oracle like every other kernel, and bit for bit against the per-tile packed kernel run on the
     same rows in slices small enough to stay on that kernel (same operand layout, same order of the sums)."""
     announce("mlp resident %s head=%s mask=%d batch=%d %s bias=%s packed=%s" % (dims, head, mask, batch, dtype, with_bias, packed))
@@ -343,11 +343,11 @@ def test_resident_kernel_run_to_run_and_philox(LY):
     from ml import _lib, primitives
     announce("mlp resident run-to-run + philox")
     rng = np.random.default_rng(41)
-    batch, dims = 24 * 4096, [32, 256, 256, 256, 64]
+    batch, dims = 24 * 5632, [32, 256, 256, 256, 64]
     x, ws, _ = make_problem(rng, batch, dims, "f16")
     xd, wd = dev(x, torch.float16), [dev(w, torch.float16) for w in ws]
     pk = LY.pack_weights(wd)
-    cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=24, rows_per_block=4096)
+    cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=24, rows_per_block=5632)
     u = primitives.philox_uniforms(cfg, batch, 64)
     for packed in (pk, None):
         first = [t.clone() for t in LY.mlp_forward(xd, wd, None, "softmax", u, 3, packed=packed)]
