@@ -9,6 +9,8 @@ A "step" is one launch of that GEMM.  The same line carries, under "extra", the 
 configurations (f32 1024^3, f16 / 8192^3, tall-skinny value-net GEMMs, the fused Leduc MLP
 forward in rows/s, the row primitives in GB/s), each with its own roofline fraction, and under
 "cpu_baseline" the NumPy restatement timed on this box's host cores in the same run.
+Every timed case is checked against the oracle after its timed loop, and the compute units' clock during the loop is
+reported next to it (`shader_clock_mhz`; the matrix-pipe peak is quoted at 2400 MHz, power-limited kernels run below).
 """
 import argparse
 import json
@@ -59,7 +61,7 @@ def time_launches(fn, steps, warmup):
     ratio is the clock the units ran at during the loop, left in CLOCK["mhz"]."""
     import torch
     from ml._lib import check, lib, stream_ptr
-    samples = torch.zeros(4, dtype=torch.int64, device="cuda")
+    samples = torch.zeros(2 * 128, dtype=torch.int64, device="cuda")
     t_end = time.perf_counter() + PREWARM_MS * 1e-3
     while time.perf_counter() < t_end:
         for _ in range(20):
@@ -74,13 +76,25 @@ def time_launches(fn, steps, warmup):
     check(lib.sp_clock_sample(samples.data_ptr(), stream_ptr()))
     for _ in range(steps):
         fn()
-    check(lib.sp_clock_sample(samples.data_ptr() + 16, stream_ptr()))
+    check(lib.sp_clock_sample(samples.data_ptr() + 1024, stream_ptr()))
     stop.record()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    c0, r0, c1, r1 = (int(v) for v in samples.cpu())
-    CLOCK["mhz"] = round((c1 - c0) / max(1, r1 - r0) * 100.0, 1)
+    CLOCK["mhz"] = clock_mhz(samples.cpu().numpy().reshape(2, 32, 4))
     return wall, start.elapsed_time(stop) / steps
+
+
+def clock_mhz(samples):
+    """Median over the XCDs of (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz from two sp_clock_sample results
+    (each 32 x [xcd, cycles, 100 MHz ticks, valid])."""
+    per_xcd = []
+    for xcd in range(16):
+        first = [r for r in samples[0] if r[3] == 1 and r[0] == xcd]
+        last = [r for r in samples[1] if r[3] == 1 and r[0] == xcd]
+        if first and last and last[0][2] > first[0][2]:
+            per_xcd.append((int(last[0][1]) - int(first[0][1])) / (int(last[0][2]) - int(first[0][2])) * 100.0)
+    per_xcd.sort()
+    return round(per_xcd[len(per_xcd) // 2], 1) if per_xcd else None
 
 
 NOMINAL_MHZ = 2400.0     # the clock the published peak rates are quoted at
@@ -191,7 +205,7 @@ def main():
         if roof["bound"] == "mfma":
             # the published peak assumes the nominal clock; a power-limited kernel runs below it, and this is the
             # fraction of what the matrix pipes could do at the clock they were actually given
-            roof["frac_at_measured_clock"] = round(roof["frac"] * NOMINAL_MHZ / mhz, 4) if mhz > 0 else None
+            roof["frac_at_measured_clock"] = round(roof["frac"] * NOMINAL_MHZ / mhz, 4) if mhz else None
         res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "tflops": round(flops / (wall * 1e-3) / 1e12, 2),
                "gbs": round(nbytes / (wall * 1e-3) / 1e9, 1), "roofline": roof, "seed": seed, "shader_clock_mhz": mhz,
                "checked_rel_frobenius": float("%.3g" % err),
@@ -208,7 +222,7 @@ def main():
     # ---------------- headline: bf16 4096^3, f32 accumulate, f32 out ----------------
     flops = 2.0 * 4096 ** 3
     if args.only:   # profiling aid: only the named extra case runs, the headline fields stay empty
-        head, a, b = {"tflops": None, "wall_ms": None, "roofline": None, "tile": None}, None, None
+        head, a, b = {"tflops": None, "wall_ms": None, "roofline": None, "tile": None, "shader_clock_mhz": None}, None, None
     else:
         head, (a, b) = gemm_case(2, 4096, 4096, 4096, "bf16")
 
@@ -359,7 +373,8 @@ def main():
                 fn = lambda: primitives.transpose_snd(xd, out=out)
                 nbytes = 2 * x.nbytes
             wall, ev = time_launches(fn, K, W)
-            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "roofline": roofline_hbm(nbytes, ev), "seed": 9}
+            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "roofline": roofline_hbm(nbytes, ev), "seed": 9,
+                    "shader_clock_mhz": CLOCK["mhz"]}
 
         def graph_case():
             # The same policy step through the reference's host surface: a layer graph (input -> matmul/relu x3 ->
@@ -407,23 +422,45 @@ def main():
     except Exception as e:  # the device query is informational only
         info = {"error": str(e)}
 
-    # HBM-side traffic of the headline kernel, measured separately with rocprofv3 --pmc (the counters
-    # cannot be read from inside this process); profiles/traffic.json holds the scaled figure
+    # HBM-side traffic per launch, measured separately with rocprofv3 --pmc (the counters cannot be read from inside
+    # this process); profiles/traffic.json holds the scaled figures together with a hash of the kernel source each
+    # was measured on.  A figure is only copied into the line while that source is unchanged: after an edit it is
+    # stale until the counters have been collected again, and the line says so instead.
     try:
+        import hashlib
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
             measured = json.load(f)
-        if head["roofline"] is not None:
-            head["roofline"]["traffic"] = measured["headline"]["traffic_bytes"]
-            head["roofline"]["traffic_measured_at"] = measured.get("measured_at")
-        for name, res in extra.items():
+
+        def source_hash(src):
+            """sha256 over a kernel source and the headers of its directory, in name order."""
+            csrc = os.path.join(ROOT, "spiral-s-ml-library_amd", "csrc")
+            h = hashlib.sha256()
+            for name in [src] + sorted(n for n in os.listdir(csrc) if n.endswith(".h")):
+                with open(os.path.join(csrc, name), "rb") as fh:
+                    h.update(fh.read())
+            return h.hexdigest()
+
+        def source_unchanged(entry):
+            src = entry.get("source")
+            return bool(src) and source_hash(src) == measured.get("source_sha256", {}).get(src)
+
+        for name, res in [("headline", head)] + list(extra.items()):
             if name in measured and res.get("roofline") is not None:
-                res["roofline"]["traffic"] = measured[name]["traffic_bytes"]
+                if source_unchanged(measured[name]):
+                    res["roofline"]["traffic"] = measured[name]["traffic_bytes"]
+                else:
+                    res["roofline"]["traffic_stale"] = "%s changed since profiles/traffic.json was measured" % measured[name].get("source")
     except (OSError, KeyError, ValueError):
         pass
 
-    # `value` and `ms_per_step` come from the same clock (wall time between two device syncs around the K
-    # launches): value = 2 * 4096^3 / ms_per_step.  `roofline.achieved` is the kernel's own rate, from HIP events
-    # on the launch stream (`event_ms_per_step`); the two differ by the host's share of a launch.
+    # `value`, `ms_per_step` and `roofline` come from the same clock (wall time between two device syncs around the
+    # K launches): value = roofline.achieved = 2 * 4096^3 / ms_per_step.  `event_ms_per_step` is the same interval
+    # between two HIP events on the launch stream; the two differ by the host's share of a launch.
+    # `mlp_rows_per_s` is the drop-in call (row-major weights, sp_mlp_forward) in the one-launch-over-many-batches
+    # timing mode; the other three combinations of weights and timing mode stand next to it.
+    mlp = {k: extra.get(k, {}).get("rows_per_s") for k in ("mlp_leduc_16384", "mlp_leduc_16384_rowmajor",
+                                                           "mlp_leduc_16384x64_one_launch",
+                                                           "mlp_leduc_16384x64_one_launch_rowmajor")}
     line = {
         "metric": "GEMM TFLOP/s (% MFMA peak) at 4096^3 bf16; fused MLP fwd rows/sec",
         "value": None if head["wall_ms"] is None else round(flops / (head["wall_ms"] * 1e-3) / 1e12, 2),
@@ -434,7 +471,13 @@ def main():
         "config": {"workload": "C = A.B^T, M=N=K=4096, A/B bf16 row-major N(0,1)/sqrt(K) (seed 2), f32 accumulate, "
                                "f32 output", "tile": head["tile"]},
         "roofline": head["roofline"], "cpu_baseline": cpu,
-        "mlp_rows_per_s": extra.get("mlp_leduc_16384", {}).get("rows_per_s"),
+        "shader_clock_mhz": head.get("shader_clock_mhz"),
+        "mlp_rows_per_s": mlp["mlp_leduc_16384x64_one_launch_rowmajor"],
+        "mlp_rows_per_s_detail": {
+            "row_major_weights_one_launch_over_64_batches": mlp["mlp_leduc_16384x64_one_launch_rowmajor"],
+            "packed_weights_one_launch_over_64_batches": mlp["mlp_leduc_16384x64_one_launch"],
+            "row_major_weights_one_launch_per_batch": mlp["mlp_leduc_16384_rowmajor"],
+            "packed_weights_one_launch_per_batch": mlp["mlp_leduc_16384"]},
         "extra": extra, "device": info,
     }
     print(json.dumps(line))

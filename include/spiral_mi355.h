@@ -76,11 +76,12 @@ typedef struct {
 } sp_kernel_info_t;
 int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
 
-/* Measurement aid: out[0] = the compute units' cycle counter, out[1] = the constant 100 MHz counter, both read by
- * one wave at the point of `stream` where the call is enqueued.  Two samples around a stretch of work give the clock
- * the units actually ran at during it: (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz -- on power-limited kernels
- * well below the nominal 2.4 GHz that the published peak rates assume.  `out` is device memory (16 bytes).  Stands
- * beside the host-side device probing of corecuda/base.spi:73; the reference has no counterpart. */
+/* Measurement aid: 32 workgroups each write four 64-bit words to `out` (device memory, 1 KiB): the number of the XCD
+ * they ran on, that XCD's cycle counter, the constant 100 MHz counter, and 1 -- read at the point of `stream` where
+ * the call is enqueued.  Two samples around a stretch of work give the clock the compute units ran at during it:
+ * per XCD, (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz (the cycle counters of different XCDs are not in step,
+ * so samples are paired by XCD number).  Power-limited kernels run well below the nominal 2.4 GHz.  Stands beside the
+ * host-side device probing of corecuda/base.spi:73; the reference has no counterpart. */
 int sp_clock_sample(uint64_t* out, void* stream);
 
 /* ------------------------------------------------------------------------------------------ */

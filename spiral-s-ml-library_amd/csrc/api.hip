@@ -93,15 +93,20 @@ static std::vector<KernelEntry>& registry() {
 
 void register_kernel(const char* name, const void* fn, int threads) { registry().push_back({name, fn, threads}); }
 
-// One wave writes the shader clock counter (s_memtime: counts the cycles the compute units run at, so it slows
-// down with the clock) and the constant 100 MHz counter (s_memrealtime) side by side.  A single workgroup always
-// lands on the same XCD, so two samples read the same pair of counters.
+// Every workgroup writes the number of the XCD it runs on, that XCD's shader clock counter (s_memtime: counts the
+// cycles the compute units run at, so it slows down with the clock) and the constant 100 MHz counter (s_memrealtime).
+// The cycle counters of different XCDs are not in step, so two samples are only compared XCD by XCD; 32 workgroups
+// land on all eight.
+constexpr int CLOCK_SAMPLE_GROUPS = 32;
 __global__ void clock_sample_kernel(unsigned long long* out) {
     if (threadIdx.x == 0) {
         const unsigned long long cycles = __builtin_amdgcn_s_memtime();
         const unsigned long long ticks = __builtin_amdgcn_s_memrealtime();
-        out[0] = cycles;
-        out[1] = ticks;
+        const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 0xfu;   // HW_REG_XCC_ID, bits 3:0
+        out[blockIdx.x * 4 + 0] = xcc;
+        out[blockIdx.x * 4 + 1] = cycles;
+        out[blockIdx.x * 4 + 2] = ticks;
+        out[blockIdx.x * 4 + 3] = 1;
     }
 }
 
@@ -113,7 +118,7 @@ extern "C" int sp_clock_sample(uint64_t* out, void* stream) {
     SP_REQUIRE_PTR(out);
     int rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
-    hipLaunchKernelGGL(clock_sample_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
+    hipLaunchKernelGGL(clock_sample_kernel, dim3(CLOCK_SAMPLE_GROUPS), dim3(64), 0, (hipStream_t)stream, (unsigned long long*)out);
     return check_launch(__func__);
 }
 

@@ -59,6 +59,10 @@ struct MlpResidentArgs {
 
 bool mlp_resident_takes(int n_layers, const int32_t* dims, int nout);
 int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a, hipStream_t stream, const char* what);
+// The same for four-layer stacks with at most 4 computed outputs: the two 256 x 256 layers as a two-stage pipeline on
+// the two waves of every SIMD (mlp_pipe.hip).  mlp_resident_launch hands such stacks on to it.
+bool mlp_pipe_takes(int n_layers, const int32_t* dims, int nout);
+int mlp_pipe_launch(int dtype, bool packed, MlpResidentArgs a, hipStream_t stream, const char* what);
 // 64-row tiles per compute unit from which the resident kernel is used: its one-time load of all weights has to pay,
 // and it walks tiles in pairs, so few tiles per unit leave units idle in the last round.  Measured against the
 // per-tile kernels (32 -> 256 -> 256 -> 256 -> 3, us per launch, per-tile / resident): packed weights 65536 rows
@@ -69,6 +73,14 @@ int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a,
 #endif
 #ifndef SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR
 #define SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR 8
+#endif
+
+// 64-row tiles per compute unit from which the pipelined kernel takes over from the resident one (for the stacks it
+// takes).  Measured, us per launch, resident / pipelined, packed weights: 98304 rows 26.1 / 24.6, 131072 33.0 / 30.7,
+// 262144 61.4 / 55.9, 524288 118.2 / 106.6, 1048576 230.2 / 207.4; row-major weights 131072 38.7 / 35.6, 262144
+// 67.2 / 61.4, 1048576 240.5 / 212.1: it wins wherever the resident kernel is used at all.
+#ifndef SP_MLP_PIPE_MIN_TILES
+#define SP_MLP_PIPE_MIN_TILES 0
 #endif
 
 // The Philox stream of a head that draws its own uniforms: the sampling node of the layer graph works on rows of

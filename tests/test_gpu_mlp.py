@@ -309,12 +309,16 @@ def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed,
     ([48, 256, 256, 256, 16], "softmax", 0, 131100, "bf16", True, False),                 # two first-layer k-steps, K0 not a multiple of 32, 16 outputs
     ([64, 256, 256, 12], "softmax", 7, 98400, "f16", "only1", True),                      # masked head with logits, head staged in LDS
     ([32, 256, 256, 256, 2], "softmax_regret_matching", 0, 98304 + 65, "bf16", False, True),   # one row in the second tile of the last pair
+    ([64, 256, 256, 256, 4], "softmax_regret_matching", 0, 131072 + 31, "f16", "all", False),  # pipelined form: two first-layer k-steps, every bias, row-major
+    ([48, 256, 256, 256, 8], "softmax", 3, 99000, "bf16", True, True),                          # pipelined form: 3 of 8 columns valid, zeros behind them
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 98304 + 32 * 256 * 9 + 5, "f16", False, True),  # a last head pass of one tile on some units
 ])
 def test_weights_resident_in_registers(LY, dims, head, mask, batch, dtype, with_bias, packed):
     """Batches of several 64-row tiles per compute unit run on the kernel that loads the weights once and keeps them in
     registers while it walks over its tiles (from six tiles per unit with packed weights, from eight with row-major
-    ones): against the oracle like every other kernel, and bit for bit against the per-tile packed kernel run on the
-    same rows in slices small enough to stay on that kernel (same operand layout, same order of the sums)."""
+    ones): against the oracle like every other kernel, and against the per-tile packed kernel run on the same rows in
+    slices small enough to stay on that kernel (same operand layout; the same order of the sums except in the output
+    layer of the pipelined form)."""
     announce("mlp resident %s head=%s mask=%d batch=%d %s bias=%s packed=%s" % (dims, head, mask, batch, dtype, with_bias, packed))
     rng = np.random.default_rng(sum(dims) + batch + 7)
     x, ws, u = make_problem(rng, batch, dims, dtype)
@@ -330,11 +334,26 @@ def test_weights_resident_in_registers(LY, dims, head, mask, batch, dtype, with_
     wd = [dev(w, t) for w in ws]
     bd = None if biases is None else [dev(b) if b is not None else None for b in biases]
     pk = LY.pack_weights(wd)
+    # four-layer stacks with at most 4 outputs take the pipelined form, whose output layer adds its k-steps slice by
+    # slice: equal to the per-tile kernel to rounding; the others add in the per-tile kernel's order: equal bit for bit
+    pipelined = len(dims) == 5 and (mask or dims[-1]) <= 4
+    # the call that asks for no logits is another instance of the kernel: the same bits -- unless only that call can
+    # leave the masked columns out of the output layer and so comes to run on the pipelined form
+    p, a = LY.mlp_forward(dev(x, t), wd, bd, head, dev(u), mask, packed=pk if packed else None)
+    if pipelined and mask:
+        assert ogemm.rel_frobenius(policy, host(p)) < 2e-5 and (host(a) != action).mean() < 1e-3
+        assert (host(a) == orow.discrete_sampling(host(p), u)).all() and (host(p)[:, mask:] == 0).all()
+    else:
+        assert (host(p) == policy).all() and (host(a) == action).all()
     step = 16384
     for lo in range(0, batch, step):
         hi = min(batch, lo + step)
         p, a = LY.mlp_forward(dev(x[lo:hi], t), None, bd, head, dev(u[lo:hi]), mask, packed=pk)
-        assert (host(p) == policy[lo:hi]).all() and (host(a) == action[lo:hi]).all(), lo
+        if pipelined:
+            assert ogemm.rel_frobenius(policy[lo:hi], host(p)) < 2e-5, lo
+            assert (host(a) != action[lo:hi]).mean() < 1e-3, lo
+        else:
+            assert (host(p) == policy[lo:hi]).all() and (host(a) == action[lo:hi]).all(), lo
 
 
 def test_resident_kernel_run_to_run_and_philox(LY):
