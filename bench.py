@@ -61,7 +61,7 @@ def time_launches(fn, steps, warmup):
     ratio is the clock the units ran at during the loop, left in CLOCK["mhz"]."""
     import torch
     from ml._lib import check, lib, stream_ptr
-    samples = torch.zeros(2 * 128, dtype=torch.int64, device="cuda")
+    samples = torch.zeros(2 * CLOCK_SLOTS * 2, dtype=torch.int64, device="cuda")
     t_end = time.perf_counter() + PREWARM_MS * 1e-3
     while time.perf_counter() < t_end:
         for _ in range(20):
@@ -71,30 +71,32 @@ def time_launches(fn, steps, warmup):
         fn()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    check(lib.sp_clock_sample(samples.data_ptr(), stream_ptr()))
     t0 = time.perf_counter()
     start.record()           # torch's current stream == the stream the library launches on
-    check(lib.sp_clock_sample(samples.data_ptr(), stream_ptr()))
     for _ in range(steps):
         fn()
-    check(lib.sp_clock_sample(samples.data_ptr() + 1024, stream_ptr()))
     stop.record()
+    check(lib.sp_clock_sample(samples.data_ptr() + CLOCK_SLOTS * 16, stream_ptr()))
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) * 1e3 / steps
-    CLOCK["mhz"] = clock_mhz(samples.cpu().numpy().reshape(2, 32, 4))
+    CLOCK["mhz"] = clock_mhz(samples.cpu().numpy().reshape(2, CLOCK_SLOTS, 2))
     return wall, start.elapsed_time(stop) / steps
 
 
+CLOCK_SLOTS = 32768      # slots of one sp_clock_sample result: (cycles, 100 MHz ticks) per SIMD of the chip
+
+
 def clock_mhz(samples):
-    """Median over the XCDs of (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz from two sp_clock_sample results
-    (each 32 x [xcd, cycles, 100 MHz ticks, valid])."""
-    per_xcd = []
-    for xcd in range(16):
-        first = [r for r in samples[0] if r[3] == 1 and r[0] == xcd]
-        last = [r for r in samples[1] if r[3] == 1 and r[0] == xcd]
-        if first and last and last[0][2] > first[0][2]:
-            per_xcd.append((int(last[0][1]) - int(first[0][1])) / (int(last[0][2]) - int(first[0][2])) * 100.0)
-    per_xcd.sort()
-    return round(per_xcd[len(per_xcd) // 2], 1) if per_xcd else None
+    """Median over the SIMDs sampled both times of (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz from two
+    sp_clock_sample results (every compute unit's cycle counter runs from a start of its own: slot by slot)."""
+    import numpy as np
+    first, last = samples[0].astype(np.int64), samples[1].astype(np.int64)
+    both = (first[:, 1] != 0) & (last[:, 1] > first[:, 1])
+    if not both.any():
+        return None
+    mhz = (last[both, 0] - first[both, 0]) / (last[both, 1] - first[both, 1]) * 100.0
+    return round(float(np.median(mhz)), 1)
 
 
 NOMINAL_MHZ = 2400.0     # the clock the published peak rates are quoted at
@@ -401,6 +403,48 @@ def main():
                               "on weights packed once when the plan is built; every run draws its own Philox uniforms "
                               "inside the kernel (nothing is carried over from run to run but the packed weights)"}
 
+        def ensemble_case():
+            # The reference's own policy network (game/leduc/model_cem.spi:55-63) through its host surface: a layer
+            # graph of E = 32 members, 128 -> 64 -> relu -> 64, masked regret matching over 3 of 64 columns, f32, on
+            # blocks_per_grid x 256 rows; graph_run_host(model, {"ensemble": 32}) is ONE fused launch.
+            ens, q, w = 32, layers.blocks_per_grid(), 256
+            probs = layers.apply("ensemble", layers.input("output_probs", (ens, q, w, 64)))
+            net = layers.pipe(layers.input("input", (q, w, 128)), layers.matmul_ensemble_with_adjoint((ens, 128, 64)),
+                              layers.relu, layers.matmul_ensemble_with_adjoint((ens, 64, 64)))
+            m = layers.create_model(layers.masked_regret_matching_(3, probs, net))
+            rng = np.random.default_rng(11)
+            xin = layers.key_extract(m, "input")
+            x = rng.standard_normal(tuple(xin.shape), dtype=np.float32)
+            xin.copy_(dev(x))
+            ws = []
+            for t in layers.key_extract_list(m, "weights"):
+                ws.append(rng.standard_normal(tuple(t.shape), dtype=np.float32) * np.float32(0.1))
+                t.copy_(dev(ws[-1]))
+            rows = q * w
+            fn = lambda: layers.graph_run_host(m, {"ensemble": ens})
+            wall, ev = time_launches(fn, max(K // 2, 20), W)
+            mhz = CLOCK["mhz"]
+            got = layers.key_extract(m, "output_probs").cpu().numpy().reshape(ens, rows, 64)
+            sample = slice(0, rows, max(1, rows // 512))
+            for e in (0, ens - 1):                                # what was timed is checked: two members, 512 rows each
+                want, _, _ = olayers.mlp_forward(x.reshape(rows, 128)[sample], [ws[0][e], ws[1][e]], None,
+                                                 olayers.HEAD_REGRET_MATCHING, None, None, 3)
+                assert ogemm.rel_frobenius(got[e][sample], want) < 1e-5, "bench ensemble output drifted from the oracle"
+            slow = lambda: layers.graph_run_host(m, {"ensemble": ens}, fuse=False)
+            _, ev_nodes = time_launches(slow, max(K // 10, 5), 2)
+            # flops the masked graph needs: the second layer only for the 3 columns the mask keeps (the reference's
+            # node-by-node pass multiplies all 64 and masks afterwards: 2 * (128 * 64 + 64 * 64) per member-row)
+            fl = 2.0 * rows * ens * (128 * 64 + 64 * 3)
+            roof = roofline_mfma(fl, ev, "f32")
+            roof["frac_counting_all_64_columns"] = round(2.0 * rows * ens * (128 * 64 + 64 * 64) / (ev * 1e-3) / 1e12 / PEAK_TFLOPS["f32"], 4)
+            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(rows * ens / (ev * 1e-3), 1),
+                    "roofline": roof, "seed": 11, "shader_clock_mhz": mhz,
+                    "rows": rows, "members": ens, "node_by_node_ms": round(ev_nodes, 5),
+                    "timing": "mean over back-to-back graph_run_host(model, {ensemble: 32}) calls, one sp_mlp_forward_ensemble "
+                              "launch each; node_by_node_ms: the same graph with fuse=False (batched GEMM, relu map, "
+                              "batched GEMM, row map: four launches); rows_per_s counts member-rows"}
+
+        cases += [("ensemble_leduc_policy_e32", ensemble_case)]
         cases += [("mlp_leduc_16384", mlp_case), ("mlp_leduc_16384_rowmajor", lambda: mlp_case(False)),
                   ("mlp_leduc_16384x64_one_launch", lambda: mlp_case(True, 64)),
                   ("mlp_leduc_16384x64_one_launch_rowmajor", lambda: mlp_case(False, 64)),
@@ -414,6 +458,15 @@ def main():
             continue
         extra[name] = fn()
         torch.cuda.empty_cache()
+
+    # The MLP's two timing modes side by side: `ms` of a one-launch-per-batch case is the launch-to-launch interval of
+    # back-to-back launches; `kernel_ms` is the time per 16384-row batch inside ONE launch over 64 batches, which no
+    # launch effect can touch (that launch takes the kernels of the family that keep the weights in registers).
+    for single, many in (("mlp_leduc_16384", "mlp_leduc_16384x64_one_launch"),
+                         ("mlp_leduc_16384_rowmajor", "mlp_leduc_16384x64_one_launch_rowmajor")):
+        if single in extra and many in extra:
+            extra[single]["kernel_ms"] = extra[many]["ms"]
+            extra[single]["kernel_ms_from"] = many
 
     info = None
     try:

@@ -76,12 +76,14 @@ typedef struct {
 } sp_kernel_info_t;
 int sp_kernel_info(const char* kernel_family, sp_kernel_info_t* out);
 
-/* Measurement aid: 32 workgroups each write four 64-bit words to `out` (device memory, 1 KiB): the number of the XCD
- * they ran on, that XCD's cycle counter, the constant 100 MHz counter, and 1 -- read at the point of `stream` where
- * the call is enqueued.  Two samples around a stretch of work give the clock the compute units ran at during it:
- * per XCD, (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz (the cycle counters of different XCDs are not in step,
- * so samples are paired by XCD number).  Power-limited kernels run well below the nominal 2.4 GHz.  Stands beside the
- * host-side device probing of corecuda/base.spi:73; the reference has no counterpart. */
+/* Measurement aid: `out` (device memory, 32768 slots of two 64-bit words = 512 KiB, zeroed by the caller) receives,
+ * in the slot of every SIMD a workgroup of the sampling kernel ran on (slot = XCD number * 4096 + bits 15:4 of the
+ * hardware id: shader engine, shader array, compute unit, SIMD), that unit's cycle counter and the constant 100 MHz
+ * counter, read at the point of `stream` where the call is enqueued; slots of places the kernel did not reach stay
+ * zero.  Two samples around a stretch of work give the clock the compute units ran at during it: per slot filled in
+ * both, (cycles1 - cycles0) / (ticks1 - ticks0) * 100 MHz (every unit's cycle counter runs from a start of its own,
+ * so samples are only compared slot by slot).  Power-limited kernels run well below the nominal 2.4 GHz.  Stands
+ * beside the host-side device probing of corecuda/base.spi:73; the reference has no counterpart. */
 int sp_clock_sample(uint64_t* out, void* stream);
 
 /* ------------------------------------------------------------------------------------------ */
@@ -407,6 +409,22 @@ int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void
                           const float* const* biases, const int32_t* dims, const float* u, const sp_philox_t* philox,
                           float* policy_out, int32_t* action_out, float* logits_out, int64_t batch, int32_t head,
                           int32_t mask_size, void* stream);
+
+/* Fused forward of an ENSEMBLE of two-layer f32 stacks on one shared input, one launch:
+ *   policy[e] = head(relu(x . W1[e]^T) . W2[e]^T),  e = 0 .. members - 1
+ * x: (batch, dims[0]) f32; weights[0]: (members, dims[1], dims[0]), weights[1]: (members, dims[2], dims[1]) f32,
+ * the stacked tensors of `matmul_ensemble` (ml/layers.spi:468-479); dims[0] a multiple of 8 in [8, 128], dims[1] = 64,
+ * dims[2] <= 64; n_layers = 2; dtype = SP_F32.  head / mask_size as for sp_mlp_forward, with at most 4 computed
+ * outputs (dims[2], or mask_size of a masked head; the columns behind the mask are written as zeros).
+ * policy_out: (members, batch, dims[2]); action_out: (members, batch) or NULL; u: (members, batch) uniforms in
+ * (0, 1] or NULL; philox: a stream over the members x batch stacked rows (member_rows = batch) or NULL; at most one
+ * of u and philox, one of them when action_out is given.
+ * Replaces: `graph_run_host model {ensemble}` (ml/layers.spi:336-344, the interpreter of :194-240 run member by
+ * member) for the graph of the reference's Leduc policy, game/leduc/model_cem.spi:55-63
+ * (input -> matmul_ensemble_with_adjoint -> relu -> matmul_ensemble_with_adjoint -> masked_regret_matching'). */
+int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layers, const void* const* weights, const int32_t* dims,
+                            int32_t members, const float* u, const sp_philox_t* philox, float* policy_out,
+                            int32_t* action_out, int64_t batch, int32_t head, int32_t mask_size, void* stream);
 
 #ifdef __cplusplus
 }

@@ -17,9 +17,9 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libspiral_mi355.so")
-SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip", "mlp_resident.hip", "mlp_pipe.hip"]
+SOURCES = ["api.hip", "row_ops.hip", "elementwise.hip", "gemm.hip", "mlp.hip", "mlp_packed.hip", "mlp_resident.hip", "mlp_pipe.hip", "mlp_ensemble.hip"]
 # sources with MFMAs or wide stores in inline asm: their device assembly is kept and scanned (isa_check.py)
-ASM_MFMA_SOURCES = ["gemm.hip", "mlp.hip", "mlp_packed.hip", "mlp_resident.hip", "mlp_pipe.hip", "row_ops.hip", "elementwise.hip"]
+ASM_MFMA_SOURCES = ["gemm.hip", "mlp.hip", "mlp_packed.hip", "mlp_resident.hip", "mlp_pipe.hip", "mlp_ensemble.hip", "row_ops.hip", "elementwise.hip"]
 # Kernel-argument preloading (gfx950): the first 14 dwords of a kernel's leading scalar parameters arrive in
 # registers with the wave instead of through a scalar load at kernel entry (a struct parameter is not preloaded;
 # the kernels that gain from it repeat the fields their first loads need as leading scalars).

@@ -95,18 +95,21 @@ void register_kernel(const char* name, const void* fn, int threads) { registry()
 
 // Every workgroup writes the number of the XCD it runs on, that XCD's shader clock counter (s_memtime: counts the
 // cycles the compute units run at, so it slows down with the clock) and the constant 100 MHz counter (s_memrealtime).
-// The cycle counters of different XCDs are not in step, so two samples are only compared XCD by XCD; 32 workgroups
-// land on all eight.
-constexpr int CLOCK_SAMPLE_GROUPS = 32;
+// Every compute unit keeps a cycle counter of its own, and they are not in step (tens of millions of cycles apart even
+// inside one XCD), so two samples can only be compared unit by unit: a workgroup writes its pair of counters into the
+// slot of the unit it ran on -- XCD number and the unit's place in it (shader engine, shader array, unit, SIMD: bits
+// 15:4 of the hardware id) -- and 8192 one-wave workgroups reach every SIMD of the chip.
+constexpr int CLOCK_SAMPLE_GROUPS = 8192;
+constexpr int CLOCK_SAMPLE_SLOTS = 8 * 4096;
 __global__ void clock_sample_kernel(unsigned long long* out) {
     if (threadIdx.x == 0) {
         const unsigned long long cycles = __builtin_amdgcn_s_memtime();
         const unsigned long long ticks = __builtin_amdgcn_s_memrealtime();
-        const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 0xfu;   // HW_REG_XCC_ID, bits 3:0
-        out[blockIdx.x * 4 + 0] = xcc;
-        out[blockIdx.x * 4 + 1] = cycles;
-        out[blockIdx.x * 4 + 2] = ticks;
-        out[blockIdx.x * 4 + 3] = 1;
+        const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11)) & 0x7u;   // HW_REG_XCC_ID, bits 3:0
+        const unsigned hw = __builtin_amdgcn_s_getreg(4 | (4 << 6) | (11 << 11));          // HW_REG_HW_ID, bits 15:4
+        typedef unsigned long long u64x2 __attribute__((ext_vector_type(2)));
+        const u64x2 rec = {cycles, ticks};
+        *reinterpret_cast<u64x2*>(out + 2 * (xcc * 4096 + (hw & 0xfffu))) = rec;              // one 16-byte store
     }
 }
 

@@ -1,0 +1,286 @@
+// Fused forward of an ENSEMBLE of small f32 stacks on one shared input: member e of E computes
+//     policy[e] = head(relu(x . W1[e]^T) . W2[e]^T)          x: (batch, K0), W1: (E, 64, K0), W2: (E, N, 64), all f32
+// in one launch, activations never leaving registers.  This is the graph of the reference's Leduc policy
+// (game/leduc/model_cem.spi:55-63: input -> matmul_ensemble_with_adjoint (E, 128, 64) -> relu ->
+// matmul_ensemble_with_adjoint (E, 64, 64) -> masked_regret_matching' 3), which the graph interpreter
+// (ml/layers.spi:194-240, 336-344) runs member by member, node by node.
+//
+// One wave per SIMD (four per workgroup, nothing shared between them: no LDS, no barrier).  A wave loads the weights
+// of its member once -- 128 registers for the first layer, 32 per computed output for the second -- and walks over
+// 32-row tiles of the batch.
+//   Layer 1 is v_mfma_f32_32x32x2_f32 with the WEIGHTS as the row operand, so a result tile is (features x batch rows)
+// and lane (r, g) -- r = lane % 32 the batch row, g = lane / 32 -- holds features 8 a + 4 g + b (a, b = 0..3) of row
+// r in register 4 a + b.  Both operands of an MFMA step take their two K-values from the lane halves g = 0, 1, and
+// WHICH K-index a (step, half) pair stands for is free as long as both operands agree: step 4 j + i, half g stands
+// for k = 8 j + 4 g + i, so every lane's inputs and weights are 16-byte loads.
+//   Layer 2 is computed for at most 4 outputs (a masked head's valid columns, or a head that narrow), which is too
+// little for the matrix pipe (a 32 x 32 tile for 3 useful rows costs a quarter of layer 1): every lane multiplies the
+// 32 features of its row that it holds (after the relu) with the matching weights -- fused multiply-adds on the
+// vector ALU -- and the two halves of a row are added across the lane halves.
+// Sums therefore add up in another order than a row-by-row dot product; f32 throughout.  The lanes with g = 0 run the
+// head for their row; the zeros behind the valid columns of a masked head are written by the whole wave, 16 bytes per
+// lane.
+#include "mlp_common.h"
+
+#pragma clang fp contract(off)
+
+namespace sp {
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+constexpr int EN_ROWS = 32;       // batch rows per tile
+constexpr int EN_HIDDEN = 64;     // width of the hidden layer
+constexpr int EN_THREADS = 256;
+constexpr int EN_MAX_OUT = 4;     // computed outputs
+
+struct EnsembleArgs {
+    const float* x;
+    const float* w1;
+    const float* w2;
+    const float* u;               // (members, batch) uniforms, or nullptr
+    float* policy;                // (members, batch, n)
+    int* action;                  // (members, batch), or nullptr
+    long batch, tiles;
+    int members, k0, n, nout, head, mask_size;
+    PhiloxStream ph;
+};
+
+#ifdef SP_EN_TIMELINE
+__device__ unsigned long long sp_en_timeline[256 * 8 * 8];
+#define SP_EN_STAMP(K) do { if (lane == 0 && wave == 0 && it >= 4 && it < 12) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + (it - 4)) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define SP_EN_STAMP(K) do {} while (0)
+#endif
+
+// KG: 8-wide groups of the input width the kernel is unrolled for; EXACT: K0 = 8 KG (else K0 < 8 KG and the groups
+// past K0 are zeros); ACTION: an action per row is wanted (a uniform per row, from a tensor or a Philox stream)
+template <int KG, bool EXACT, bool ACTION>
+__global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const EnsembleArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 31, g = lane >> 5;
+    const int e = blockIdx.y;
+    const int K0 = EXACT ? 8 * KG : a.k0;
+    const int N = a.n, NOUT = a.nout;
+    const int groups = K0 >> 3;
+    const long batch = a.batch, tiles = a.tiles;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    // ---- the member's weights, once ----
+    f32x4 w1v[2][KG];             // [feature tile][j]: W1[e][32 t + r][8 j + 4 g .. + 3]
+    {
+        const float* w1 = a.w1 + (long)e * EN_HIDDEN * K0;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int j = 0; j < KG; ++j) {
+                const int jj = EXACT || j < groups ? j : 0;
+                const f32x4 v = *reinterpret_cast<const f32x4*>(w1 + (long)(32 * t + r) * K0 + 8 * jj + 4 * g);
+                w1v[t][j] = EXACT || j < groups ? v : zero4;
+            }
+    }
+    f32x4 w2v[EN_MAX_OUT][2][4];  // [output][t][a]: W2[e][o][32 t + 8 a + 4 g .. + 3]: the features this lane half holds
+    {
+        const float* w2 = a.w2 + (long)e * N * EN_HIDDEN;
+#pragma unroll
+        for (int o = 0; o < EN_MAX_OUT; ++o)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int a4 = 0; a4 < 4; ++a4) {
+                    const f32x4 v = *reinterpret_cast<const f32x4*>(w2 + (long)(o < NOUT ? o : 0) * EN_HIDDEN + 32 * t + 8 * a4 + 4 * g);
+                    w2v[o][t][a4] = o < NOUT ? v : zero4;
+                }
+    }
+
+    // inputs of a tile: lane (r, g) takes x[row0 + r][8 j + 4 g .. + 3]; rows past the batch read the last row (their
+    // results are not stored), groups past K0 read group 0 and count as zeros
+    auto load_x = [&](long tile, f32x4 (&xv)[KG]) {
+        long row = tile * EN_ROWS + r;
+        row = row < batch ? row : batch - 1;
+        const float* xr = a.x + row * K0 + 4 * g;
+#pragma unroll
+        for (int j = 0; j < KG; ++j) xv[j] = *reinterpret_cast<const f32x4*>(xr + 8 * (EXACT || j < groups ? j : 0));
+    };
+
+    const long stride = (long)gridDim.x * 4;
+    long tile = (long)blockIdx.x * 4 + wave;
+    if (tile >= tiles) return;
+    f32x4 xv[KG];
+    load_x(tile, xv);
+    const HeadOut out = HeadOut{a.policy, ACTION ? a.action : nullptr, nullptr, a.head, N};
+    const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
+    const bool wave_fill = N > NOUT && (N & 3) == 0;
+    const int s4 = N >> 2, c0 = (NOUT + 3) >> 2;
+
+    // the head of a tile: lane (r, 0) holds the outputs of row r; the zeros behind the valid columns of a masked head
+    // are written by the whole wave, 16 bytes per lane: lane l takes pieces l, l + 64, ... of the tile's 32 s4 pieces.
+    // 64-wide rows (16 pieces): a lane's pieces are 1 KiB apart, all in one column -- eight stores in a straight line;
+    // other widths walk (row and column of a piece advance by fixed steps: no division inside the walk).
+    const int fill_r0 = wave_fill ? lane / s4 : 0, fill_c0 = wave_fill ? lane - fill_r0 * s4 : 0;
+    const int fill_dr = wave_fill ? 64 / s4 : 0, fill_dc = wave_fill ? 64 - fill_dr * s4 : 0;
+    auto finish = [&](long t, const float (&p)[4], float u) {
+        const long row0 = t * EN_ROWS;
+        const long first = (long)e * batch + row0;              // row of the stacked (members x batch) outputs
+        int fill_end = 1 << 30;
+        if (wave_fill) {
+            fill_end = 4 * c0;
+            float* block = a.policy + first * N;
+            const int rows_here = batch - row0 < EN_ROWS ? (int)(batch - row0) : EN_ROWS;
+            if (s4 == 16 && rows_here == EN_ROWS) {
+                if (fill_c0 >= c0) {
+                    f32x4* mine = reinterpret_cast<f32x4*>(block) + lane;
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) mine[64 * k] = zero4;
+                }
+            } else {
+                int rr = fill_r0, c = fill_c0;
+                for (int idx = lane; idx < EN_ROWS * s4; idx += 64) {
+                    if (c >= c0 && rr < rows_here) *reinterpret_cast<f32x4*>(block + rr * N + 4 * c) = zero4;
+                    rr += fill_dr;
+                    c += fill_dc;
+                    if (c >= s4) {
+                        c -= s4;
+                        ++rr;
+                    }
+                }
+            }
+        }
+        if (g == 0 && row0 + r < batch) head_row4_any(a.head, out, p, first + r, NOUT, limit, u, fill_end);
+    };
+
+    int it = -1;
+    for (; tile < tiles; tile += stride) {
+        ++it;
+        SP_EN_STAMP(0);
+        // ---- layer 1: (64 features x 32 rows) += W1 . x^T, two K-values per step ----
+        f32x16 acc[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KG; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w1v[t][j][i], xv[j][i], acc[t], 0, 0, 0);
+        SP_EN_STAMP(1);
+        // the next tile's inputs are on their way while this one passes through the second layer and the head
+        const long next = tile + stride;
+        load_x(next < tiles ? next : tile, xv);
+        float u = 1.f;
+        if constexpr (ACTION) {
+            long row = tile * EN_ROWS + r;
+            row = (long)e * batch + (row < batch ? row : batch - 1);
+            u = a.u != nullptr ? a.u[row] : reference_row_uniform(a.ph, row);
+        }
+        SP_EN_STAMP(2);
+
+        // ---- relu; layer 2: this lane's 32 features of its row against the matching weights, then the other half's ----
+        float p[4];
+#pragma unroll
+        for (int o = 0; o < EN_MAX_OUT; ++o) {
+            float s0 = 0.f, s1 = 0.f;                          // (two chains: an FMA need not wait for the one before)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 16; i += 2) {
+                    s0 = __builtin_fmaf(w2v[o][t][i >> 2][i & 3], fmaxf(acc[t][i], 0.f), s0);
+                    s1 = __builtin_fmaf(w2v[o][t][(i + 1) >> 2][(i + 1) & 3], fmaxf(acc[t][i + 1], 0.f), s1);
+                }
+            const float mine = s0 + s1;
+            p[o] = mine + __shfl_xor(mine, 32);
+        }
+        SP_EN_STAMP(3);
+        finish(tile, p, u);
+        SP_EN_STAMP(4);
+    }
+}
+#undef SP_EN_STAMP
+
+}  // namespace sp
+
+using namespace sp;
+
+template <int KG>
+static const void* pick_ensemble_kernel_kg(bool exact, bool action) {
+    if (exact) return action ? (const void*)mlp_ensemble_kernel<KG, true, true> : (const void*)mlp_ensemble_kernel<KG, true, false>;
+    return action ? (const void*)mlp_ensemble_kernel<KG, false, true> : (const void*)mlp_ensemble_kernel<KG, false, false>;
+}
+static const void* pick_ensemble_kernel(int kg, bool exact, bool action) {
+    return kg == 4 ? pick_ensemble_kernel_kg<4>(exact, action) : kg == 8 ? pick_ensemble_kernel_kg<8>(exact, action)
+                                                                         : pick_ensemble_kernel_kg<16>(exact, action);
+}
+
+// Reference role: the body of `graph_run_host model {ensemble}` (ml/layers.spi:336-344) for a graph of the shape
+// input -> matmul_ensemble -> relu -> matmul_ensemble -> head (game/leduc/model_cem.spi:55-63).
+extern "C" int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layers, const void* const* weights,
+                                       const int32_t* dims, int32_t members, const float* u, const sp_philox_t* philox,
+                                       float* policy_out, int32_t* action_out, int64_t batch, int32_t head,
+                                       int32_t mask_size, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(policy_out);
+    SP_OPTIONAL_PTR(u); SP_OPTIONAL_PTR(action_out);
+    if (weights == nullptr || dims == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: weights/dims is NULL");
+    if (dtype != SP_F32) return fail(SP_ERR_DTYPE, "sp_mlp_forward_ensemble: dtype must be f32");
+    if (n_layers != 2) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: two layers, got %d", n_layers);
+    if (members <= 0 || members > 65535) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: members must be in [1, 65535]");
+    if (batch <= 0 || batch > (1ll << 40) / members) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: batch must be positive (and members x batch below 2^40)");
+    if (head < SP_HEAD_NONE || head > SP_HEAD_SOFTMAX_RM) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: unknown head %d", head);
+    if (action_out != nullptr && u == nullptr && philox == nullptr)
+        return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: action requested but u and philox are NULL");
+    if (u != nullptr && philox != nullptr) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: at most one of u and philox may be given");
+    const int k0 = dims[0], hidden = dims[1], n = dims[2];
+    if (k0 < 8 || k0 % 8 != 0 || k0 > 128)
+        return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: input width %d must be a multiple of 8 in [8, 128]", k0);
+    if (hidden != EN_HIDDEN) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: hidden width must be %d, got %d", EN_HIDDEN, hidden);
+    if (n <= 0 || n > MLP_MAX_OUT) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: output width %d must be in [1, %d]", n, MLP_MAX_OUT);
+    if (mask_size < 0 || mask_size > n) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: mask_size must be in [0, %d], got %d", n, mask_size);
+    // a masked head gives probability zero to the columns past the mask: only the valid ones are computed
+    const int nout = head != SP_HEAD_NONE && mask_size > 0 ? mask_size : n;
+    if (nout > EN_MAX_OUT)
+        return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: at most 4 computed outputs (the head's width, or its mask), got %d", nout);
+    for (int i = 0; i < 2; ++i) {
+        if (weights[i] == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: weights[%d] is NULL", i);
+        if (!aligned16(weights[i])) return fail(SP_ERR_ALIGN, "sp_mlp_forward_ensemble: weights[%d] is not 16-byte aligned", i);
+    }
+    if (!aligned16(x)) return fail(SP_ERR_ALIGN, "sp_mlp_forward_ensemble: x is not 16-byte aligned");
+    if (n % 4 == 0 && !aligned16(policy_out)) return fail(SP_ERR_ALIGN, "sp_mlp_forward_ensemble: policy_out is not 16-byte aligned");
+    EnsembleArgs a{};
+    a.ph.philox_mode = -1;
+    int rc = mlp_set_philox(a.ph, philox, (int64_t)members * batch, n, __func__);
+    if (rc != SP_OK) return rc;
+    rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    a.x = (const float*)x; a.w1 = (const float*)weights[0]; a.w2 = (const float*)weights[1]; a.u = u;
+    a.policy = policy_out; a.action = action_out; a.batch = batch; a.members = members; a.k0 = k0; a.n = n; a.nout = nout;
+    a.head = head; a.mask_size = mask_size;
+    a.tiles = (batch + EN_ROWS - 1) / EN_ROWS;
+    // one workgroup (4 waves, one per SIMD) per compute unit while the members leave room for that: a wave then keeps
+    // its member's weights for all its tiles
+    const long cus = device_cu_count();
+    long gx = (cus + members - 1) / members;
+    const long most = (a.tiles + 3) / 4;
+    if (gx > most) gx = most;
+    if (gx < 1) gx = 1;
+    const int kg = k0 <= 32 ? 4 : k0 <= 64 ? 8 : 16;
+    const void* kernel = pick_ensemble_kernel(kg, k0 == 8 * kg, action_out != nullptr);
+    void* args[] = {(void*)&a};
+    hipError_t err = hipLaunchKernel(kernel, dim3((unsigned)gx, (unsigned)members), dim3(EN_THREADS), args, 0, (hipStream_t)stream);
+    if (err != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward_ensemble: launch failed: %s", hipGetErrorString(err));
+    return check_launch(__func__);
+}
+
+namespace {
+struct MlpEnsembleKernelNames {
+    MlpEnsembleKernelNames() { register_kernel("mlp_forward_ensemble", (const void*)mlp_ensemble_kernel<16, true, false>, EN_THREADS); }
+} mlp_ensemble_kernel_names;
+}  // namespace
+
+#ifdef SP_EN_TIMELINE
+extern "C" int sp_debug_ensemble_timeline(unsigned long long* host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(sp::sp_en_timeline), sizeof(unsigned long long) * 256 * 8 * 8);
+}
+#endif

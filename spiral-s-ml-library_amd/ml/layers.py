@@ -119,6 +119,38 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
     return out + (logits,) if want_logits else out
 
 
+def mlp_forward_ensemble(x, weights, head="regret_matching", u=None, mask_size=0, policy_out=None, action_out=None,
+                         rng=None):
+    """policy[, action] of every member of an ensemble of two-layer f32 stacks on one shared input, one launch:
+    policy[e] = head(relu(x . weights[0][e]^T) . weights[1][e]^T).
+
+    x: (batch, in) f32, in a multiple of 8 up to 128; weights[0]: (E, 64, in), weights[1]: (E, out, 64) f32 (the
+    tensors of `matmul_ensemble`, ml/layers.spi:468-479); head and mask_size as for mlp_forward, with at most 4
+    computed outputs (out, or mask_size).  u: (E, batch) uniforms or rng: a Philox stream over the E * batch stacked
+    rows (member_rows = batch) for an action per member and row; without either only the policy (E, batch, out) is
+    computed -- the graph of the reference's Leduc policy, game/leduc/model_cem.spi:55-63."""
+    if len(weights) != 2:
+        raise ValueError("two weight tensors (E, 64, in) and (E, out, 64) expected")
+    w1, w2 = weights
+    if x.dtype != torch.float32 or w1.dtype != torch.float32 or w2.dtype != torch.float32:
+        raise TypeError("x and the weights must be f32")
+    members, batch = w1.shape[0], x.shape[0]
+    assert w2.shape[0] == members, "both layers need one matrix per member"
+    assert w1.shape[2] == x.shape[1] and w2.shape[2] == w1.shape[1], "The K dimension of the A and B tensors must match."
+    dims = [x.shape[1], w1.shape[1], w2.shape[1]]
+    policy = policy_out if policy_out is not None else \
+        torch.empty((members, batch, dims[-1]), dtype=torch.float32, device=x.device)
+    action = action_out
+    if action is None and (u is not None or rng is not None):
+        action = torch.empty((members, batch), dtype=torch.int32, device=x.device)
+    wp = (C.c_void_p * 2)(ptr(w1, name="weights[0]"), ptr(w2, name="weights[1]"))
+    dp = (C.c_int32 * 3)(*dims)
+    check(lib.sp_mlp_forward_ensemble(_lib.SP_F32, ptr(x, name="x"), 2, wp, dp, members, ptr(u, torch.float32, "u"),
+                                      C.byref(rng) if rng is not None else None, ptr(policy, torch.float32, "policy_out"),
+                                      ptr(action, torch.int32, "action_out"), batch, HEADS[head], mask_size, stream_ptr()))
+    return (policy, action) if action is not None else policy
+
+
 # ----------------------------------------------------------------------------------------------
 # the layer graph (ml/layers.spi:6-55)
 # ----------------------------------------------------------------------------------------------
@@ -773,6 +805,100 @@ def _batchable_key(model, sizes):
     return key if ok[0] else None
 
 
+_ENSEMBLE_HEADS = {"softmax": "softmax", "masked_softmax": "softmax", "regret_matching": "regret_matching",
+                   "masked_regret_matching": "regret_matching", "softmax_and_discrete_sample": "softmax",
+                   "masked_softmax_and_discrete_sample": "softmax",
+                   "regret_matching_and_discrete_sample": "regret_matching",
+                   "masked_regret_matching_and_discrete_sample": "regret_matching"}
+
+
+def _fused_ensemble_plan(model, key):
+    """`input -> matmul_ensemble -> relu -> matmul_ensemble -> head` over f32 tensors with the members' outputs stacked
+    under `apply key` (the Leduc policy of game/leduc/model_cem.spi:55-63) in the shapes sp_mlp_forward_ensemble takes:
+    (x node, [stacked weight nodes], stacked output node(s), top node) or None."""
+    top = model.graph
+
+    def passive(k):   # tensors only, nothing to compute: the tables a model keeps beside its network
+        if isinstance(k, (Layer, KeyScalar)):
+            return True
+        if isinstance(k, (KeyGraph, Fst, Snd)):
+            return passive(k.x)
+        if isinstance(k, (Pair, Zip, Apply)):
+            return passive(k.a) and passive(k.b)
+        return False
+
+    while isinstance(top, Pair) and passive(top.b):
+        top = top.a
+    sampling = isinstance(top, BlockRowMapReduce)
+    if not isinstance(top, (BlockRowMap, BlockRowMapReduce)) or top.f not in _ENSEMBLE_HEADS or top.out is None:
+        return None
+
+    def stacked(k):   # `apply key t` -> t
+        while isinstance(k, KeyGraph):
+            k = k.x
+        if isinstance(k, Apply) and isinstance(k.b, KeyScalar) and k.b.key == key and passive(k.a):
+            return k.a
+        return None
+
+    if sampling:
+        out = top.out
+        while isinstance(out, KeyGraph):
+            out = out.x
+        if not isinstance(out, Pair):
+            return None
+        outs = (stacked(out.a), stacked(out.b))
+    else:
+        outs = (stacked(top.out),)
+    if any(o is None for o in outs):
+        return None
+    second = top.a
+    if not isinstance(second, BlockMatmul):
+        return None
+    hidden = second.a
+    if not (isinstance(hidden, BlockMap) and hidden.f == "relu" and hidden.out is None and isinstance(hidden.a, BlockMatmul)):
+        return None
+    first = hidden.a
+    weights = [stacked(first.b), stacked(second.b)]
+    x = first.a
+    while isinstance(x, KeyGraph):
+        x = x.x
+    if any(w is None for w in weights) or not isinstance(x, Layer):
+        return None
+    return x, weights, outs, top
+
+
+def _run_fused_ensemble(model, key, count, ls):
+    """One sp_mlp_forward_ensemble launch in place of the batched pass, where the graph is of that shape."""
+    plan = _fused_ensemble_plan(model, key)
+    if plan is None:
+        return False
+    x_node, w_nodes, out_nodes, top = plan
+    tensor = lambda node: graph_extract(Model(node, model.dims, model.data))
+    x, (w1, w2) = tensor(x_node), [tensor(w) for w in w_nodes]
+    probs = tensor(out_nodes[0])
+    if x.dim() != 3 or w1.dim() != 3 or w2.dim() != 3 or any(t.dtype != torch.float32 for t in (x, w1, w2, probs)):
+        return False
+    q, w, k0 = x.shape
+    cols = w2.shape[1]
+    computed = top.size or cols
+    if not (w1.shape[0] == w2.shape[0] == count and w1.shape[1] == w2.shape[2] == 64 and w1.shape[2] == k0 and
+            k0 % 8 == 0 and 8 <= k0 <= 128 and cols <= 64 and computed <= 4 and probs.shape == (count, q, w, cols)):
+        return False
+    action, rng = None, None
+    if len(out_nodes) == 2:
+        action = tensor(out_nodes[1])
+        if action.shape != (count, q, w) or action.dtype != torch.int32 or cols % 4 != 0:
+            return False
+        # member e draws what the e-th sequential run would: every run takes one sampling node's draws
+        draws = _sampling_draws(w, cols)
+        rng = _prim.philox(_lib.PHILOX_LAYER, seed=ls.seed, threads_per_block=THREADS_PER_BLOCK, blocks_per_grid=q,
+                           rows_per_block=w, offset=ls.draws, member_rows=q * w, member_draws=draws)
+        ls.draws += draws
+    mlp_forward_ensemble(_flat(x), (w1, w2), _ENSEMBLE_HEADS[top.f], None, top.size, probs.reshape(count, q * w, cols),
+                         action.reshape(count, q * w) if action is not None else None, rng)
+    return True
+
+
 def _graph_run_batched(model, key, count, ls):
     """`loop.linear {key=count} fun indices => graph_run_device m ls indices` (ml/layers.spi:343-344) as ONE
     pass: `apply key t` yields the whole tensor, every node downstream works on `count` stacked members
@@ -944,19 +1070,20 @@ def graph_run_host(model, sizes=None, seed=_prim.CONSTANT_SEED, fuse=True, batch
         return
     tape = _lib.start_tape()
     try:
-        _graph_run_walk(model, sizes, seed, batched)
+        _graph_run_walk(model, sizes, seed, batched, fuse)
     finally:
         _lib.stop_tape()
     tapes[tape_key] = (tuple(d["array"] for d in data), tape)
 
 
-def _graph_run_walk(model, sizes, seed, batched):
-    """One run by walking the graph: a single batched pass over one key where that is possible, else every
-    combination of the key indices in turn."""
+def _graph_run_walk(model, sizes, seed, batched, fuse=True):
+    """One run by walking the graph: a single batched pass over one key where that is possible (a single fused launch
+    where the graph is a two-layer relu stack per member), else every combination of the key indices in turn."""
     ls = create_layer_state(seed)
     key = _batchable_key(model, sizes) if batched and sizes else None
     if key is not None and sizes[key] > 1:
-        _graph_run_batched(model, key, sizes[key], ls)
+        if not (fuse and _run_fused_ensemble(model, key, sizes[key], ls)):
+            _graph_run_batched(model, key, sizes[key], ls)
         return
     keys = list(sizes)
     for combo in itertools.product(*[range(sizes[k]) for k in keys]):

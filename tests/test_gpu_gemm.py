@@ -415,6 +415,30 @@ def test_device_and_kernel_info():
         _lib.kernel_info("no_such_kernel")
 
 
+def test_clock_sample_gives_the_shader_clock():
+    """Two sp_clock_sample results around a stretch of work: per SIMD sampled both times the cycle counter's advance
+    over the 100 MHz counter's is the shader clock; the SIMDs of the chip agree on it, and it lies in the part's range."""
+    announce("clock sample")
+    from ml import _lib, matmul
+    slots = 32768
+    samples = torch.zeros((2, slots, 2), dtype=torch.int64, device="cuda")
+    a = torch.randn((2048, 2048), device="cuda").to(torch.bfloat16)
+    c = torch.empty((2048, 2048), dtype=torch.float32, device="cuda")
+    for _ in range(50):
+        matmul.matmul_abt(a, a, c=c)
+    _lib.check(_lib.lib.sp_clock_sample(samples[0].data_ptr(), _lib.stream_ptr()))
+    for _ in range(200):
+        matmul.matmul_abt(a, a, c=c)
+    _lib.check(_lib.lib.sp_clock_sample(samples[1].data_ptr(), _lib.stream_ptr()))
+    s = host(samples)
+    both = (s[0, :, 1] != 0) & (s[1, :, 1] > s[0, :, 1])
+    assert both.sum() >= 512                      # most of the chip's 1024 SIMDs were reached both times
+    mhz = (s[1, both, 0] - s[0, both, 0]) / (s[1, both, 1] - s[0, both, 1]) * 100.0
+    med = np.median(mhz)
+    assert 500 < med < 2600
+    assert (np.abs(mhz - med) < 0.05 * med).mean() > 0.9      # (the XCDs settle a few percent apart under a power limit)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("e,m,n,k,shared", [(16, 1536, 64, 64, "a"), (5, 256, 256, 128, None), (3, 100, 24, 40, "a"),
                                             (4, 128, 512, 64, "b"), (40, 64, 64, 64, "a")])

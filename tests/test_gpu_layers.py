@@ -306,3 +306,46 @@ def test_replayed_runs_see_new_inputs_and_weights(L, kind):
         if previous is not None:
             assert not (got[0] == previous).all()
         previous = got[0]
+
+
+@pytest.mark.parametrize("sampling", [False, True])
+def test_leduc_policy_graph_runs_as_one_launch(L, sampling):
+    """The graph of the reference's Leduc policy (game/leduc/model_cem.spi:55-63: input -> matmul_ensemble_with_adjoint
+    (E, 128, 64) -> relu -> matmul_ensemble_with_adjoint (E, 64, 64) -> masked_regret_matching' 3 into the members'
+    stacked output (or, second case, masked_softmax_and_discrete_sample' 3), paired with a table that computes nothing): `graph_run_host model {ensemble}` takes the fused
+    ensemble kernel, and gives what the batched node-by-node pass gives (f32 bar: 1e-5) -- with a sampling head also the
+    same draws per member: actions bit-exact given the policy and the stream."""
+    from ml import _lib
+    announce("layers leduc policy graph, sampling=%s" % sampling)
+    ensemble, w = 8, 256
+    probs = L.apply("ensemble", L.input("output_probs", (ensemble, Q, w, 64)))
+    x = L.pipe(L.input("input", (Q, w, 128)), L.matmul_ensemble_with_adjoint((ensemble, 128, 64)), L.relu,
+               L.matmul_ensemble_with_adjoint((ensemble, 64, 64)))
+    if sampling:
+        out = L.pair(probs, L.apply("ensemble", L.input("output_indices", (ensemble, Q, w), "int")))
+        neural = L.masked_softmax_and_discrete_sample_(3, out, x)
+    else:
+        neural = L.masked_regret_matching_(3, probs, x)
+    g = L.pair(neural, L.input("cem_table", (ensemble, 16, 4)))
+    m = L.create_model(g)
+    L.pass_init(m)
+    fill(L.key_extract(m, "input"), np.random.default_rng(5))
+    assert L._fused_ensemble_plan(m, "ensemble") is not None
+    L.graph_run_host(m, {"ensemble": ensemble}, fuse=False)
+    want_p = host(L.key_extract(m, "output_probs")).copy()
+    want_i = host(L.key_extract(m, "output_indices")).copy() if sampling else None
+    L.key_extract(m, "output_probs").fill_(7)
+    for run in range(2):          # the second run replays the recorded launch
+        L.graph_run_host(m, {"ensemble": ensemble})
+        got_p = host(L.key_extract(m, "output_probs"))
+        assert ogemm.rel_frobenius(got_p.reshape(-1, 64), want_p.reshape(-1, 64)) < 1e-5
+        assert (got_p[..., 3:] == 0).all() and np.abs(got_p.sum(axis=-1) - 1).max() < 1e-5
+        if sampling:
+            got_i = host(L.key_extract(m, "output_indices"))
+            assert (got_i != want_i).mean() < 1e-3          # (a policy one ulp apart can move a threshold across a draw)
+            per_node = ophilox.draws_per_sampling_node(w, 64)
+            for e in range(ensemble):
+                u = ophilox.row_uniforms_layer(Q, w, 64, offset=e * per_node)
+                assert (got_i[e].reshape(-1) == orow.discrete_sampling(got_p[e].reshape(-1, 64), u)).all()
+    tape = m._tapes[(L._prim.CONSTANT_SEED, True, True, (("ensemble", ensemble),))][1]
+    assert len(tape.calls) == 1 and tape.calls[0][0].__name__ == "sp_mlp_forward_ensemble"

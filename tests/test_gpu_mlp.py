@@ -376,3 +376,60 @@ def test_resident_kernel_run_to_run_and_philox(LY):
         drawn = LY.mlp_forward(xd, wd, None, "softmax", None, 3, packed=packed, rng=cfg)
         assert all(torch.equal(a, b) for a, b in zip(first, drawn))
         assert (host(first[1]) == orow.discrete_sampling(host(first[0]), host(u))).all()
+
+
+@pytest.mark.parametrize("members,batch,dims,head,mask,sample", [
+    (32, 6144, [128, 64, 64], "regret_matching", 3, None),      # the reference's Leduc policy: 3 valid of 64 columns, no sampling
+    (5, 1000, [128, 64, 64], "softmax", 3, "u"),                 # ragged last tile, uniforms from a tensor
+    (3, 4100, [64, 64, 4], "softmax_regret_matching", 0, "u"),   # a head 4 wide, no mask: dense rows
+    (7, 777, [24, 64, 6], "regret_matching", 2, "philox"),       # K0 not a multiple of 32, row width not a multiple of 4
+    (300, 64, [8, 64, 64], "softmax", 4, "philox"),              # more members than compute units
+])
+def test_ensemble_forward(LY, members, batch, dims, head, mask, sample):
+    """sp_mlp_forward_ensemble -- every member's relu(x.W1^T).W2^T + head in one launch -- against the oracle's
+    forward of each member on its own (f32: relative Frobenius error below 1e-5, the f32 bar), zeros behind the
+    mask, and actions bit-exact given the kernel's own policy and the member's uniforms."""
+    from ml import _lib, primitives
+    from oracle import philox as ophilox
+    announce("mlp ensemble members=%d batch=%d dims=%s head=%s mask=%d sample=%s" % (members, batch, dims, head, mask, sample))
+    rng = np.random.default_rng(members * 1000 + batch)
+    x = rng.standard_normal((batch, dims[0]), dtype=np.float32)
+    w1 = rng.standard_normal((members, dims[1], dims[0]), dtype=np.float32) * np.float32(1 / np.sqrt(dims[0]))
+    w2 = rng.standard_normal((members, dims[2], dims[1]), dtype=np.float32) * np.float32(1 / np.sqrt(dims[1]))
+    u, cfg = None, None
+    if sample == "u":
+        u = (1 - rng.random((members, batch), dtype=np.float32)).astype(np.float32)
+    elif sample == "philox":
+        # the stacked rows of the members, each member a run of its own `member_draws` further into every thread's stream
+        cols = dims[2] if dims[2] % 4 == 0 else 8
+        cfg = primitives.philox(_lib.PHILOX_LAYER, blocks_per_grid=1, rows_per_block=batch, member_rows=batch, member_draws=12)
+        u = host(primitives.philox_uniforms(cfg, members * batch, cols)).reshape(members, batch)
+        if dims[2] % 4 != 0:
+            sample = "u"          # (a Philox stream needs 16-byte rows: such a head takes the same numbers as a tensor)
+    out = LY.mlp_forward_ensemble(dev(x), (dev(w1), dev(w2)), head, dev(u) if sample == "u" else None, mask,
+                                  rng=cfg if sample == "philox" else None)
+    policy, action = (host(out[0]), host(out[1])) if sample else (host(out), None)
+    assert policy.shape == (members, batch, dims[2])
+    for e in range(members):
+        want, _, _ = olayers.mlp_forward(x, [w1[e], w2[e]], None, HEAD_CODE[head], None, None, mask or None)
+        assert ogemm.rel_frobenius(policy[e], want) < 1e-5, e
+        if mask:
+            assert (policy[e][:, mask:] == 0).all()
+        assert np.abs(policy[e].sum(axis=1) - 1).max() < 1e-5
+        if sample:
+            assert (action[e] == orow.discrete_sampling(policy[e], u[e])).all(), e
+    if sample:
+        assert len(np.unique(action)) > 1
+
+
+def test_ensemble_rejects_what_it_does_not_take(LY):
+    from ml import _lib
+    x = torch.zeros((64, 128), dtype=torch.float32, device="cuda")
+    w1 = torch.zeros((2, 64, 128), dtype=torch.float32, device="cuda")
+    with pytest.raises(_lib.SpiralError) as err:      # 64 computed outputs: left to the node-by-node pass
+        LY.mlp_forward_ensemble(x, (w1, torch.zeros((2, 64, 64), dtype=torch.float32, device="cuda")), "softmax")
+    assert err.value.code == -2
+    with pytest.raises(_lib.SpiralError) as err:      # a hidden layer of another width
+        LY.mlp_forward_ensemble(x, (torch.zeros((2, 32, 128), dtype=torch.float32, device="cuda"),
+                                    torch.zeros((2, 4, 32), dtype=torch.float32, device="cuda")), "softmax")
+    assert err.value.code == -2
