@@ -46,8 +46,11 @@ struct EnsembleArgs {
 };
 
 #ifdef SP_EN_TIMELINE
+#ifndef SP_EN_TL_FIRST
+#define SP_EN_TL_FIRST 4
+#endif
 __device__ unsigned long long sp_en_timeline[256 * 8 * 8];
-#define SP_EN_STAMP(K) do { if (lane == 0 && wave == 0 && it >= 4 && it < 12) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + (it - 4)) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
+#define SP_EN_STAMP(K) do { if (lane == 0 && wave == 0 && it >= SP_EN_TL_FIRST && it < SP_EN_TL_FIRST + 8) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + (it - SP_EN_TL_FIRST)) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
 #else
 #define SP_EN_STAMP(K) do {} while (0)
 #endif
@@ -65,6 +68,12 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
     const int groups = K0 >> 3;
     const long batch = a.batch, tiles = a.tiles;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#ifdef SP_EN_TIMELINE
+#define SP_EN_MARK(K) do { if (lane == 0 && wave == 0) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + 0) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define SP_EN_MARK(K) do {} while (0)
+#endif
+    SP_EN_MARK(5);
 
     // ---- the member's weights, once ----
     f32x4 w1v[2][KG];             // [feature tile][j]: W1[e][32 t + r][8 j + 4 g .. + 3]
@@ -95,19 +104,22 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
 
     // inputs of a tile: lane (r, g) takes x[row0 + r][8 j + 4 g .. + 3]; rows past the batch read the last row (their
     // results are not stored), groups past K0 read group 0 and count as zeros
-    auto load_x = [&](long tile, f32x4 (&xv)[KG]) {
+    auto x_row = [&](long tile) {
         long row = tile * EN_ROWS + r;
         row = row < batch ? row : batch - 1;
-        const float* xr = a.x + row * K0 + 4 * g;
-#pragma unroll
-        for (int j = 0; j < KG; ++j) xv[j] = *reinterpret_cast<const f32x4*>(xr + 8 * (EXACT || j < groups ? j : 0));
+        return a.x + row * K0 + 4 * g;
     };
+    auto load_piece = [&](const float* xr, int j) { return *reinterpret_cast<const f32x4*>(xr + 8 * (EXACT || j < groups ? j : 0)); };
 
     const long stride = (long)gridDim.x * 4;
     long tile = (long)blockIdx.x * 4 + wave;
     if (tile >= tiles) return;
     f32x4 xv[KG];
-    load_x(tile, xv);
+    {
+        const float* xr = x_row(tile);
+#pragma unroll
+        for (int j = 0; j < KG; ++j) xv[j] = load_piece(xr, j);
+    }
     const HeadOut out = HeadOut{a.policy, ACTION ? a.action : nullptr, nullptr, a.head, N};
     const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
     const bool wave_fill = N > NOUT && (N & 3) == 0;
@@ -150,26 +162,29 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
     };
 
     int it = -1;
+    SP_EN_MARK(6);
     for (; tile < tiles; tile += stride) {
         ++it;
         SP_EN_STAMP(0);
-        // ---- layer 1: (64 features x 32 rows) += W1 . x^T, two K-values per step ----
+        // ---- layer 1: (64 features x 32 rows) += W1 . x^T, two K-values per step.  A register of inputs is asked for
+        //      the NEXT tile's values as soon as this tile's MFMAs have read it: they arrive a whole tile ahead. ----
+        const long next = tile + stride;
+        const float* const xr_next = x_row(next < tiles ? next : tile);
         f32x16 acc[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int i = 0; i < 16; ++i) acc[t][i] = 0.f;
 #pragma unroll
-        for (int j = 0; j < KG; ++j)
+        for (int j = 0; j < KG; ++j) {
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w1v[t][j][i], xv[j][i], acc[t], 0, 0, 0);
+            xv[j] = load_piece(xr_next, j);
+        }
         SP_EN_STAMP(1);
-        // the next tile's inputs are on their way while this one passes through the second layer and the head
-        const long next = tile + stride;
-        load_x(next < tiles ? next : tile, xv);
         float u = 1.f;
         if constexpr (ACTION) {
             long row = tile * EN_ROWS + r;
@@ -197,8 +212,10 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
         finish(tile, p, u);
         SP_EN_STAMP(4);
     }
+    SP_EN_MARK(7);
 }
 #undef SP_EN_STAMP
+#undef SP_EN_MARK
 
 }  // namespace sp
 
