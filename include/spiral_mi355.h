@@ -317,8 +317,8 @@ int sp_reduce_set_poll_limit(int64_t microseconds);
 
 /* sp_reduce_sum for callers that cannot allocate device memory or hand over a workspace (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.  The
- * partial sums and their valid marks live in a 16 KiB array inside the library's own device image, one copy
- * per GPU, kept until the process ends; the call allocates nothing and uses no memset.  Same kernel, same grid and
+ * partial sums and their valid marks live in a 16 KiB + 16 B array (the marked slots and the give-up counter) inside
+ * the library's own device image, one copy per GPU, kept until the process ends; the call allocates nothing and uses no memset.  Same kernel, same grid and
  * therefore bit-identical results to sp_reduce_sum.  n must not exceed sp_reduce_sum_static_max_n() (2^36
  * elements), else SP_ERR_SHAPE.  All calls on one GPU share the array: calls that may overlap in time (different
  * streams, different threads) race and must be serialised by the caller. */
