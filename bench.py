@@ -526,6 +526,9 @@ def main():
         "roofline": head["roofline"], "cpu_baseline": cpu,
         "shader_clock_mhz": head.get("shader_clock_mhz"),
         "mlp_rows_per_s": mlp["mlp_leduc_16384x64_one_launch_rowmajor"],
+        "mlp_rows_per_s_note": "the drop-in call sp_mlp_forward on the row-major weights the reference keeps, ONE launch over 64 "
+                               "batches of 16384 rows (weights stay in registers across the batches); the packed-weights figures "
+                               "assume weights packed once outside the timed region; the per-batch launch modes are in the detail",
         "mlp_rows_per_s_detail": {
             "row_major_weights_one_launch_over_64_batches": mlp["mlp_leduc_16384x64_one_launch_rowmajor"],
             "packed_weights_one_launch_over_64_batches": mlp["mlp_leduc_16384x64_one_launch"],

@@ -302,7 +302,7 @@ def test_four_wave_kernel_on_tall_shapes_is_exact_on_integers(MM, dtype):
 
 
 @pytest.mark.parametrize("m,n,k", [(65536, 256, 1152), (65536, 2048, 512), (4096, 512, 8192), (6144, 8192, 256),
-                                   (8192, 6144, 1152), (8192, 8192, 128)])
+                                   (8192, 6144, 1152), (8192, 8192, 128), (8192, 8192, 256)])
 def test_streamed_and_written_through_outputs_are_exact_on_integers(MM, m, n, k):
     """The stores of C carry a cache policy chosen per launch: written through the L2, or -- operands of 140 MiB and
     more, or an output of 384 MiB and more -- streamed past the caches.  The streamed form on the eight-wave kernel
