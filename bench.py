@@ -444,7 +444,42 @@ def main():
                               "launch each; node_by_node_ms: the same graph with fuse=False (batched GEMM, relu map, "
                               "batched GEMM, row map: four launches); rows_per_s counts member-rows"}
 
-        cases += [("ensemble_leduc_policy_e32", ensemble_case)]
+        def cfr_case():
+            # The reference's CFR model (game/leduc/model_cfr.spi:56-61): E = 4 members, 128 -> 128, binarize into 4096
+            # worlds, f32, on blocks_per_grid x 256 rows; graph_run_host(model, {"ensemble": 4}) is ONE launch that computes
+            # the 32 columns the hash can see and never writes the product.
+            ens, q, w = 4, layers.blocks_per_grid(), 256
+            world = layers.apply("ensemble", layers.input("output_world_id", (ens, q, w), "int"))
+            net = layers.pipe(layers.input("input", (q, w, 128)), layers.matmul_ensemble((ens, 128, 128)))
+            m = layers.create_model(layers.binarize_(1 << 12, world, net))
+            rng = np.random.default_rng(12)
+            xin = layers.key_extract(m, "input")
+            x = rng.standard_normal(tuple(xin.shape), dtype=np.float32)
+            xin.copy_(dev(x))
+            wt = layers.key_extract_list(m, "weights")[0]
+            wv = rng.standard_normal(tuple(wt.shape), dtype=np.float32)
+            wt.copy_(dev(wv))
+            rows = q * w
+            fn = lambda: layers.graph_run_host(m, {"ensemble": ens})
+            wall, ev = time_launches(fn, K, W)
+            mhz = CLOCK["mhz"]
+            got = layers.key_extract(m, "output_world_id").cpu().numpy().reshape(ens, rows).view(np.uint32)
+            sample = slice(0, rows, max(1, rows // 2048))
+            for e in (0, ens - 1):                                # what was timed is checked (signs next to zero aside)
+                y = ogemm.gemm_abt(x.reshape(rows, 128)[sample], wv[e])
+                sure = (np.abs(y[:, :32]) > 1e-4).all(axis=1)
+                assert (got[e][sample][sure] == orow.binarize(y, 1 << 12)[sure]).all(), "bench CFR hash drifted from the oracle"
+            slow = lambda: layers.graph_run_host(m, {"ensemble": ens}, fuse=False)
+            _, ev_nodes = time_launches(slow, max(K // 10, 5), 2)
+            fl = 2.0 * rows * ens * 128 * 32               # the 32 columns the device's 32-bit shift lets the hash see
+            return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(rows * ens / (ev * 1e-3), 1),
+                    "roofline": roofline_mfma(fl, ev, "f32"), "seed": 12, "shader_clock_mhz": mhz, "rows": rows,
+                    "members": ens, "node_by_node_ms": round(ev_nodes, 5),
+                    "timing": "mean over back-to-back graph_run_host(model, {ensemble: 4}) calls, one sp_ensemble_binarize "
+                              "launch each; node_by_node_ms: the same graph with fuse=False (batched GEMM over all 128 "
+                              "columns, then the row hash); rows_per_s counts member-rows"}
+
+        cases += [("ensemble_leduc_policy_e32", ensemble_case), ("ensemble_leduc_cfr_e4", cfr_case)]
         cases += [("mlp_leduc_16384", mlp_case), ("mlp_leduc_16384_rowmajor", lambda: mlp_case(False)),
                   ("mlp_leduc_16384x64_one_launch", lambda: mlp_case(True, 64)),
                   ("mlp_leduc_16384x64_one_launch_rowmajor", lambda: mlp_case(False, 64)),

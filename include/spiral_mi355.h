@@ -410,21 +410,34 @@ int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers, const void
                           float* policy_out, int32_t* action_out, float* logits_out, int64_t batch, int32_t head,
                           int32_t mask_size, void* stream);
 
-/* Fused forward of an ENSEMBLE of two-layer f32 stacks on one shared input, one launch:
- *   policy[e] = head(relu(x . W1[e]^T) . W2[e]^T),  e = 0 .. members - 1
- * x: (batch, dims[0]) f32; weights[0]: (members, dims[1], dims[0]), weights[1]: (members, dims[2], dims[1]) f32,
- * the stacked tensors of `matmul_ensemble` (ml/layers.spi:468-479); dims[0] a multiple of 8 in [8, 128], dims[1] = 64,
- * dims[2] <= 64; n_layers = 2; dtype = SP_F32.  head / mask_size as for sp_mlp_forward, with at most 4 computed
- * outputs (dims[2], or mask_size of a masked head; the columns behind the mask are written as zeros).
- * policy_out: (members, batch, dims[2]); action_out: (members, batch) or NULL; u: (members, batch) uniforms in
+/* Fused forward of an ENSEMBLE of one- or two-layer f32 stacks on one shared input, one launch:
+ *   n_layers = 2:  policy[e] = head(relu(x . W1[e]^T) . W2[e]^T)
+ *   n_layers = 1:  policy[e] = head(x . W1[e]^T),                 e = 0 .. members - 1
+ * x: (batch, dims[0]) f32; weights[i]: (members, dims[i + 1], dims[i]) f32, the stacked tensors of `matmul_ensemble`
+ * (ml/layers.spi:468-479).  Two layers: dims[0] a multiple of 8 in [8, 128], dims[1] = 64; one layer: dims[0] a
+ * multiple of 8 in [8, 256].  Output width dims[n_layers] <= 64; dtype = SP_F32.  head / mask_size as for
+ * sp_mlp_forward, with at most 4 computed outputs (the output width, or mask_size of a masked head; the columns behind
+ * the mask are written as zeros).
+ * policy_out: (members, batch, dims[n_layers]); action_out: (members, batch) or NULL; u: (members, batch) uniforms in
  * (0, 1] or NULL; philox: a stream over the members x batch stacked rows (member_rows = batch) or NULL; at most one
  * of u and philox, one of them when action_out is given.
  * Replaces: `graph_run_host model {ensemble}` (ml/layers.spi:336-344, the interpreter of :194-240 run member by
- * member) for the graph of the reference's Leduc policy, game/leduc/model_cem.spi:55-63
- * (input -> matmul_ensemble_with_adjoint -> relu -> matmul_ensemble_with_adjoint -> masked_regret_matching'). */
+ * member) for the graphs of the reference's CEM policies: game/leduc/model_cem.spi:55-63
+ * (input -> matmul_ensemble_with_adjoint -> relu -> matmul_ensemble_with_adjoint -> masked_regret_matching') and
+ * game/nl_hu_holdem/model_cem.spi:84-100 (input -> matmul_ensemble_with_adjoint -> masked_regret_matching'). */
 int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layers, const void* const* weights, const int32_t* dims,
                             int32_t members, const float* u, const sp_philox_t* philox, float* policy_out,
                             int32_t* action_out, int64_t batch, int32_t head, int32_t mask_size, void* stream);
+
+/* out[e][r] = (OR over j of (not (y[r, j] <= 0)) << j) mod modulo with y = x . W[e]^T: one ensemble layer and the hash
+ * head `binarize` in one launch; y is never written.  x: (batch, k0) f32, k0 a multiple of 8 in [8, 256]; weights:
+ * (members, n, k0) f32; out: (members, batch) u32.  As in sp_row_binarize the shift is the device's 32-bit shift
+ * (columns j >= 32 contribute nothing, so only the first 32 rows of every W[e] are read) and a NaN sets its bit.
+ * Replaces: `graph_run_host model {ensemble}` for input -> matmul_ensemble -> binarize' (the reference's CFR
+ * models, game/leduc/model_cfr.spi:56-61, game/nl_hu_holdem/model_cfr.spi:82-88; ml/layers.spi:439-446,
+ * ml/primitives.spi:817-821). */
+int sp_ensemble_binarize(int dtype, const void* x, const void* weights, uint32_t* out, int32_t members, int64_t batch,
+                         int32_t k0, int32_t n, uint32_t modulo, void* stream);
 
 #ifdef __cplusplus
 }

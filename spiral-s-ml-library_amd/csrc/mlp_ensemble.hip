@@ -42,6 +42,8 @@ struct EnsembleArgs {
     int* action;                  // (members, batch), or nullptr
     long batch, tiles;
     int members, k0, n, nout, head, mask_size;
+    unsigned* words;              // (members, batch) hash words of the binarize head, or nullptr
+    unsigned modulo;
     PhiloxStream ph;
 };
 
@@ -217,6 +219,116 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
 #undef SP_EN_STAMP
 #undef SP_EN_MARK
 
+// ONE ensemble layer and its head: policy[e] = head(x . W[e]^T) for a head of at most 4 computed outputs, or
+// word[e][r] = (OR over j < 32 of (not (y[r][j] <= 0)) << j) mod modulo with y = x . W[e]^T -- the graphs of the
+// reference's other agents (game/nl_hu_holdem/model_cem.spi:84-100: matmul_ensemble_with_adjoint -> masked regret
+// matching; game/leduc/model_cfr.spi:56-61 and game/nl_hu_holdem/model_cfr.spi:82-88: matmul_ensemble -> binarize,
+// ml/primitives.spi:817-821).  Either head needs at most the first 32 output columns, so the layer is ONE 32 x 32
+// MFMA tile per 32 batch rows (the weights' rows past the needed columns are zeros) instead of the full product, and the
+// (members x batch x outputs) activations are never written.  Same walk, same operand mapping and the same input
+// prefetch as the first layer of the kernel above; lane (r, g) ends up with outputs 8 a + 4 g + b of row r.
+// MODE 0: policy, 1: policy and action, 2: binarize.
+template <int KG, bool EXACT, int MODE>
+__global__ __launch_bounds__(EN_THREADS) void ensemble_layer_kernel(const EnsembleArgs a) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = lane & 31, g = lane >> 5;
+    const int e = blockIdx.y;
+    const int K0 = EXACT ? 8 * KG : a.k0;
+    const int N = a.n, NOUT = a.nout;                        // NOUT: rows of W that are read (<= 32)
+    const int groups = K0 >> 3;
+    const long batch = a.batch, tiles = a.tiles;
+    const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+
+    f32x4 wv[KG];                                            // W[e][r][8 j + 4 g .. + 3], rows past NOUT are zeros
+    {
+        const float* w = a.w1 + ((long)e * N + (r < NOUT ? r : 0)) * K0 + 4 * g;
+#pragma unroll
+        for (int j = 0; j < KG; ++j) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(w + 8 * (EXACT || j < groups ? j : 0));
+            wv[j] = (EXACT || j < groups) && r < NOUT ? v : zero4;
+        }
+    }
+    auto x_row = [&](long tile) {
+        long row = tile * EN_ROWS + r;
+        row = row < batch ? row : batch - 1;
+        return a.x + row * K0 + 4 * g;
+    };
+    auto load_piece = [&](const float* xr, int j) { return *reinterpret_cast<const f32x4*>(xr + 8 * (EXACT || j < groups ? j : 0)); };
+
+    const long stride = (long)gridDim.x * 4;
+    long tile = (long)blockIdx.x * 4 + wave;
+    if (tile >= tiles) return;
+    f32x4 xv[KG];
+    {
+        const float* xr = x_row(tile);
+#pragma unroll
+        for (int j = 0; j < KG; ++j) xv[j] = load_piece(xr, j);
+    }
+    const HeadOut out = HeadOut{a.policy, MODE == 1 ? a.action : nullptr, nullptr, a.head, N};
+    const int limit = a.mask_size > 0 ? a.mask_size : NOUT;
+    const bool wave_fill = MODE != 2 && N > NOUT && (N & 3) == 0;
+    const int s4 = N >> 2, c0 = (NOUT + 3) >> 2;
+    const int fill_r0 = wave_fill ? lane / s4 : 0, fill_c0 = wave_fill ? lane - fill_r0 * s4 : 0;
+    const int fill_dr = wave_fill ? 64 / s4 : 0, fill_dc = wave_fill ? 64 - fill_dr * s4 : 0;
+
+    for (; tile < tiles; tile += stride) {
+        const long next = tile + stride;
+        const float* const xr_next = x_row(next < tiles ? next : tile);
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+        for (int j = 0; j < KG; ++j) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[j][i], xv[j][i], acc, 0, 0, 0);
+            xv[j] = load_piece(xr_next, j);
+        }
+        const long row0 = tile * EN_ROWS;
+        const long first = (long)e * batch + row0;              // row of the stacked (members x batch) outputs
+        if constexpr (MODE == 2) {
+            unsigned word = 0;
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                word |= (acc[i] <= 0.f ? 0u : 1u) << (8 * (i >> 2) + 4 * g + (i & 3));
+            word |= (unsigned)__shfl_xor((int)word, 32);
+            if (g == 0 && row0 + r < batch) a.words[first + r] = word % a.modulo;
+        } else {
+            float u = 1.f;
+            if constexpr (MODE == 1) {
+                const long row = first + (row0 + r < batch ? r : 0);
+                u = a.u != nullptr ? a.u[row] : reference_row_uniform(a.ph, row);
+            }
+            int fill_end = 1 << 30;
+            if (wave_fill) {
+                fill_end = 4 * c0;
+                float* block = a.policy + first * N;
+                const int rows_here = batch - row0 < EN_ROWS ? (int)(batch - row0) : EN_ROWS;
+                if (s4 == 16 && rows_here == EN_ROWS) {
+                    if (fill_c0 >= c0) {
+                        f32x4* mine = reinterpret_cast<f32x4*>(block) + lane;
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) mine[64 * k] = zero4;
+                    }
+                } else {
+                    int rr = fill_r0, c = fill_c0;
+                    for (int idx = lane; idx < EN_ROWS * s4; idx += 64) {
+                        if (c >= c0 && rr < rows_here) *reinterpret_cast<f32x4*>(block + rr * N + 4 * c) = zero4;
+                        rr += fill_dr;
+                        c += fill_dc;
+                        if (c >= s4) {
+                            c -= s4;
+                            ++rr;
+                        }
+                    }
+                }
+            }
+            const float p[4] = {acc[0], acc[1], acc[2], acc[3]};
+            if (g == 0 && row0 + r < batch) head_row4_any(a.head, out, p, first + r, NOUT, limit, u, fill_end);
+        }
+    }
+}
+
 }  // namespace sp
 
 using namespace sp;
@@ -231,8 +343,34 @@ static const void* pick_ensemble_kernel(int kg, bool exact, bool action) {
                                                                          : pick_ensemble_kernel_kg<16>(exact, action);
 }
 
+template <int KG, int MODE>
+static const void* pick_layer_kernel_kg(bool exact) {
+    return exact ? (const void*)ensemble_layer_kernel<KG, true, MODE> : (const void*)ensemble_layer_kernel<KG, false, MODE>;
+}
+template <int MODE>
+static const void* pick_layer_kernel(int kg, bool exact) {
+    return kg == 4 ? pick_layer_kernel_kg<4, MODE>(exact) : kg == 8 ? pick_layer_kernel_kg<8, MODE>(exact)
+         : kg == 16 ? pick_layer_kernel_kg<16, MODE>(exact) : pick_layer_kernel_kg<32, MODE>(exact);
+}
+
+// One workgroup (4 waves, one per SIMD) per compute unit while the members leave room for that: a wave then keeps its
+// member's weights for all its tiles.
+static int ensemble_launch(const void* kernel, EnsembleArgs& a, hipStream_t stream, const char* what) {
+    a.tiles = (a.batch + EN_ROWS - 1) / EN_ROWS;
+    const long cus = device_cu_count();
+    long gx = (cus + a.members - 1) / a.members;
+    const long most = (a.tiles + 3) / 4;
+    if (gx > most) gx = most;
+    if (gx < 1) gx = 1;
+    void* args[] = {(void*)&a};
+    hipError_t err = hipLaunchKernel(kernel, dim3((unsigned)gx, (unsigned)a.members), dim3(EN_THREADS), args, 0, stream);
+    if (err != hipSuccess) return fail(SP_ERR_DEVICE, "%s: launch failed: %s", what, hipGetErrorString(err));
+    return check_launch(what);
+}
+
 // Reference role: the body of `graph_run_host model {ensemble}` (ml/layers.spi:336-344) for a graph of the shape
-// input -> matmul_ensemble -> relu -> matmul_ensemble -> head (game/leduc/model_cem.spi:55-63).
+// input -> matmul_ensemble -> relu -> matmul_ensemble -> head (game/leduc/model_cem.spi:55-63) or
+// input -> matmul_ensemble -> head (game/nl_hu_holdem/model_cem.spi:84-100).
 extern "C" int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layers, const void* const* weights,
                                        const int32_t* dims, int32_t members, const float* u, const sp_philox_t* philox,
                                        float* policy_out, int32_t* action_out, int64_t batch, int32_t head,
@@ -242,24 +380,26 @@ extern "C" int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layer
     SP_OPTIONAL_PTR(u); SP_OPTIONAL_PTR(action_out);
     if (weights == nullptr || dims == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: weights/dims is NULL");
     if (dtype != SP_F32) return fail(SP_ERR_DTYPE, "sp_mlp_forward_ensemble: dtype must be f32");
-    if (n_layers != 2) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: two layers, got %d", n_layers);
+    if (n_layers != 1 && n_layers != 2) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: one or two layers, got %d", n_layers);
     if (members <= 0 || members > 65535) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: members must be in [1, 65535]");
     if (batch <= 0 || batch > (1ll << 40) / members) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: batch must be positive (and members x batch below 2^40)");
     if (head < SP_HEAD_NONE || head > SP_HEAD_SOFTMAX_RM) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: unknown head %d", head);
     if (action_out != nullptr && u == nullptr && philox == nullptr)
         return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: action requested but u and philox are NULL");
     if (u != nullptr && philox != nullptr) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: at most one of u and philox may be given");
-    const int k0 = dims[0], hidden = dims[1], n = dims[2];
-    if (k0 < 8 || k0 % 8 != 0 || k0 > 128)
-        return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: input width %d must be a multiple of 8 in [8, 128]", k0);
-    if (hidden != EN_HIDDEN) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: hidden width must be %d, got %d", EN_HIDDEN, hidden);
+    const int k0 = dims[0], n = dims[n_layers];
+    const int k_max = n_layers == 2 ? 128 : 256;
+    if (k0 < 8 || k0 % 8 != 0 || k0 > k_max)
+        return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: input width %d must be a multiple of 8 in [8, %d]", k0, k_max);
+    if (n_layers == 2 && dims[1] != EN_HIDDEN)
+        return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: hidden width must be %d, got %d", EN_HIDDEN, dims[1]);
     if (n <= 0 || n > MLP_MAX_OUT) return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: output width %d must be in [1, %d]", n, MLP_MAX_OUT);
     if (mask_size < 0 || mask_size > n) return fail(SP_ERR_ARG, "sp_mlp_forward_ensemble: mask_size must be in [0, %d], got %d", n, mask_size);
     // a masked head gives probability zero to the columns past the mask: only the valid ones are computed
     const int nout = head != SP_HEAD_NONE && mask_size > 0 ? mask_size : n;
     if (nout > EN_MAX_OUT)
         return fail(SP_ERR_SHAPE, "sp_mlp_forward_ensemble: at most 4 computed outputs (the head's width, or its mask), got %d", nout);
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < n_layers; ++i) {
         if (weights[i] == nullptr) return fail(SP_ERR_NULL, "sp_mlp_forward_ensemble: weights[%d] is NULL", i);
         if (!aligned16(weights[i])) return fail(SP_ERR_ALIGN, "sp_mlp_forward_ensemble: weights[%d] is not 16-byte aligned", i);
     }
@@ -271,23 +411,39 @@ extern "C" int sp_mlp_forward_ensemble(int dtype, const void* x, int32_t n_layer
     if (rc != SP_OK) return rc;
     rc = require_gfx950(__func__);
     if (rc != SP_OK) return rc;
-    a.x = (const float*)x; a.w1 = (const float*)weights[0]; a.w2 = (const float*)weights[1]; a.u = u;
+    a.x = (const float*)x; a.w1 = (const float*)weights[0]; a.w2 = n_layers == 2 ? (const float*)weights[1] : nullptr; a.u = u;
     a.policy = policy_out; a.action = action_out; a.batch = batch; a.members = members; a.k0 = k0; a.n = n; a.nout = nout;
     a.head = head; a.mask_size = mask_size;
-    a.tiles = (batch + EN_ROWS - 1) / EN_ROWS;
-    // one workgroup (4 waves, one per SIMD) per compute unit while the members leave room for that: a wave then keeps
-    // its member's weights for all its tiles
-    const long cus = device_cu_count();
-    long gx = (cus + members - 1) / members;
-    const long most = (a.tiles + 3) / 4;
-    if (gx > most) gx = most;
-    if (gx < 1) gx = 1;
-    const int kg = k0 <= 32 ? 4 : k0 <= 64 ? 8 : 16;
-    const void* kernel = pick_ensemble_kernel(kg, k0 == 8 * kg, action_out != nullptr);
-    void* args[] = {(void*)&a};
-    hipError_t err = hipLaunchKernel(kernel, dim3((unsigned)gx, (unsigned)members), dim3(EN_THREADS), args, 0, (hipStream_t)stream);
-    if (err != hipSuccess) return fail(SP_ERR_DEVICE, "sp_mlp_forward_ensemble: launch failed: %s", hipGetErrorString(err));
-    return check_launch(__func__);
+    const int kg = k0 <= 32 ? 4 : k0 <= 64 ? 8 : k0 <= 128 ? 16 : 32;
+    const void* kernel = n_layers == 2 ? pick_ensemble_kernel(kg, k0 == 8 * kg, action_out != nullptr)
+                       : action_out != nullptr ? pick_layer_kernel<1>(kg, k0 == 8 * kg) : pick_layer_kernel<0>(kg, k0 == 8 * kg);
+    return ensemble_launch(kernel, a, (hipStream_t)stream, __func__);
+}
+
+// Reference role: `graph_run_host model {ensemble}` for input -> matmul_ensemble -> binarize' (game/leduc/model_cfr.spi:56-61,
+// game/nl_hu_holdem/model_cfr.spi:82-88; ml/layers.spi:439-446, ml/primitives.spi:817-821).
+extern "C" int sp_ensemble_binarize(int dtype, const void* x, const void* weights, uint32_t* out, int32_t members,
+                                    int64_t batch, int32_t k0, int32_t n, uint32_t modulo, void* stream) {
+    SP_REQUIRE_PTR(x);
+    SP_REQUIRE_PTR(weights);
+    SP_REQUIRE_PTR(out);
+    if (dtype != SP_F32) return fail(SP_ERR_DTYPE, "sp_ensemble_binarize: dtype must be f32");
+    if (members <= 0 || members > 65535) return fail(SP_ERR_SHAPE, "sp_ensemble_binarize: members must be in [1, 65535]");
+    if (batch <= 0 || batch > (1ll << 40) / members) return fail(SP_ERR_SHAPE, "sp_ensemble_binarize: batch must be positive (and members x batch below 2^40)");
+    if (k0 < 8 || k0 % 8 != 0 || k0 > 256)
+        return fail(SP_ERR_SHAPE, "sp_ensemble_binarize: input width %d must be a multiple of 8 in [8, 256]", k0);
+    if (n <= 0) return fail(SP_ERR_SHAPE, "sp_ensemble_binarize: output width must be positive");
+    if (modulo == 0) return fail(SP_ERR_ARG, "sp_ensemble_binarize: modulo must be positive");
+    if (!aligned16(x) || !aligned16(weights)) return fail(SP_ERR_ALIGN, "sp_ensemble_binarize: x / weights not 16-byte aligned");
+    int rc = require_gfx950(__func__);
+    if (rc != SP_OK) return rc;
+    EnsembleArgs a{};
+    a.ph.philox_mode = -1;
+    a.x = (const float*)x; a.w1 = (const float*)weights; a.batch = batch; a.members = members; a.k0 = k0; a.n = n;
+    a.nout = n < 32 ? n : 32;          // the device's 32-bit shift drops the columns from 32 on
+    a.words = out; a.modulo = modulo;
+    const int kg = k0 <= 32 ? 4 : k0 <= 64 ? 8 : k0 <= 128 ? 16 : 32;
+    return ensemble_launch(pick_layer_kernel<2>(kg, k0 == 8 * kg), a, (hipStream_t)stream, __func__);
 }
 
 namespace {

@@ -88,6 +88,7 @@ SIGNATURES = {
                                         C.POINTER(PhiloxConfig), _P, _P, _P, _I64, _I32, _I32, _P]),
     "sp_mlp_forward_ensemble": (C.c_int, [C.c_int, _P, _I32, C.POINTER(_P), C.POINTER(C.c_int32), _I32, _P,
                                           C.POINTER(PhiloxConfig), _P, _P, _I64, _I32, _I32, _P]),
+    "sp_ensemble_binarize": (C.c_int, [C.c_int, _P, _P, _P, _I32, _I64, _I32, _I32, _U32, _P]),
 }
 
 
@@ -108,7 +109,7 @@ LAUNCHES = frozenset(("sp_gemm_abt", "sp_gemm_abt_batched", "sp_row_ops", "sp_ro
                       "sp_row_sample", "sp_philox_uniforms", "sp_row_get_prob", "sp_cem_resample", "sp_cem_resample_philox",
                       "sp_row_reduce_f32", "sp_cem_update_mask",
                       "sp_row_binarize", "sp_map_f32", "sp_reduce_sum", "sp_reduce", "sp_row_l1_normalize", "sp_reduce_sum_static", "sp_transpose_inner_b32", "sp_mlp_forward", "sp_mlp_pack_weights",
-                      "sp_mlp_forward_packed", "sp_mlp_forward_ensemble"))
+                      "sp_mlp_forward_packed", "sp_mlp_forward_ensemble", "sp_ensemble_binarize"))
 
 
 class Tape:

@@ -121,34 +121,52 @@ def mlp_forward(x, weights, biases=None, head="softmax_regret_matching", u=None,
 
 def mlp_forward_ensemble(x, weights, head="regret_matching", u=None, mask_size=0, policy_out=None, action_out=None,
                          rng=None):
-    """policy[, action] of every member of an ensemble of two-layer f32 stacks on one shared input, one launch:
-    policy[e] = head(relu(x . weights[0][e]^T) . weights[1][e]^T).
+    """policy[, action] of every member of an ensemble of one- or two-layer f32 stacks on one shared input, one launch:
+    policy[e] = head(relu(x . weights[0][e]^T) . weights[1][e]^T), or head(x . weights[0][e]^T) for a single layer.
 
-    x: (batch, in) f32, in a multiple of 8 up to 128; weights[0]: (E, 64, in), weights[1]: (E, out, 64) f32 (the
-    tensors of `matmul_ensemble`, ml/layers.spi:468-479); head and mask_size as for mlp_forward, with at most 4
-    computed outputs (out, or mask_size).  u: (E, batch) uniforms or rng: a Philox stream over the E * batch stacked
-    rows (member_rows = batch) for an action per member and row; without either only the policy (E, batch, out) is
-    computed -- the graph of the reference's Leduc policy, game/leduc/model_cem.spi:55-63."""
-    if len(weights) != 2:
-        raise ValueError("two weight tensors (E, 64, in) and (E, out, 64) expected")
-    w1, w2 = weights
-    if x.dtype != torch.float32 or w1.dtype != torch.float32 or w2.dtype != torch.float32:
+    x: (batch, in) f32; two layers: weights[0]: (E, 64, in), weights[1]: (E, out, 64), in a multiple of 8 up to 128;
+    one layer: weights[0]: (E, out, in), in a multiple of 8 up to 256 (the tensors of `matmul_ensemble`,
+    ml/layers.spi:468-479); head and mask_size as for mlp_forward, with at most 4 computed outputs (out, or mask_size).
+    u: (E, batch) uniforms or rng: a Philox stream over the E * batch stacked rows (member_rows = batch) for an action
+    per member and row; without either only the policy (E, batch, out) is computed -- the graphs of the reference's CEM
+    policies, game/leduc/model_cem.spi:55-63 and game/nl_hu_holdem/model_cem.spi:84-100."""
+    n = len(weights)
+    if n not in (1, 2):
+        raise ValueError("one weight tensor (E, out, in), or two: (E, 64, in) and (E, out, 64)")
+    if x.dtype != torch.float32 or any(w.dtype != torch.float32 for w in weights):
         raise TypeError("x and the weights must be f32")
-    members, batch = w1.shape[0], x.shape[0]
-    assert w2.shape[0] == members, "both layers need one matrix per member"
-    assert w1.shape[2] == x.shape[1] and w2.shape[2] == w1.shape[1], "The K dimension of the A and B tensors must match."
-    dims = [x.shape[1], w1.shape[1], w2.shape[1]]
+    members, batch = weights[0].shape[0], x.shape[0]
+    assert all(w.shape[0] == members for w in weights), "every layer needs one matrix per member"
+    dims = [x.shape[1]] + [w.shape[1] for w in weights]
+    for i, w in enumerate(weights):
+        assert w.shape[2] == dims[i], "The K dimension of the A and B tensors must match."
     policy = policy_out if policy_out is not None else \
         torch.empty((members, batch, dims[-1]), dtype=torch.float32, device=x.device)
     action = action_out
     if action is None and (u is not None or rng is not None):
         action = torch.empty((members, batch), dtype=torch.int32, device=x.device)
-    wp = (C.c_void_p * 2)(ptr(w1, name="weights[0]"), ptr(w2, name="weights[1]"))
-    dp = (C.c_int32 * 3)(*dims)
-    check(lib.sp_mlp_forward_ensemble(_lib.SP_F32, ptr(x, name="x"), 2, wp, dp, members, ptr(u, torch.float32, "u"),
+    wp = (C.c_void_p * n)(*[ptr(w, name="weights[%d]" % i) for i, w in enumerate(weights)])
+    dp = (C.c_int32 * (n + 1))(*dims)
+    check(lib.sp_mlp_forward_ensemble(_lib.SP_F32, ptr(x, name="x"), n, wp, dp, members, ptr(u, torch.float32, "u"),
                                       C.byref(rng) if rng is not None else None, ptr(policy, torch.float32, "policy_out"),
                                       ptr(action, torch.int32, "action_out"), batch, HEADS[head], mask_size, stream_ptr()))
     return (policy, action) if action is not None else policy
+
+
+def ensemble_binarize(x, weights, modulo, out=None):
+    """out[e][r] = binarize(x[r] . weights[e]^T) mod modulo for every member of an ensemble layer, one launch, the
+    product never written: the graph of the reference's CFR models (`matmul_ensemble -> binarize'`,
+    game/leduc/model_cfr.spi:56-61; ml/primitives.spi:817-821).  x: (batch, in) f32, in a multiple of 8 up to 256;
+    weights: (E, out, in) f32; out: (E, batch) i32 holding the u32 words."""
+    if x.dtype != torch.float32 or weights.dtype != torch.float32:
+        raise TypeError("x and the weights must be f32")
+    members, n, k0 = weights.shape
+    assert k0 == x.shape[1], "The K dimension of the A and B tensors must match."
+    if out is None:
+        out = torch.empty((members, x.shape[0]), dtype=torch.int32, device=x.device)
+    check(lib.sp_ensemble_binarize(_lib.SP_F32, ptr(x, name="x"), ptr(weights, name="weights"), ptr(out, torch.int32, "out"),
+                                   members, x.shape[0], k0, n, modulo, stream_ptr()))
+    return out
 
 
 # ----------------------------------------------------------------------------------------------
@@ -813,8 +831,10 @@ _ENSEMBLE_HEADS = {"softmax": "softmax", "masked_softmax": "softmax", "regret_ma
 
 
 def _fused_ensemble_plan(model, key):
-    """`input -> matmul_ensemble -> relu -> matmul_ensemble -> head` over f32 tensors with the members' outputs stacked
-    under `apply key` (the Leduc policy of game/leduc/model_cem.spi:55-63) in the shapes sp_mlp_forward_ensemble takes:
+    """`input -> matmul_ensemble [-> relu -> matmul_ensemble] -> head` over f32 tensors with the members' outputs stacked
+    under `apply key` -- the graphs of the reference's agents (game/leduc/model_cem.spi:55-63,
+    game/nl_hu_holdem/model_cem.spi:84-100: a policy head; game/leduc/model_cfr.spi:56-61,
+    game/nl_hu_holdem/model_cfr.spi:82-88: one layer and `binarize'`):
     (x node, [stacked weight nodes], stacked output node(s), top node) or None."""
     top = model.graph
 
@@ -830,7 +850,10 @@ def _fused_ensemble_plan(model, key):
     while isinstance(top, Pair) and passive(top.b):
         top = top.a
     sampling = isinstance(top, BlockRowMapReduce)
-    if not isinstance(top, (BlockRowMap, BlockRowMapReduce)) or top.f not in _ENSEMBLE_HEADS or top.out is None:
+    hashing = isinstance(top, BlockRowReduce) and top.f == "binarize"
+    if not hashing and (not isinstance(top, (BlockRowMap, BlockRowMapReduce)) or top.f not in _ENSEMBLE_HEADS):
+        return None
+    if top.out is None:
         return None
 
     def stacked(k):   # `apply key t` -> t
@@ -851,15 +874,16 @@ def _fused_ensemble_plan(model, key):
         outs = (stacked(top.out),)
     if any(o is None for o in outs):
         return None
-    second = top.a
-    if not isinstance(second, BlockMatmul):
+    last = top.a
+    if not isinstance(last, BlockMatmul):
         return None
-    hidden = second.a
-    if not (isinstance(hidden, BlockMap) and hidden.f == "relu" and hidden.out is None and isinstance(hidden.a, BlockMatmul)):
-        return None
-    first = hidden.a
-    weights = [stacked(first.b), stacked(second.b)]
-    x = first.a
+    weights = [stacked(last.b)]
+    x = last.a
+    if isinstance(x, BlockMap):
+        if hashing or not (x.f == "relu" and x.out is None and isinstance(x.a, BlockMatmul)):
+            return None
+        weights.insert(0, stacked(x.a.b))
+        x = x.a.a
     while isinstance(x, KeyGraph):
         x = x.x
     if any(w is None for w in weights) or not isinstance(x, Layer):
@@ -868,21 +892,31 @@ def _fused_ensemble_plan(model, key):
 
 
 def _run_fused_ensemble(model, key, count, ls):
-    """One sp_mlp_forward_ensemble launch in place of the batched pass, where the graph is of that shape."""
+    """One sp_mlp_forward_ensemble / sp_ensemble_binarize launch in place of the batched pass, where the graph is of
+    that shape."""
     plan = _fused_ensemble_plan(model, key)
     if plan is None:
         return False
     x_node, w_nodes, out_nodes, top = plan
     tensor = lambda node: graph_extract(Model(node, model.dims, model.data))
-    x, (w1, w2) = tensor(x_node), [tensor(w) for w in w_nodes]
-    probs = tensor(out_nodes[0])
-    if x.dim() != 3 or w1.dim() != 3 or w2.dim() != 3 or any(t.dtype != torch.float32 for t in (x, w1, w2, probs)):
+    x, ws = tensor(x_node), [tensor(w) for w in w_nodes]
+    first_out = tensor(out_nodes[0])
+    if x.dim() != 3 or any(w.dim() != 3 or w.dtype != torch.float32 or w.shape[0] != count for w in ws) or x.dtype != torch.float32:
         return False
     q, w, k0 = x.shape
-    cols = w2.shape[1]
+    cols = ws[-1].shape[1]
+    if ws[0].shape[2] != k0 or k0 % 8 != 0 or k0 < 8:
+        return False
+    if isinstance(top, BlockRowReduce):           # binarize
+        if len(ws) != 1 or k0 > 256 or first_out.shape != (count, q, w) or first_out.dtype != torch.int32 or top.arg <= 0:
+            return False
+        ensemble_binarize(_flat(x), ws[0], top.arg, first_out.reshape(count, q * w))
+        return True
+    probs = first_out
     computed = top.size or cols
-    if not (w1.shape[0] == w2.shape[0] == count and w1.shape[1] == w2.shape[2] == 64 and w1.shape[2] == k0 and
-            k0 % 8 == 0 and 8 <= k0 <= 128 and cols <= 64 and computed <= 4 and probs.shape == (count, q, w, cols)):
+    if len(ws) == 2 and not (ws[0].shape[1] == ws[1].shape[2] == 64 and k0 <= 128):
+        return False
+    if not (k0 <= 256 and cols <= 64 and computed <= 4 and probs.dtype == torch.float32 and probs.shape == (count, q, w, cols)):
         return False
     action, rng = None, None
     if len(out_nodes) == 2:
@@ -894,7 +928,7 @@ def _run_fused_ensemble(model, key, count, ls):
         rng = _prim.philox(_lib.PHILOX_LAYER, seed=ls.seed, threads_per_block=THREADS_PER_BLOCK, blocks_per_grid=q,
                            rows_per_block=w, offset=ls.draws, member_rows=q * w, member_draws=draws)
         ls.draws += draws
-    mlp_forward_ensemble(_flat(x), (w1, w2), _ENSEMBLE_HEADS[top.f], None, top.size, probs.reshape(count, q * w, cols),
+    mlp_forward_ensemble(_flat(x), ws, _ENSEMBLE_HEADS[top.f], None, top.size, probs.reshape(count, q * w, cols),
                          action.reshape(count, q * w) if action is not None else None, rng)
     return True
 

@@ -349,3 +349,43 @@ def test_leduc_policy_graph_runs_as_one_launch(L, sampling):
                 assert (got_i[e].reshape(-1) == orow.discrete_sampling(got_p[e].reshape(-1, 64), u)).all()
     tape = m._tapes[(L._prim.CONSTANT_SEED, True, True, (("ensemble", ensemble),))][1]
     assert len(tape.calls) == 1 and tape.calls[0][0].__name__ == "sp_mlp_forward_ensemble"
+
+
+def test_cfr_and_holdem_graphs_run_as_one_launch(L):
+    """The other model graphs of the reference's agents: `input -> matmul_ensemble (E, 128, 128) -> binarize' 4096`
+    (game/leduc/model_cfr.spi:56-61, game/nl_hu_holdem/model_cfr.spi:82-88) and `input -> matmul_ensemble_with_adjoint
+    (E, 128, 64) -> masked_regret_matching' 3` (game/nl_hu_holdem/model_cem.spi:84-100), each paired with a table that
+    computes nothing: one launch per run, results as the batched node-by-node pass gives them."""
+    announce("layers cfr / holdem cem graphs")
+    ensemble, w = 4, 256
+    world = L.apply("ensemble", L.input("output_world_id", (ensemble, Q, w), "int"))
+    g = L.pair(L.binarize_(1 << 12, world, L.pipe(L.input("input", (Q, w, 128)), L.matmul_ensemble((ensemble, 128, 128)))),
+               L.input("cfr_table", (ensemble, 8, 4)))
+    m = L.create_model(g)
+    L.pass_init(m)
+    fill(L.key_extract(m, "input"), np.random.default_rng(6))
+    L.graph_run_host(m, {"ensemble": ensemble}, fuse=False)
+    want = host(L.key_extract(m, "output_world_id")).copy()
+    L.key_extract(m, "output_world_id").fill_(-1)
+    for _ in range(2):
+        L.graph_run_host(m, {"ensemble": ensemble})
+        got = host(L.key_extract(m, "output_world_id"))
+        assert (got != want).mean() < 1e-3 and (got >= 0).all() and (got < 4096).all()   # (signs of outputs next to zero)
+    tape = m._tapes[(L._prim.CONSTANT_SEED, True, True, (("ensemble", ensemble),))][1]
+    assert len(tape.calls) == 1 and tape.calls[0][0].__name__ == "sp_ensemble_binarize"
+
+    probs = L.apply("ensemble", L.input("output_probs", (ensemble, Q, w, 64)))
+    g = L.pair(L.masked_regret_matching_(3, probs, L.pipe(L.input("input", (Q, w, 128)),
+                                                           L.matmul_ensemble_with_adjoint((ensemble, 128, 64)))),
+               L.input("cem_table", (ensemble, 16, 4)))
+    m = L.create_model(g)
+    L.pass_init(m)
+    fill(L.key_extract(m, "input"), np.random.default_rng(7))
+    L.graph_run_host(m, {"ensemble": ensemble}, fuse=False)
+    want_p = host(L.key_extract(m, "output_probs")).copy()
+    L.key_extract(m, "output_probs").fill_(7)
+    L.graph_run_host(m, {"ensemble": ensemble})
+    got_p = host(L.key_extract(m, "output_probs"))
+    assert ogemm.rel_frobenius(got_p.reshape(-1, 64), want_p.reshape(-1, 64)) < 1e-5 and (got_p[..., 3:] == 0).all()
+    tape = m._tapes[(L._prim.CONSTANT_SEED, True, True, (("ensemble", ensemble),))][1]
+    assert len(tape.calls) == 1 and tape.calls[0][0].__name__ == "sp_mlp_forward_ensemble"

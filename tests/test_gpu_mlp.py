@@ -433,3 +433,61 @@ def test_ensemble_rejects_what_it_does_not_take(LY):
         LY.mlp_forward_ensemble(x, (torch.zeros((2, 32, 128), dtype=torch.float32, device="cuda"),
                                     torch.zeros((2, 4, 32), dtype=torch.float32, device="cuda")), "softmax")
     assert err.value.code == -2
+
+
+@pytest.mark.parametrize("members,batch,k0,n,head,mask,sample", [
+    (4, 6144, 128, 64, "regret_matching", 3, None),     # the reference's hold'em CEM policy: one layer, 3 valid of 64 columns
+    (6, 1000, 256, 64, "softmax", 4, "u"),              # the widest input, a ragged last tile, sampling
+    (3, 333, 40, 3, "softmax_regret_matching", 0, "u"),  # input width not a multiple of 32, a dense 3-wide head
+])
+def test_single_layer_ensemble_forward(LY, members, batch, k0, n, head, mask, sample):
+    """sp_mlp_forward_ensemble with ONE layer per member (policy[e] = head(x . W[e]^T), only the head's valid columns
+    computed) against the oracle's forward of each member (f32 bar 1e-5), zeros behind the mask, actions exact given
+    the kernel's policy."""
+    announce("ensemble single layer members=%d batch=%d k0=%d n=%d head=%s mask=%d" % (members, batch, k0, n, head, mask))
+    rng = np.random.default_rng(members + batch + k0)
+    x = rng.standard_normal((batch, k0), dtype=np.float32)
+    w = rng.standard_normal((members, n, k0), dtype=np.float32) * np.float32(1 / np.sqrt(k0))
+    u = (1 - rng.random((members, batch), dtype=np.float32)).astype(np.float32) if sample else None
+    out = LY.mlp_forward_ensemble(dev(x), (dev(w),), head, dev(u) if sample else None, mask)
+    policy, action = (host(out[0]), host(out[1])) if sample else (host(out), None)
+    for e in range(members):
+        want, _, _ = olayers.mlp_forward(x, [w[e]], None, HEAD_CODE[head], None, None, mask or None)
+        assert ogemm.rel_frobenius(policy[e], want) < 1e-5, e
+        if mask:
+            assert (policy[e][:, mask:] == 0).all()
+        if sample:
+            assert (action[e] == orow.discrete_sampling(policy[e], u[e])).all(), e
+
+
+@pytest.mark.parametrize("members,batch,k0,n,modulo", [
+    (4, 6144, 128, 128, 1 << 12),     # the reference's CFR models: 128 outputs hashed into 4096 worlds
+    (5, 1001, 256, 20, 1000003),      # fewer than 32 columns, a modulus that is not a power of two, a ragged last tile
+    (3, 64, 24, 40, 1 << 31),         # every one of the 32 counted bits kept
+])
+def test_ensemble_binarize(LY, members, batch, k0, n, modulo):
+    """sp_ensemble_binarize (one ensemble layer + the hash head, the product never written) against the oracle's
+    binarize of the oracle's product.  A bit can only differ where an output is so close to zero that the order of the
+    sum decides its sign: such entries are left out of the comparison (and are counted: there must be next to none)."""
+    from ml import primitives
+    announce("ensemble binarize members=%d batch=%d k0=%d n=%d modulo=%d" % (members, batch, k0, n, modulo))
+    rng = np.random.default_rng(members * 7 + batch + n)
+    x = rng.standard_normal((batch, k0), dtype=np.float32)
+    w = rng.standard_normal((members, n, k0), dtype=np.float32)
+    got = host(LY.ensemble_binarize(dev(x), dev(w), modulo)).view(np.uint32)
+    assert got.shape == (members, batch)
+    close = 0
+    for e in range(members):
+        y = ogemm.gemm_abt(x, w[e])
+        want = orow.binarize(y, modulo)
+        sure = (np.abs(y[:, :32]) > 1e-4).all(axis=1)       # rows whose counted outputs are all clear of zero
+        close += int((~sure).sum())
+        assert (got[e][sure] == want[sure]).all(), e
+        # and exactly the node-by-node result on the same product computed by the library's own GEMM
+    assert close < 0.02 * members * batch
+    # the row kernel on the library's own product gives the same words wherever the signs are not in question
+    from ml import matmul
+    y0 = matmul.matmul_abt(dev(x), dev(w[0]))
+    node = host(primitives.binarize(y0, modulo)).view(np.uint32)
+    sure0 = (np.abs(host(y0)[:, :32]) > 1e-4).all(axis=1)
+    assert (node[sure0] == got[0][sure0]).all()
