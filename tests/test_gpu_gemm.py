@@ -436,7 +436,7 @@ def test_clock_sample_gives_the_shader_clock():
     mhz = (s[1, both, 0] - s[0, both, 0]) / (s[1, both, 1] - s[0, both, 1]) * 100.0
     med = np.median(mhz)
     assert 500 < med < 2600
-    assert (np.abs(mhz - med) < 0.05 * med).mean() > 0.9      # (the XCDs settle a few percent apart under a power limit)
+    assert (np.abs(mhz - med) < 0.10 * med).mean() > 0.9      # (the XCDs settle a few percent apart under a power limit)
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
