@@ -17,9 +17,9 @@
 // little for the matrix pipe (a 32 x 32 tile for 3 useful rows costs a quarter of layer 1): every lane multiplies the
 // 32 features of its row that it holds (after the relu) with the matching weights -- fused multiply-adds on the
 // vector ALU -- and the two halves of a row are added across the lane halves.
-// Sums therefore add up in another order than a row-by-row dot product; f32 throughout.  The lanes with g = 0 run the
-// head for their row; the zeros behind the valid columns of a masked head are written by the whole wave, 16 bytes per
-// lane.
+// Sums therefore add up in another order than a row-by-row dot product; f32 throughout.  Tiles go through in pairs: the lanes
+// with g = 0 run the head for their row of the first tile, the lanes with g = 1 for the second; the zeros behind the
+// valid columns of a masked head are written by the whole wave, 16 bytes per lane.
 #include "mlp_common.h"
 
 #pragma clang fp contract(off)
@@ -47,16 +47,6 @@ struct EnsembleArgs {
     PhiloxStream ph;
 };
 
-#ifdef SP_EN_TIMELINE
-#ifndef SP_EN_TL_FIRST
-#define SP_EN_TL_FIRST 4
-#endif
-__device__ unsigned long long sp_en_timeline[256 * 8 * 8];
-#define SP_EN_STAMP(K) do { if (lane == 0 && wave == 0 && it >= SP_EN_TL_FIRST && it < SP_EN_TL_FIRST + 8) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + (it - SP_EN_TL_FIRST)) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define SP_EN_STAMP(K) do {} while (0)
-#endif
-
 // KG: 8-wide groups of the input width the kernel is unrolled for; EXACT: K0 = 8 KG (else K0 < 8 KG and the groups
 // past K0 are zeros); ACTION: an action per row is wanted (a uniform per row, from a tensor or a Philox stream)
 template <int KG, bool EXACT, bool ACTION>
@@ -70,12 +60,6 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
     const int groups = K0 >> 3;
     const long batch = a.batch, tiles = a.tiles;
     const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-#ifdef SP_EN_TIMELINE
-#define SP_EN_MARK(K) do { if (lane == 0 && wave == 0) sp_en_timeline[((blockIdx.y * gridDim.x + blockIdx.x) * 8 + 0) * 8 + (K)] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define SP_EN_MARK(K) do {} while (0)
-#endif
-    SP_EN_MARK(5);
 
     // ---- the member's weights, once ----
     f32x4 w1v[2][KG];             // [feature tile][j]: W1[e][32 t + r][8 j + 4 g .. + 3]
@@ -127,51 +111,41 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
     const bool wave_fill = N > NOUT && (N & 3) == 0;
     const int s4 = N >> 2, c0 = (NOUT + 3) >> 2;
 
-    // the head of a tile: lane (r, 0) holds the outputs of row r; the zeros behind the valid columns of a masked head
-    // are written by the whole wave, 16 bytes per lane: lane l takes pieces l, l + 64, ... of the tile's 32 s4 pieces.
-    // 64-wide rows (16 pieces): a lane's pieces are 1 KiB apart, all in one column -- eight stores in a straight line;
-    // other widths walk (row and column of a piece advance by fixed steps: no division inside the walk).
+    // The zeros behind the valid columns of a masked head are written by the whole wave, 16 bytes per lane: lane l takes
+    // pieces l, l + 64, ... of a tile's 32 s4 pieces.  64-wide rows (16 pieces): a lane's pieces are 1 KiB apart, all in
+    // one column -- eight stores in a straight line; other widths walk (row and column of a piece advance by fixed
+    // steps: no division inside the walk).
     const int fill_r0 = wave_fill ? lane / s4 : 0, fill_c0 = wave_fill ? lane - fill_r0 * s4 : 0;
     const int fill_dr = wave_fill ? 64 / s4 : 0, fill_dc = wave_fill ? 64 - fill_dr * s4 : 0;
-    auto finish = [&](long t, const float (&p)[4], float u) {
+    auto fill_zeros = [&](long t) {
         const long row0 = t * EN_ROWS;
-        const long first = (long)e * batch + row0;              // row of the stacked (members x batch) outputs
-        int fill_end = 1 << 30;
-        if (wave_fill) {
-            fill_end = 4 * c0;
-            float* block = a.policy + first * N;
-            const int rows_here = batch - row0 < EN_ROWS ? (int)(batch - row0) : EN_ROWS;
-            if (s4 == 16 && rows_here == EN_ROWS) {
-                if (fill_c0 >= c0) {
-                    f32x4* mine = reinterpret_cast<f32x4*>(block) + lane;
+        float* block = a.policy + ((long)e * batch + row0) * N;
+        const int rows_here = batch - row0 < EN_ROWS ? (int)(batch - row0) : EN_ROWS;
+        if (s4 == 16 && rows_here == EN_ROWS) {
+            if (fill_c0 >= c0) {
+                f32x4* mine = reinterpret_cast<f32x4*>(block) + lane;
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) mine[64 * k] = zero4;
-                }
-            } else {
-                int rr = fill_r0, c = fill_c0;
-                for (int idx = lane; idx < EN_ROWS * s4; idx += 64) {
-                    if (c >= c0 && rr < rows_here) *reinterpret_cast<f32x4*>(block + rr * N + 4 * c) = zero4;
-                    rr += fill_dr;
-                    c += fill_dc;
-                    if (c >= s4) {
-                        c -= s4;
-                        ++rr;
-                    }
+                for (int k = 0; k < 8; ++k) mine[64 * k] = zero4;
+            }
+        } else {
+            int rr = fill_r0, c = fill_c0;
+            for (int idx = lane; idx < EN_ROWS * s4; idx += 64) {
+                if (c >= c0 && rr < rows_here) *reinterpret_cast<f32x4*>(block + rr * N + 4 * c) = zero4;
+                rr += fill_dr;
+                c += fill_dc;
+                if (c >= s4) {
+                    c -= s4;
+                    ++rr;
                 }
             }
         }
-        if (g == 0 && row0 + r < batch) head_row4_any(a.head, out, p, first + r, NOUT, limit, u, fill_end);
     };
 
-    int it = -1;
-    SP_EN_MARK(6);
-    for (; tile < tiles; tile += stride) {
-        ++it;
-        SP_EN_STAMP(0);
+    // Both layers of one tile; the outputs of row r end up in BOTH lanes (r, 0) and (r, 1).
+    auto forward = [&](long next_tile, float (&p)[4]) {
         // ---- layer 1: (64 features x 32 rows) += W1 . x^T, two K-values per step.  A register of inputs is asked for
         //      the NEXT tile's values as soon as this tile's MFMAs have read it: they arrive a whole tile ahead. ----
-        const long next = tile + stride;
-        const float* const xr_next = x_row(next < tiles ? next : tile);
+        const float* const xr_next = x_row(next_tile);
         f32x16 acc[2];
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -186,19 +160,11 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w1v[t][j][i], xv[j][i], acc[t], 0, 0, 0);
             xv[j] = load_piece(xr_next, j);
         }
-        SP_EN_STAMP(1);
-        float u = 1.f;
-        if constexpr (ACTION) {
-            long row = tile * EN_ROWS + r;
-            row = (long)e * batch + (row < batch ? row : batch - 1);
-            u = a.u != nullptr ? a.u[row] : reference_row_uniform(a.ph, row);
-        }
-        SP_EN_STAMP(2);
-
         // ---- relu; layer 2: this lane's 32 features of its row against the matching weights, then the other half's ----
-        float p[4];
 #pragma unroll
         for (int o = 0; o < EN_MAX_OUT; ++o) {
+            p[o] = 0.f;
+            if (o >= NOUT) continue;                           // (uniform)
             float s0 = 0.f, s1 = 0.f;                          // (two chains: an FMA need not wait for the one before)
 #pragma unroll
             for (int t = 0; t < 2; ++t)
@@ -210,14 +176,39 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
             const float mine = s0 + s1;
             p[o] = mine + __shfl_xor(mine, 32);
         }
-        SP_EN_STAMP(3);
-        finish(tile, p, u);
-        SP_EN_STAMP(4);
+    };
+
+    // Tiles go through in pairs and the heads of a pair run together -- lanes (r, 0) finish row r of the first tile,
+    // lanes (r, 1) row r of the second: the head is a chain of dependent instructions that costs the same for 64 lanes
+    // as for 32, and vector-ALU work does not hide behind f32 MFMAs.
+    for (; tile < tiles; tile += 2 * stride) {
+        const long tile_b = tile + stride;
+        const bool has_b = tile_b < tiles;                      // (uniform)
+        float p[4] = {0.f, 0.f, 0.f, 0.f};                     // of this lane's row: the first tile's for g = 0, the second's for g = 1
+#pragma unroll 1
+        for (int half = 0; half < (has_b ? 2 : 1); ++half) {
+            const long after = tile + (half + 1) * stride;      // the tile whose inputs are requested meanwhile
+            float ph[4];
+            forward(after < tiles ? after : tile, ph);
+#pragma unroll
+            for (int n = 0; n < 4; ++n) p[n] = g == half ? ph[n] : p[n];
+        }
+        int fill_end = 1 << 30;
+        if (wave_fill) {
+            fill_end = 4 * c0;
+            fill_zeros(tile);
+            if (has_b) fill_zeros(tile_b);
+        }
+        const long my_tile = g == 0 ? tile : tile_b;
+        const long my_row = my_tile * EN_ROWS + r;
+        if ((g == 0 || has_b) && my_row < batch) {
+            const long grow = (long)e * batch + my_row;
+            float u = 1.f;
+            if constexpr (ACTION) u = a.u != nullptr ? a.u[grow] : reference_row_uniform(a.ph, grow);
+            head_row4_any(a.head, out, p, grow, NOUT, limit, u, fill_end);
+        }
     }
-    SP_EN_MARK(7);
 }
-#undef SP_EN_STAMP
-#undef SP_EN_MARK
 
 // ONE ensemble layer and its head: policy[e] = head(x . W[e]^T) for a head of at most 4 computed outputs, or
 // word[e][r] = (OR over j < 32 of (not (y[r][j] <= 0)) << j) mod modulo with y = x . W[e]^T -- the graphs of the
@@ -451,9 +442,3 @@ struct MlpEnsembleKernelNames {
     MlpEnsembleKernelNames() { register_kernel("mlp_forward_ensemble", (const void*)mlp_ensemble_kernel<16, true, false>, EN_THREADS); }
 } mlp_ensemble_kernel_names;
 }  // namespace
-
-#ifdef SP_EN_TIMELINE
-extern "C" int sp_debug_ensemble_timeline(unsigned long long* host_out) {
-    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(sp::sp_en_timeline), sizeof(unsigned long long) * 256 * 8 * 8);
-}
-#endif
