@@ -200,3 +200,36 @@ def test_packed_mlp_argument_errors(L):
     assert call(dd=dims(32, 256, 256, 256, 64)) == -6 and "16 outputs" in _err(L)     # wide head, no mask
     assert call(dd=dims(32, 256, 256, 256, 64), mask=3, logits=p) == -6               # wide masked head with logits
     assert call(mask=4) == -5
+
+
+def test_ensemble_argument_errors(L):
+    lib = L.lib
+    p = C.c_void_p(0x6000)
+    dims = lambda *d: (C.c_int32 * len(d))(*d)
+    w2 = (C.c_void_p * 2)(p, p)
+    call = lambda dtype=0, x=p, n=2, w=w2, dd=dims(128, 64, 64), members=4, u=None, pol=p, act=None, batch=64, head=2, mask=3: \
+        lib.sp_mlp_forward_ensemble(dtype, x, n, w, dd, members, u, None, pol, act, batch, head, mask, None)
+    assert call(dtype=1) == -4                                       # f32 only
+    assert call(x=None) == -1 and call(pol=None) == -1 and call(w=None) == -1
+    assert call(n=3) == -2 and "one or two layers" in _err(L)
+    assert call(dd=dims(128, 32, 64)) == -2 and "hidden width" in _err(L)
+    assert call(dd=dims(136, 64, 64)) == -2                         # two layers: inputs up to 128 wide
+    assert call(dd=dims(20, 64, 64)) == -2                          # a multiple of 8
+    assert call(mask=0) == -2 and "at most 4 computed outputs" in _err(L)
+    assert call(mask=65) == -5
+    assert call(members=0) == -2 and call(batch=0) == -2
+    assert call(act=p) == -1                                        # an action without uniforms
+    assert call(w=(C.c_void_p * 2)(p, None)) == -1
+    assert call(x=C.c_void_p(0x6004)) == -3
+    # one layer: inputs up to 256 wide, the same head limits
+    one = (C.c_void_p * 1)(p)
+    assert call(n=1, w=one, dd=dims(264, 64)) == -2
+    assert call(n=1, w=one, dd=dims(256, 64), mask=5) == -2
+    hash_call = lambda dtype=0, x=p, w=p, out=p, members=4, batch=64, k0=128, n=128, modulo=4096: \
+        lib.sp_ensemble_binarize(dtype, x, w, out, members, batch, k0, n, modulo, None)
+    assert hash_call(dtype=2) == -4
+    assert hash_call(x=None) == -1 and hash_call(w=None) == -1 and hash_call(out=None) == -1
+    assert hash_call(k0=260) == -2 and hash_call(k0=12) == -2 and hash_call(n=0) == -2
+    assert hash_call(modulo=0) == -5 and "modulo" in _err(L)
+    assert hash_call(members=70000) == -2
+    assert hash_call(w=C.c_void_p(0x6008)) == -3
