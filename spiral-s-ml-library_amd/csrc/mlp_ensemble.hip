@@ -159,6 +159,7 @@ __global__ __launch_bounds__(EN_THREADS) void mlp_ensemble_kernel(const Ensemble
                 for (int t = 0; t < 2; ++t)
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(w1v[t][j][i], xv[j][i], acc[t], 0, 0, 0);
             xv[j] = load_piece(xr_next, j);
+            __builtin_amdgcn_sched_barrier(0);      // (keeps every load behind the MFMAs that free its register)
         }
         // ---- relu; layer 2: this lane's 32 features of its row against the matching weights, then the other half's ----
 #pragma unroll
@@ -274,6 +275,8 @@ __global__ __launch_bounds__(EN_THREADS) void ensemble_layer_kernel(const Ensemb
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[j][i], xv[j][i], acc, 0, 0, 0);
             xv[j] = load_piece(xr_next, j);
+            __builtin_amdgcn_sched_barrier(0);      // (left alone, the scheduler sinks the loads to the end of the tile,
+                                                    //  and the next tile then starts by waiting for all of them)
         }
         const long row0 = tile * EN_ROWS;
         const long first = (long)e * batch + row0;              // row of the stacked (members x batch) outputs
