@@ -334,6 +334,8 @@ def main():
             nbytes = rows * cols * 4 * (3 if materialise else 1) + rows * 4 * 5
             res = {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(rows / (ev * 1e-3), 1),
                    "roofline": roofline_hbm(nbytes, ev), "seed": 8, "sigma": 2.0, "shader_clock_mhz": CLOCK["mhz"]}
+            assert (outs["argmax"].cpu().numpy() == orow.argmax(x)).all(), "bench row ops: argmax"
+            assert (outs["rowmax"].cpu().numpy() == x.max(axis=1)).all(), "bench row ops: row maximum"
             if materialise:
                 # what was timed is checked: argmax exact, the sampled index exact given the kernel's own running sums,
                 # and how many rows would sample another index under a left-to-right running sum of the same
@@ -375,6 +377,14 @@ def main():
                 fn = lambda: primitives.transpose_snd(xd, out=out)
                 nbytes = 2 * x.nbytes
             wall, ev = time_launches(fn, K, W)
+            got = out.cpu().numpy()
+            if kind == "map_relu":
+                assert (got == np.maximum(x, np.float32(0))).all(), "bench map: output differs from the oracle"
+            elif kind == "reduce_sum":
+                want = float(x.sum(dtype=np.float64))
+                assert abs(float(got[0]) - want) <= 1e-5 * float(np.abs(x).sum(dtype=np.float64)), "bench reduce: sum"
+            else:
+                assert (got == x.T).all(), "bench transpose: output differs from the oracle"
             return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "roofline": roofline_hbm(nbytes, ev), "seed": 9,
                     "shader_clock_mhz": CLOCK["mhz"]}
 
@@ -395,6 +405,10 @@ def main():
                 t.copy_(dev(olayers.weight_init(rng, t.shape[0], t.shape[1]), torch.float16))
             fn = lambda: layers.graph_run_host(m, static_weights=True)
             wall, ev = time_launches(fn, max(K, 200), W)
+            probs, acts = layers.graph_extract(m)
+            probs, acts = probs.cpu().numpy().reshape(batch, 64), acts.cpu().numpy().reshape(batch)
+            assert (probs[:, 3:] == 0).all() and np.abs(probs.sum(axis=1) - 1).max() < 1e-5, "bench graph: policy rows"
+            assert ((acts >= 0) & (acts < 3)).all() and (probs[np.arange(batch), acts] > 0).all(), "bench graph: actions"
             fl = 2.0 * batch * (32 * 256 + 256 * 256 + 256 * 256 + 256 * 64)
             return {"ms": round(ev, 5), "wall_ms": round(wall, 5), "rows_per_s": round(batch / (ev * 1e-3), 1),
                     "roofline": roofline_mfma(fl, ev, "f16"), "seed": 10,
