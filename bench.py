@@ -259,6 +259,7 @@ def main():
             ("gemm_bf16_65536x1024x512", lambda: gemm_case(5, 65536, 1024, 512, "bf16")[0]),
             ("gemm_bf16_65536x256x2048", lambda: gemm_case(6, 65536, 256, 2048, "bf16")[0]),
             ("gemm_bf16_65536x256x256_bias_relu", lambda: gemm_case(4, 65536, 256, 256, "bf16", bias_relu=True)[0]),
+            ("gemm_bf16_65536x1024x512_bias_relu", lambda: gemm_case(5, 65536, 1024, 512, "bf16", bias_relu=True)[0]),
         ]
 
         def mlp_case(packed=True, batches=1):
