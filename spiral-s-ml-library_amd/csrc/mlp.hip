@@ -1036,7 +1036,8 @@ extern "C" int sp_mlp_forward(int dtype, const void* x, int32_t n_layers, const 
         mask_size < dims[n_layers])
         a.nout = mask_size;
     if (h256 && mlp_resident_takes(n_layers, dims, a.nout) &&
-        (batch + 63) / 64 >= (long)SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR * cus) {
+        (batch + 63) / 64 >= (long)(mlp_pipe_takes(n_layers, dims, a.nout) ? SP_MLP_PIPE_MIN_TILES_ROWMAJOR
+                                                                           : SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR) * cus) {
         // many tiles per compute unit: the kernel that loads the weights once and keeps them in registers
         MlpResidentArgs r{};
         r.x = x; r.u = u; r.policy = policy_out; r.action = action_out; r.logits = logits_out;

@@ -75,12 +75,16 @@ int mlp_pipe_launch(int dtype, bool packed, MlpResidentArgs a, hipStream_t strea
 #define SP_MLP_RESIDENT_MIN_TILES_ROWMAJOR 8
 #endif
 
-// 64-row tiles per compute unit from which the pipelined kernel takes over from the resident one (for the stacks it
-// takes).  Measured, us per launch, resident / pipelined, packed weights: 98304 rows 26.1 / 24.6, 131072 33.0 / 30.7,
-// 262144 61.4 / 55.9, 524288 118.2 / 106.6, 1048576 230.2 / 207.4; row-major weights 131072 38.7 / 35.6, 262144
-// 67.2 / 61.4, 1048576 240.5 / 212.1: it wins wherever the resident kernel is used at all.
-#ifndef SP_MLP_PIPE_MIN_TILES
-#define SP_MLP_PIPE_MIN_TILES 0
+// The same thresholds for the stacks the pipelined kernel takes (it fills faster than the resident one pays back its
+// weight load).  Measured, us per launch, per-tile kernels / pipelined, packed weights: 32768 rows 10.3 / 12.4, 49152
+// 15.2 / 15.4, 65536 19.9 / 18.2, 81920 25.0 / 24.3, 98304 29.3 / 24.5, 131072 38.5 / 30.7; row-major weights: 65536
+// 21.6 / 23.2, 81920 30.9 / 26.6, 98304 31.8 / 29.4, 131072 41.9 / 36.0.  (Resident / pipelined on the stacks both take:
+// 98304 rows 26.1 / 24.6, 262144 61.4 / 55.9, 1048576 230.2 / 207.4: the pipelined one wherever it applies.)
+#ifndef SP_MLP_PIPE_MIN_TILES_PACKED
+#define SP_MLP_PIPE_MIN_TILES_PACKED 4
+#endif
+#ifndef SP_MLP_PIPE_MIN_TILES_ROWMAJOR
+#define SP_MLP_PIPE_MIN_TILES_ROWMAJOR 5
 #endif
 
 // The Philox stream of a head that draws its own uniforms: the sampling node of the layer graph works on rows of

@@ -620,7 +620,8 @@ extern "C" int sp_mlp_forward_packed(int dtype, const void* x, int32_t n_layers,
     a.x = x; a.packed = packed; a.u = u; a.policy = policy_out; a.action = action_out; a.logits = logits_out;
     a.batch = batch; a.head = head; a.mask_size = mask_size; a.k0 = dims[0]; a.out_stride = dims[n_layers];
     if (mlp_resident_takes(n_layers, dims, a.nout) &&
-        (batch + PK_ROWS - 1) / PK_ROWS >= (long)SP_MLP_RESIDENT_MIN_TILES_PACKED * device_cu_count()) {
+        (batch + PK_ROWS - 1) / PK_ROWS >= (long)(mlp_pipe_takes(n_layers, dims, a.nout) ? SP_MLP_PIPE_MIN_TILES_PACKED
+                                                                                         : SP_MLP_RESIDENT_MIN_TILES_PACKED) * device_cu_count()) {
         // several tiles per compute unit: the kernel that loads the weights once and keeps them in registers
         MlpResidentArgs r{};
         r.x = x; r.packed = packed; r.u = u; r.policy = policy_out; r.action = action_out; r.logits = logits_out;

@@ -498,8 +498,7 @@ bool mlp_resident_takes(int n_layers, const int32_t* dims, int nout) {
 // Launches the resident kernel on `a` (every field but `tiles` filled in by the caller, who has checked the stack with
 // mlp_resident_takes): one workgroup per compute unit, fewer when there are fewer tiles.
 int mlp_resident_launch(int dtype, bool packed, int n_layers, MlpResidentArgs a, hipStream_t stream, const char* what) {
-    if (n_layers == 4 && a.k0 <= 64 && a.nout <= 4 && (a.batch + 63) / 64 >= (long)SP_MLP_PIPE_MIN_TILES * device_cu_count())
-        return mlp_pipe_launch(dtype, packed, a, stream, what);
+    if (n_layers == 4 && a.k0 <= 64 && a.nout <= 4) return mlp_pipe_launch(dtype, packed, a, stream, what);
     const long pairs = (a.batch + RS_PAIR_ROWS - 1) / RS_PAIR_ROWS;
     if (pairs > 0x7fffffffl - 4096) return fail(SP_ERR_SHAPE, "%s: batch too large", what);
     a.tiles = (int)pairs;                                  // the kernel walks pairs of tiles

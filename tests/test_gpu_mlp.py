@@ -312,11 +312,13 @@ def test_head_draws_its_own_uniforms(LY, dims, mask, batch, want_logits, packed,
     ([64, 256, 256, 256, 4], "softmax_regret_matching", 0, 131072 + 31, "f16", "all", False),  # pipelined form: two first-layer k-steps, every bias, row-major
     ([48, 256, 256, 256, 8], "softmax", 3, 99000, "bf16", True, True),                          # pipelined form: 3 of 8 columns valid, zeros behind them
     ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 98304 + 32 * 256 * 9 + 5, "f16", False, True),  # a last head pass of one tile on some units
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 65536 + 7, "f16", False, True),      # the smallest batch the pipelined form takes, packed
+    ([32, 256, 256, 256, 3], "softmax_regret_matching", 0, 81920 + 33, "f16", False, False),    # ... and from row-major weights
 ])
 def test_weights_resident_in_registers(LY, dims, head, mask, batch, dtype, with_bias, packed):
-    """Batches of several 64-row tiles per compute unit run on the kernel that loads the weights once and keeps them in
-    registers while it walks over its tiles (from six tiles per unit with packed weights, from eight with row-major
-    ones): against the oracle like every other kernel, and against the per-tile packed kernel run on the same rows in
+    """Batches of several 64-row tiles per compute unit run on the kernels that load the weights once and keep them in
+    registers while they walk over their tiles (from six tiles per unit with packed weights, from eight with row-major
+    ones; the pipelined form of four-layer stacks from four and five): against the oracle like every other kernel, and against the per-tile packed kernel run on the same rows in
     slices small enough to stay on that kernel (same operand layout; the same order of the sums except in the output
     layer of the pipelined form)."""
     announce("mlp resident %s head=%s mask=%d batch=%d %s bias=%s packed=%s" % (dims, head, mask, batch, dtype, with_bias, packed))
